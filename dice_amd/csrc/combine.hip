@@ -1,0 +1,130 @@
+// Combine: routing-weighted sum of a token's k expert rows, the shared-expert
+// add, and the staleness-cache blend / put, in one pass.
+//
+// Replaces mul_ + scatter_reduce_ of SparseMoeBlock.moe_infer (reference
+// models.py:377-381) = final.mul_(w).view(N,k,h).sum(1) of moe_infer_ep
+// (expertpara/ep_fwd.py:190-195), `y + shared_experts(identity)`
+// (models.py:355-357) and the skip blend / put (ep_fwd.py:176-188).
+//
+// HBM-bound.  Each thread owns one 16-byte column chunk of one token: it reads
+// the k slot rows (or the cached row for the skipped slot), the shared row,
+// and writes y (and the cache row on a "put" step).  Accumulation is fp32 in
+// slot order with a single rounding, no atomics, so the result is
+// deterministic.
+#include "common.h"
+
+namespace dice {
+namespace {
+
+template <typename T> struct Pack;  // 16 bytes of T
+template <> struct Pack<float> {
+  static constexpr int kN = 4;
+  f32x4_t v;
+  __device__ __forceinline__ float get(int i) const { return v[i]; }
+  __device__ __forceinline__ void set(int i, float f) { v[i] = f; }
+};
+template <> struct Pack<bf16_t> {
+  static constexpr int kN = 8;
+  bf16x8_t v;
+  __device__ __forceinline__ float get(int i) const { return (float)v[i]; }
+  __device__ __forceinline__ void set(int i, float f) { v[i] = (bf16_t)f; }
+};
+template <> struct Pack<f16_t> {
+  static constexpr int kN = 8;
+  f16x8_t v;
+  __device__ __forceinline__ float get(int i) const { return (float)v[i]; }
+  __device__ __forceinline__ void set(int i, float f) { v[i] = (f16_t)f; }
+};
+
+constexpr int kMaxTopK = 8;
+
+template <typename T>
+__global__ __launch_bounds__(256) void combine_kernel(
+    const Pack<T> *__restrict__ slot_out, const int32_t *__restrict__ inv_perm,
+    const float *__restrict__ topk_weight, const Pack<T> *__restrict__ shared_out,
+    const uint8_t *__restrict__ skip_mask, const Pack<T> *__restrict__ cache_in,
+    Pack<T> *__restrict__ cache_out, Pack<T> *__restrict__ y, int64_t n_tokens, int top_k,
+    int vec_per_row) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_tokens * vec_per_row) return;
+  const int64_t t = i / vec_per_row;
+  const int c = (int)(i - t * vec_per_row);
+  float acc[Pack<T>::kN];
+#pragma unroll
+  for (int e = 0; e < Pack<T>::kN; ++e) acc[e] = 0.f;
+  for (int j = 0; j < top_k; ++j) {
+    const int64_t s = t * top_k + j;
+    const float w = topk_weight[s];
+    const bool skipped = skip_mask && skip_mask[s];
+    Pack<T> row;
+    if (skipped && cache_in) {
+      row = cache_in[t * vec_per_row + c];
+    } else {
+      const int64_t src = inv_perm ? (int64_t)inv_perm[s] : s;
+      row = slot_out[src * vec_per_row + c];
+      if (skipped && cache_out) cache_out[t * vec_per_row + c] = row;
+    }
+#pragma unroll
+    for (int e = 0; e < Pack<T>::kN; ++e) acc[e] = fmaf(w, row.get(e), acc[e]);
+  }
+  if (shared_out) {
+    Pack<T> sh = shared_out[i];
+#pragma unroll
+    for (int e = 0; e < Pack<T>::kN; ++e) acc[e] += sh.get(e);
+  }
+  Pack<T> o;
+#pragma unroll
+  for (int e = 0; e < Pack<T>::kN; ++e) o.set(e, acc[e]);
+  y[i] = o;
+}
+
+template <typename T>
+int launch_combine(const void *slot_out, const int32_t *inv_perm, const float *w,
+                   const void *shared_out, const uint8_t *skip, const void *cache_in,
+                   void *cache_out, void *y, int64_t n_tokens, int top_k, int hidden,
+                   hipStream_t s) {
+  const int vec_per_row = hidden / Pack<T>::kN;
+  const int64_t total = n_tokens * vec_per_row;
+  const int64_t blocks = (total + 255) / 256;
+  hipLaunchKernelGGL(combine_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s,
+                     (const Pack<T> *)slot_out, inv_perm, w, (const Pack<T> *)shared_out, skip,
+                     (const Pack<T> *)cache_in, (Pack<T> *)cache_out, (Pack<T> *)y, n_tokens, top_k,
+                     vec_per_row);
+  return launch_status("dice_combine");
+}
+
+}  // namespace
+}  // namespace dice
+
+extern "C" int dice_combine(const void *slot_out, const int32_t *inv_perm,
+                            const float *topk_weight, const void *shared_out,
+                            const uint8_t *skip_mask, const void *cache_in, void *cache_out,
+                            void *y, int dtype, int64_t n_tokens, int top_k, int hidden,
+                            void *stream) {
+  using namespace dice;
+  DICE_REQUIRE(slot_out && topk_weight && y, DICE_ERR_BAD_ARG, "dice_combine: null pointer");
+  DICE_REQUIRE(top_k >= 1 && top_k <= kMaxTopK, DICE_ERR_BAD_ARG, "dice_combine: top_k %d outside [1, %d]",
+               top_k, kMaxTopK);
+  DICE_REQUIRE(!(cache_in || cache_out) || skip_mask, DICE_ERR_BAD_ARG,
+               "dice_combine: a cache pointer needs skip_mask");
+  DICE_REQUIRE(!(cache_in && cache_out), DICE_ERR_BAD_ARG,
+               "dice_combine: a step either reads (skip) or writes (put) the cache, not both");
+  const size_t es = dtype_size(dtype);
+  DICE_REQUIRE(es == 2 || es == 4, DICE_ERR_UNSUPPORTED, "dice_combine: dtype %d", dtype);
+  DICE_REQUIRE(hidden > 0 && ((size_t)hidden * es) % 16 == 0, DICE_ERR_BAD_ARG,
+               "dice_combine: hidden %d rows are not a multiple of 16 bytes", hidden);
+  if (n_tokens <= 0) return DICE_OK;
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case DICE_F32:
+      return launch_combine<float>(slot_out, inv_perm, topk_weight, shared_out, skip_mask, cache_in,
+                                   cache_out, y, n_tokens, top_k, hidden, s);
+    case DICE_BF16:
+      return launch_combine<bf16_t>(slot_out, inv_perm, topk_weight, shared_out, skip_mask, cache_in,
+                                    cache_out, y, n_tokens, top_k, hidden, s);
+    case DICE_F16:
+      return launch_combine<f16_t>(slot_out, inv_perm, topk_weight, shared_out, skip_mask, cache_in,
+                                   cache_out, y, n_tokens, top_k, hidden, s);
+  }
+  return fail(DICE_ERR_UNSUPPORTED, "dice_combine: dtype %d", dtype);
+}

@@ -1,0 +1,314 @@
+// Dispatch tables: per-expert histogram, exclusive scan and the stable
+// slot permutation, plus the optional row gather.
+//
+// Replaces argsort + bincount + cumsum of SparseMoeBlock.moe_infer (reference
+// models.py:365-367) and of moe_infer_ep (expertpara/ep_fwd.py:70-76,100-106),
+// including the slot drop of a skip step (ep_fwd.py:57-66).
+//
+// Slots are cut into contiguous spans, one per wavefront.  Inside a span a wave
+// walks 64 slots per round; lanes that hold the same expert find each other
+// with a handful of ballots, so a lane's rank among its peers is a popcount and
+// only one lane per expert touches the LDS counter.  The order inside an expert
+// group is therefore (span, round, lane) = ascending slot index: stable and
+// independent of any atomic's timing.  Integer/byte work, HBM traffic is
+// 4 B read + 8 B written per slot.
+#include "common.h"
+
+namespace dice {
+namespace {
+
+constexpr int kMaxExperts = 256;
+constexpr int kFusedWaves = 16;       // single-workgroup path: 1024 threads
+constexpr int64_t kFusedMaxSlots = 65536;
+constexpr int kTileWaves = 4;         // multi-workgroup path: 256 threads
+constexpr int kTileRounds = 8;        // 512 slots per wave
+
+// Bit mask of the lanes of this wave whose (valid) slot names the same expert.
+__device__ __forceinline__ uint64_t peers_of(int e, bool valid, int nbits) {
+  uint64_t mask = __ballot(valid);
+  for (int b = 0; b < nbits; ++b) {
+    const bool bit = (e >> b) & 1;
+    const uint64_t bal = __ballot(bit);
+    mask &= bit ? bal : ~bal;
+  }
+  return valid ? mask : 0ull;
+}
+
+struct SlotInfo {
+  int64_t slot;
+  int e;
+  bool in_range;  // slot < n_slots
+  bool valid;     // in range, not skipped, expert id legal
+};
+
+__device__ __forceinline__ SlotInfo read_slot(const int32_t *idx, const uint8_t *skip,
+                                              int64_t n_slots, int n_experts, int64_t slot) {
+  SlotInfo s;
+  s.slot = slot;
+  s.in_range = slot < n_slots;
+  s.e = 0;
+  s.valid = false;
+  if (s.in_range) {
+    const int e = idx[slot];
+    const bool dropped = skip && skip[slot];
+    s.valid = !dropped && e >= 0 && e < n_experts;
+    s.e = s.valid ? e : 0;
+  }
+  return s;
+}
+
+// Adds this wave's per-expert counts over its span into row[] (LDS).
+__device__ __forceinline__ void count_span(const int32_t *idx, const uint8_t *skip, int64_t n_slots,
+                                           int n_experts, int nbits, int64_t span_begin, int rounds,
+                                           volatile int32_t *row, int lane) {
+  for (int r = 0; r < rounds; ++r) {
+    SlotInfo s = read_slot(idx, skip, n_slots, n_experts, span_begin + (int64_t)r * kWave + lane);
+    const uint64_t m = peers_of(s.e, s.valid, nbits);
+    if (s.valid && (__ffsll((unsigned long long)m) - 1) == lane) row[s.e] += __popcll(m);
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// Writes perm / inv_perm for this wave's span; row[] holds the next free
+// grouped position per expert and is advanced as the span is walked.
+__device__ __forceinline__ void rank_span(const int32_t *idx, const uint8_t *skip, int64_t n_slots,
+                                          int n_experts, int nbits, int64_t span_begin, int rounds,
+                                          volatile int32_t *row, int lane, int32_t *perm,
+                                          int32_t *inv_perm) {
+  const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  for (int r = 0; r < rounds; ++r) {
+    SlotInfo s = read_slot(idx, skip, n_slots, n_experts, span_begin + (int64_t)r * kWave + lane);
+    const uint64_t m = peers_of(s.e, s.valid, nbits);
+    int pos = -1;
+    if (s.valid) pos = row[s.e] + __popcll(m & below);
+    __builtin_amdgcn_wave_barrier();
+    if (s.valid) {
+      perm[pos] = (int32_t)s.slot;
+      if ((__ffsll((unsigned long long)m) - 1) == lane) row[s.e] += __popcll(m);
+    }
+    if (s.in_range) inv_perm[s.slot] = pos;
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+__global__ __launch_bounds__(kFusedWaves *kWave) void dispatch_fused_kernel(
+    const int32_t *__restrict__ idx, const uint8_t *__restrict__ skip, int64_t n_slots,
+    int n_experts, int nbits, int rounds, int32_t *__restrict__ counts,
+    int32_t *__restrict__ offsets, int32_t *__restrict__ perm, int32_t *__restrict__ inv_perm) {
+  __shared__ volatile int32_t wrow[kFusedWaves][kMaxExperts];
+  __shared__ int32_t eoff[kMaxExperts + 1];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int64_t span = (int64_t)rounds * kWave;
+  const int64_t begin = wave * span;
+
+  for (int e = lane; e < n_experts; e += kWave) wrow[wave][e] = 0;
+  __syncthreads();
+  count_span(idx, skip, n_slots, n_experts, nbits, begin, rounds, wrow[wave], lane);
+  __syncthreads();
+
+  // Exclusive scan of the per-expert totals by the first wave.
+  if (wave == 0) {
+    int carry = 0;
+    for (int c = 0; c < n_experts; c += kWave) {
+      const int e = c + lane;
+      int tot = 0;
+      if (e < n_experts)
+        for (int w = 0; w < kFusedWaves; ++w) tot += wrow[w][e];
+      int inc = tot;
+#pragma unroll
+      for (int o = 1; o < kWave; o <<= 1) {
+        int up = __shfl_up(inc, o, kWave);
+        if (lane >= o) inc += up;
+      }
+      if (e < n_experts) {
+        eoff[e] = carry + inc - tot;
+        counts[e] = tot;
+        offsets[e] = carry + inc - tot;
+      }
+      carry += __shfl(inc, kWave - 1, kWave);
+    }
+    if (lane == 0) {
+      eoff[n_experts] = carry;
+      offsets[n_experts] = carry;
+    }
+  }
+  __syncthreads();
+  // Turn counts into start positions: expert-major, wave-minor.
+  for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
+    int base = eoff[e];
+    for (int w = 0; w < kFusedWaves; ++w) {
+      const int t = wrow[w][e];
+      wrow[w][e] = base;
+      base += t;
+    }
+  }
+  __syncthreads();
+  rank_span(idx, skip, n_slots, n_experts, nbits, begin, rounds, wrow[wave], lane, perm, inv_perm);
+  const int total = eoff[n_experts];
+  for (int64_t i = total + threadIdx.x; i < n_slots; i += blockDim.x) perm[i] = -1;
+}
+
+__global__ __launch_bounds__(kTileWaves *kWave) void dispatch_count_kernel(
+    const int32_t *__restrict__ idx, const uint8_t *__restrict__ skip, int64_t n_slots,
+    int n_experts, int nbits, int units, int32_t *__restrict__ unit_cnt) {
+  __shared__ volatile int32_t wrow[kTileWaves][kMaxExperts];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int unit = blockIdx.x * kTileWaves + wave;
+  for (int e = lane; e < n_experts; e += kWave) wrow[wave][e] = 0;
+  __syncthreads();
+  if (unit < units) {
+    count_span(idx, skip, n_slots, n_experts, nbits, (int64_t)unit * kTileRounds * kWave,
+               kTileRounds, wrow[wave], lane);
+    for (int e = lane; e < n_experts; e += kWave) unit_cnt[(size_t)e * units + unit] = wrow[wave][e];
+  }
+}
+
+// One workgroup: in-place exclusive scan of unit_cnt in expert-major order,
+// plus counts[] and offsets[].
+__global__ __launch_bounds__(1024) void dispatch_scan_kernel(int32_t *__restrict__ unit_cnt,
+                                                             int n_experts, int units,
+                                                             int32_t *__restrict__ counts,
+                                                             int32_t *__restrict__ offsets) {
+  __shared__ int32_t wave_tot[16];
+  __shared__ int32_t eoff[kMaxExperts + 1];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int64_t total = (int64_t)n_experts * units;
+  const int64_t per = (total + 1023) / 1024;
+  const int64_t b = (int64_t)threadIdx.x * per;
+  const int64_t e_ = b + per < total ? b + per : total;
+  int local = 0;
+  for (int64_t i = b; i < e_; ++i) local += unit_cnt[i];
+  int inc = local;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    int up = __shfl_up(inc, o, kWave);
+    if (lane >= o) inc += up;
+  }
+  if (lane == kWave - 1) wave_tot[wave] = inc;
+  __syncthreads();
+  int base = 0;
+  for (int w = 0; w < wave; ++w) base += wave_tot[w];
+  int run = base + inc - local;
+  for (int64_t i = b; i < e_; ++i) {
+    const int c = unit_cnt[i];
+    unit_cnt[i] = run;
+    if (i % units == 0) eoff[i / units] = run;
+    run += c;
+  }
+  if (threadIdx.x == 1023) eoff[n_experts] = run;
+  __syncthreads();
+  for (int e = threadIdx.x; e <= n_experts; e += blockDim.x) {
+    offsets[e] = eoff[e];
+    if (e < n_experts) counts[e] = eoff[e + 1] - eoff[e];
+  }
+}
+
+__global__ __launch_bounds__(kTileWaves *kWave) void dispatch_rank_kernel(
+    const int32_t *__restrict__ idx, const uint8_t *__restrict__ skip, int64_t n_slots,
+    int n_experts, int nbits, int units, const int32_t *__restrict__ unit_base,
+    const int32_t *__restrict__ offsets, int32_t *__restrict__ perm,
+    int32_t *__restrict__ inv_perm) {
+  __shared__ volatile int32_t wrow[kTileWaves][kMaxExperts];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int unit = blockIdx.x * kTileWaves + wave;
+  if (unit >= units) return;
+  for (int e = lane; e < n_experts; e += kWave) wrow[wave][e] = unit_base[(size_t)e * units + unit];
+  __builtin_amdgcn_wave_barrier();
+  const int64_t begin = (int64_t)unit * kTileRounds * kWave;
+  rank_span(idx, skip, n_slots, n_experts, nbits, begin, kTileRounds, wrow[wave], lane, perm, inv_perm);
+  const int total = offsets[n_experts];
+  for (int r = 0; r < kTileRounds; ++r) {
+    const int64_t i = begin + (int64_t)r * kWave + lane;
+    if (i >= total && i < n_slots) perm[i] = -1;
+  }
+}
+
+template <typename V>
+__global__ __launch_bounds__(256) void gather_rows_kernel(const V *__restrict__ x,
+                                                          const int32_t *__restrict__ perm,
+                                                          int slots_per_token, int64_t n_rows,
+                                                          int vec_per_row, V *__restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_rows * vec_per_row) return;
+  const int64_t r = i / vec_per_row;
+  const int c = (int)(i - r * vec_per_row);
+  const int slot = perm[r];
+  if (slot < 0) return;
+  out[i] = x[(int64_t)(slot / slots_per_token) * vec_per_row + c];
+}
+
+int bits_for(int n_experts) {
+  int nbits = 1;
+  while ((1 << nbits) < n_experts) ++nbits;
+  return nbits;
+}
+
+}  // namespace
+}  // namespace dice
+
+extern "C" size_t dice_dispatch_workspace_bytes(int64_t n_slots, int n_experts) {
+  using namespace dice;
+  if (n_slots <= kFusedMaxSlots || n_experts <= 0) return 256;
+  const int64_t units = (n_slots + kTileRounds * kWave - 1) / (kTileRounds * kWave);
+  return align_up((size_t)units * n_experts * sizeof(int32_t), 256);
+}
+
+extern "C" int dice_dispatch(const int32_t *flat_idx, const uint8_t *skip_mask, int64_t n_slots,
+                             int n_experts, int32_t *counts, int32_t *offsets, int32_t *perm,
+                             int32_t *inv_perm, void *workspace, size_t workspace_bytes,
+                             void *stream) {
+  using namespace dice;
+  DICE_REQUIRE(counts && offsets && (n_slots == 0 || (flat_idx && perm && inv_perm)),
+               DICE_ERR_BAD_ARG, "dice_dispatch: null pointer");
+  DICE_REQUIRE(n_experts >= 1 && n_experts <= kMaxExperts, DICE_ERR_UNSUPPORTED,
+               "dice_dispatch: n_experts %d outside [1, %d]", n_experts, kMaxExperts);
+  DICE_REQUIRE(n_slots >= 0 && n_slots < (1ll << 31), DICE_ERR_BAD_ARG,
+               "dice_dispatch: n_slots %lld outside [0, 2^31)", (long long)n_slots);
+  hipStream_t s = (hipStream_t)stream;
+  const int nbits = bits_for(n_experts);
+  if (n_slots <= kFusedMaxSlots) {
+    int rounds = (int)((n_slots + kFusedWaves * kWave - 1) / (kFusedWaves * kWave));
+    hipLaunchKernelGGL(dispatch_fused_kernel, dim3(1), dim3(kFusedWaves * kWave), 0, s, flat_idx,
+                       skip_mask, n_slots, n_experts, nbits, rounds, counts, offsets, perm, inv_perm);
+    return launch_status("dice_dispatch");
+  }
+  const int64_t units64 = (n_slots + kTileRounds * kWave - 1) / (kTileRounds * kWave);
+  const int units = (int)units64;
+  const size_t need = dice_dispatch_workspace_bytes(n_slots, n_experts);
+  DICE_REQUIRE(workspace && workspace_bytes >= need, DICE_ERR_WORKSPACE,
+               "dice_dispatch: workspace %zu < %zu bytes", workspace_bytes, need);
+  int32_t *unit_cnt = (int32_t *)workspace;
+  const int blocks = (units + kTileWaves - 1) / kTileWaves;
+  hipLaunchKernelGGL(dispatch_count_kernel, dim3(blocks), dim3(kTileWaves * kWave), 0, s, flat_idx,
+                     skip_mask, n_slots, n_experts, nbits, units, unit_cnt);
+  hipLaunchKernelGGL(dispatch_scan_kernel, dim3(1), dim3(1024), 0, s, unit_cnt, n_experts, units,
+                     counts, offsets);
+  hipLaunchKernelGGL(dispatch_rank_kernel, dim3(blocks), dim3(kTileWaves * kWave), 0, s, flat_idx,
+                     skip_mask, n_slots, n_experts, nbits, units, unit_cnt, offsets, perm, inv_perm);
+  return launch_status("dice_dispatch");
+}
+
+extern "C" int dice_gather_rows(const void *x, int dtype, const int32_t *perm, int slots_per_token,
+                                int64_t n_rows, int hidden, void *out, void *stream) {
+  using namespace dice;
+  DICE_REQUIRE(x && perm && out, DICE_ERR_BAD_ARG, "dice_gather_rows: null pointer");
+  DICE_REQUIRE(slots_per_token >= 1, DICE_ERR_BAD_ARG, "dice_gather_rows: slots_per_token %d < 1",
+               slots_per_token);
+  const size_t es = dtype_size(dtype);
+  DICE_REQUIRE(es == 2 || es == 4, DICE_ERR_UNSUPPORTED, "dice_gather_rows: dtype %d", dtype);
+  const size_t row_bytes = (size_t)hidden * es;
+  DICE_REQUIRE(hidden > 0 && row_bytes % 16 == 0, DICE_ERR_BAD_ARG,
+               "dice_gather_rows: row of %zu bytes is not a multiple of 16", row_bytes);
+  if (n_rows <= 0) return DICE_OK;
+  const int vec_per_row = (int)(row_bytes / 16);
+  const int64_t total = n_rows * vec_per_row;
+  const int64_t blocks = (total + 255) / 256;
+  hipLaunchKernelGGL(gather_rows_kernel<u32x4_t>, dim3((unsigned)blocks), dim3(256), 0,
+                     (hipStream_t)stream, (const u32x4_t *)x, perm, slots_per_token, n_rows,
+                     vec_per_row, (u32x4_t *)out);
+  return launch_status("dice_gather_rows");
+}

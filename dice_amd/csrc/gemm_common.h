@@ -1,0 +1,112 @@
+// Problem description and tile scheduling shared by the grouped expert GEMMs.
+//
+// One launch covers every expert: grouped rows [offsets[e], offsets[e+1]) of
+// the activation matrix multiply expert e's weight matrix.  The row counts
+// live on the device, so the host sizes the grid from an upper bound and each
+// workgroup derives its own (expert, m-tile, n-tile) from the offset table;
+// surplus workgroups exit at once.  No host synchronisation is needed, unlike
+// the reference's bincount().cpu() (models.py:366).
+#pragma once
+
+#include "common.h"
+
+namespace dice {
+
+enum GemmMode { kFc1Swiglu = 0, kFc1Gelu = 1, kFc2 = 2 };
+
+struct GemmParams {
+  const void *a;           // activations, row stride lda elements
+  const int32_t *a_perm;   // grouped row -> slot; source row = slot / a_div.  NULL: identity
+  int a_div;
+  int lda;
+  const int32_t *offsets;  // [n_experts + 1] grouped row ranges
+  int n_experts;
+  const void *w;           // [n_experts, w_rows, k]
+  int w_rows;              // weight rows per expert (2*n for SwiGLU fc1, else n)
+  int up_offset;           // SwiGLU: first up_proj row inside an expert's block (= n)
+  const float *bias;       // [n_experts, n] or NULL
+  const float *w_scale;    // [n_experts, w_rows] or NULL (fp8 weights)
+  void *c;                 // output, row stride ldc elements
+  int ldc;
+  const int32_t *c_perm;   // grouped row -> output row.  NULL: identity
+  int n;                   // output columns
+  int k;                   // reduction length
+};
+
+struct TileCoord {
+  int expert;
+  int row_begin;   // first grouped row of the tile
+  int rows_valid;  // rows of the tile that belong to the expert (1..BM)
+  int n0;          // first output column
+  bool active;
+};
+
+constexpr int kNumXcd = 8;
+
+// Upper bound on the grid for `max_rows` grouped rows.
+inline int64_t max_tiles(int64_t max_rows, int n_experts, int n, int bm, int bn_out) {
+  const int64_t m_tiles = (max_rows + bm - 1) / bm + n_experts;
+  const int64_t n_tiles = (n + bn_out - 1) / bn_out;
+  const int64_t total = m_tiles * n_tiles;
+  return (total + kNumXcd - 1) / kNumXcd * kNumXcd;
+}
+
+// Maps blockIdx.x to a tile.  Hardware hands consecutive workgroup ids to the
+// eight XCDs round-robin; the remap gives each XCD one contiguous run of the
+// logical tile order (expert-major, then n-tile, m-tile fastest), so the
+// workgroups that share an L2 work on the same expert's weights and re-use
+// the same weight tile across neighbouring m-tiles.
+template <int BM, int BN_OUT>
+__device__ __forceinline__ TileCoord locate_tile(const GemmParams &p) {
+  TileCoord t;
+  t.active = false;
+  const int n_tiles = (p.n + BN_OUT - 1) / BN_OUT;
+  int total_mt = 0;
+  for (int e = 0; e < p.n_experts; ++e) {
+    const int cnt = p.offsets[e + 1] - p.offsets[e];
+    total_mt += (cnt + BM - 1) / BM;
+  }
+  const int total = total_mt * n_tiles;
+  const int per_xcd = (total + kNumXcd - 1) / kNumXcd;
+  const int xcd = blockIdx.x % kNumXcd;
+  const int j = blockIdx.x / kNumXcd;
+  const int logical = xcd * per_xcd + j;
+  if (j >= per_xcd || logical >= total) return t;
+  int base = 0;
+  for (int e = 0; e < p.n_experts; ++e) {
+    const int begin = p.offsets[e];
+    const int cnt = p.offsets[e + 1] - begin;
+    const int mt = (cnt + BM - 1) / BM;
+    const int span = mt * n_tiles;
+    if (logical < base + span) {
+      const int r = logical - base;
+      const int n_tile = r / mt;
+      const int m_tile = r - n_tile * mt;
+      t.expert = e;
+      t.row_begin = begin + m_tile * BM;
+      const int left = cnt - m_tile * BM;
+      t.rows_valid = left < BM ? left : BM;
+      t.n0 = n_tile * BN_OUT;
+      t.active = true;
+      return t;
+    }
+    base += span;
+  }
+  return t;
+}
+
+__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
+
+// tanh-approximate GELU, the closed form of torch gelu(approximate="tanh").
+__device__ __forceinline__ float gelu_tanh_f(float x) {
+  const float k0 = 0.7978845608028654f;  // sqrt(2/pi)
+  const float k1 = 0.044715f;
+  const float inner = k0 * (x + k1 * x * x * x);
+  return 0.5f * x * (1.0f + tanhf(inner));
+}
+
+int launch_grouped_gemm_f32(const GemmParams &p, int mode, int64_t max_rows, hipStream_t s);
+int launch_grouped_gemm_bf16(const GemmParams &p, int mode, int w_dtype, int64_t max_rows,
+                             hipStream_t s);
+
+}  // namespace dice

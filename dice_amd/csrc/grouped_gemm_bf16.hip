@@ -1,0 +1,300 @@
+// bf16 grouped expert GEMM on CDNA4 matrix cores (v_mfma_f32_32x32x16_bf16).
+//
+// Computes, for every expert e and its grouped rows r,
+//   fc1 (SwiGLU): h[r, n] = silu(A[r] . Wg[e, n]) * (A[r] . Wu[e, n])
+//   fc1 (GELU)  : h[r, n] = gelu_tanh(A[r] . W1[e, n] + b1[e, n])
+//   fc2         : out[dst(r), n] = h[r] . W2[e, n] (+ b2[e, n])
+// i.e. MoeMLP.forward of the reference (models.py:252-273) for all experts of
+// moe_infer's loop (models.py:368-377) in one launch.  fp32 accumulation, one
+// rounding to bf16 at the end.
+//
+// Layout.  Activations and weights are both k-contiguous ("NT" GEMM), which is
+// the layout the MFMA operands want: a lane supplies 8 consecutive k values of
+// one row.  A BMxBK activation tile and a BNxBK weight tile are staged in LDS
+// (double buffered); rows are 128 bytes = eight 16-byte chunks and the chunk
+// index is XOR-swizzled with the row so that the 16-byte fragment reads of a
+// wave spread over all banks.  The weight tile is the MFMA "A" operand and the
+// activation tile the "B" operand, which leaves every lane with 4 consecutive
+// output columns of one row: packed 8-byte stores, and gate/up values of the
+// same (row, column) in the same lane for the SwiGLU epilogue.
+//
+// fc1 reads its rows through the dispatch permutation (no gathered copy of x
+// is ever written) and fc2 writes each row straight to its slot position (the
+// un-permute of the reference's _local_combine, expertpara/ep_fwd.py:350-354).
+//
+// fp8 (e4m3) weights are widened to bf16 while they are copied into LDS, so
+// the MFMA loop is unchanged; the per-output-channel scale is applied to the
+// fp32 accumulator in the epilogue.
+#include "gemm_common.h"
+
+namespace dice {
+namespace {
+
+constexpr int kBK = 64;  // bf16 elements per k step = 128 bytes per LDS row
+
+__device__ __forceinline__ int swizzle(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+// Element offset of 16-byte chunk `chunk` of row `row` inside a [rows][64] tile.
+__device__ __forceinline__ int lds_off(int row, int chunk) {
+  return row * kBK + ((chunk ^ swizzle(row)) << 3);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int MODE, bool W_FP8>
+__global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_kernel(GemmParams p) {
+  constexpr int NT = WAVES_M * WAVES_N * kWave;
+  constexpr bool SWIGLU = MODE == kFc1Swiglu;
+  constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
+  constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  static_assert(TM >= 1 && TN >= 1, "wave tile must hold at least one 32x32 block");
+  static_assert(!SWIGLU || TN % 2 == 0, "SwiGLU needs gate and up blocks in the same wave");
+  constexpr int A_ROWS_PER_PASS = NT / 8;
+  constexpr int A_PASSES = BM / A_ROWS_PER_PASS;
+  // bf16 weights: 8 threads x 16 B per row; fp8: 4 threads x 16 B per row.
+  constexpr int B_THREADS_PER_ROW = W_FP8 ? 4 : 8;
+  constexpr int B_ROWS_PER_PASS = NT / B_THREADS_PER_ROW;
+  constexpr int B_PASSES = BN / B_ROWS_PER_PASS;
+  static_assert(A_PASSES >= 1 && B_PASSES >= 1, "tile too small for the workgroup");
+  constexpr int A_STAGE = BM * kBK, B_STAGE = BN * kBK;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  bf16_t *As = reinterpret_cast<bf16_t *>(lds_raw);
+  bf16_t *Bs = As + 2 * A_STAGE;
+
+  const TileCoord t = locate_tile<BM, BN_OUT>(p);
+  if (!t.active) return;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+  // ---- global -> register -> LDS copy assignment ----
+  const int a_chunk = tid & 7, a_row0 = tid >> 3;
+  const bf16_t *a_base = (const bf16_t *)p.a;
+  uint32_t a_src[A_PASSES];
+#pragma unroll
+  for (int i = 0; i < A_PASSES; ++i) {
+    const int rt = a_row0 + i * A_ROWS_PER_PASS;
+    const int gr = t.row_begin + (rt < t.rows_valid ? rt : t.rows_valid - 1);
+    const int src = p.a_perm ? p.a_perm[gr] / p.a_div : gr;
+    a_src[i] = (uint32_t)src * (uint32_t)p.lda + a_chunk * 8;
+  }
+  const int b_chunk = tid % B_THREADS_PER_ROW, b_row0 = tid / B_THREADS_PER_ROW;
+  const size_t w_expert = (size_t)t.expert * p.w_rows * p.k;
+  uint32_t b_src[B_PASSES];
+#pragma unroll
+  for (int i = 0; i < B_PASSES; ++i) {
+    const int rt = b_row0 + i * B_ROWS_PER_PASS;
+    int col = t.n0 + (SWIGLU ? (rt % (BN / 2)) : rt);
+    if (col >= p.n) col = t.n0;
+    const int wrow = (SWIGLU && rt >= BN / 2) ? p.up_offset + col : col;
+    b_src[i] = (uint32_t)wrow * (uint32_t)p.k + b_chunk * (W_FP8 ? 16 : 8);
+  }
+
+  u32x4_t a_reg[A_PASSES], b_reg[B_PASSES];
+  auto load_global = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < A_PASSES; ++i)
+      a_reg[i] = *reinterpret_cast<const u32x4_t *>(a_base + a_src[i] + k0);
+    if (W_FP8) {
+      const uint8_t *wb = (const uint8_t *)p.w + w_expert;
+#pragma unroll
+      for (int i = 0; i < B_PASSES; ++i)
+        b_reg[i] = *reinterpret_cast<const u32x4_t *>(wb + b_src[i] + k0);
+    } else {
+      const bf16_t *wb = (const bf16_t *)p.w + w_expert;
+#pragma unroll
+      for (int i = 0; i < B_PASSES; ++i)
+        b_reg[i] = *reinterpret_cast<const u32x4_t *>(wb + b_src[i] + k0);
+    }
+  };
+  auto store_lds = [&](int stage) {
+    bf16_t *as = As + stage * A_STAGE;
+    bf16_t *bs = Bs + stage * B_STAGE;
+#pragma unroll
+    for (int i = 0; i < A_PASSES; ++i) {
+      const int rt = a_row0 + i * A_ROWS_PER_PASS;
+      *reinterpret_cast<u32x4_t *>(as + lds_off(rt, a_chunk)) = a_reg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < B_PASSES; ++i) {
+      const int rt = b_row0 + i * B_ROWS_PER_PASS;
+      if (W_FP8) {
+        // 16 e4m3 bytes -> 16 bf16 = chunks 2c and 2c+1 of the row.
+        u32x4_t lo, hi;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          bf16x2_t c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(b_reg[i][q], 1.0f, false);
+          bf16x2_t c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(b_reg[i][q], 1.0f, true);
+          lo[2 * q] = __builtin_bit_cast(uint32_t, c0);
+          lo[2 * q + 1] = __builtin_bit_cast(uint32_t, c1);
+          bf16x2_t d0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(b_reg[i][q + 2], 1.0f, false);
+          bf16x2_t d1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(b_reg[i][q + 2], 1.0f, true);
+          hi[2 * q] = __builtin_bit_cast(uint32_t, d0);
+          hi[2 * q + 1] = __builtin_bit_cast(uint32_t, d1);
+        }
+        *reinterpret_cast<u32x4_t *>(bs + lds_off(rt, 2 * b_chunk)) = lo;
+        *reinterpret_cast<u32x4_t *>(bs + lds_off(rt, 2 * b_chunk + 1)) = hi;
+      } else {
+        *reinterpret_cast<u32x4_t *>(bs + lds_off(rt, b_chunk)) = b_reg[i];
+      }
+    }
+  };
+
+  // LDS row of 32-row block j of this wave's weight operand.
+  auto w_block_row = [&](int j) {
+    if (SWIGLU) {
+      constexpr int HALF = TN / 2;
+      return j < HALF ? wn * (WTN / 2) + j * 32 : BN / 2 + wn * (WTN / 2) + (j - HALF) * 32;
+    }
+    return wn * WTN + j * 32;
+  };
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  const int kt_count = p.k / kBK;
+
+  load_global(0);
+  store_lds(0);
+  __syncthreads();
+  for (int kt = 0; kt < kt_count; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < kt_count) load_global((kt + 1) * kBK);
+    const bf16_t *as = As + cur * A_STAGE;
+    const bf16_t *bs = Bs + cur * B_STAGE;
+#pragma unroll
+    for (int kk = 0; kk < kBK / 16; ++kk) {
+      const int chunk = kk * 2 + frag_half;
+      bf16x8_t wf[TN], af[TM];
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        wf[j] = *reinterpret_cast<const bf16x8_t *>(bs + lds_off(w_block_row(j) + frag_row, chunk));
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        af[i] = *reinterpret_cast<const bf16x8_t *>(as + lds_off(wm * WTM + i * 32 + frag_row, chunk));
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[j], af[i], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < kt_count) store_lds(cur ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane holds row (lane&31), columns 8*q + 4*(lane>>5) + {0..3} of each block ----
+  bf16_t *c = (bf16_t *)p.c;
+  const float *bias = p.bias ? p.bias + (size_t)t.expert * p.n : nullptr;
+  const float *scale = p.w_scale ? p.w_scale + (size_t)t.expert * p.w_rows : nullptr;
+  constexpr int OUT_BLOCKS = SWIGLU ? TN / 2 : TN;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = wm * WTM + i * 32 + frag_row;
+    if (m >= t.rows_valid) continue;
+    const int gr = t.row_begin + m;
+    const int64_t orow = p.c_perm ? p.c_perm[gr] : gr;
+    bf16_t *crow = c + orow * p.ldc;
+#pragma unroll
+    for (int j = 0; j < OUT_BLOCKS; ++j) {
+      const int nb = t.n0 + (SWIGLU ? wn * (WTN / 2) : wn * WTN) + j * 32 + frag_half * 4;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = nb + q * 8;
+        if (n >= p.n) continue;
+        bf16x4_t o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float v = acc[i][j][q * 4 + r];
+          if (scale) v *= scale[n + r];
+          if (SWIGLU) {
+            float u = acc[i][j + OUT_BLOCKS][q * 4 + r];
+            if (scale) u *= scale[p.up_offset + n + r];
+            v = silu_f(v) * u;
+          } else {
+            if (bias) v += bias[n + r];
+            if (MODE == kFc1Gelu) v = gelu_tanh_f(v);
+          }
+          o[r] = (bf16_t)v;
+        }
+        *reinterpret_cast<bf16x4_t *>(crow + n) = o;
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int MODE, bool W_FP8>
+int launch_cfg(const GemmParams &p, int64_t max_rows, hipStream_t s) {
+  constexpr int BN_OUT = MODE == kFc1Swiglu ? BN / 2 : BN;
+  constexpr int NT = WAVES_M * WAVES_N * kWave;
+  constexpr size_t lds = 2ull * (BM + BN) * kBK * sizeof(bf16_t);
+  const int64_t grid = max_tiles(max_rows, p.n_experts, p.n, BM, BN_OUT);
+  if (grid <= 0) return DICE_OK;
+  if (grid >= (1ll << 31)) return fail(DICE_ERR_UNSUPPORTED, "bf16 expert GEMM: grid too large");
+  auto kern = grouped_gemm_bf16_kernel<BM, BN, WAVES_M, WAVES_N, MODE, W_FP8>;
+  if (lds > 48 * 1024) {
+    static thread_local bool configured = false;
+    if (!configured) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess)
+        return fail(DICE_ERR_LAUNCH, "bf16 expert GEMM: LDS attribute: %s", hipGetErrorString(e));
+      configured = true;
+    }
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NT), lds, s, p);
+  return launch_status("grouped_gemm_bf16");
+}
+
+int g_cfg_fc1 = 0, g_cfg_fc2 = 0;
+
+template <int MODE, bool W_FP8>
+int launch_mode(const GemmParams &p, int cfg, int64_t max_rows, hipStream_t s) {
+  switch (cfg) {
+    case 1:
+      return launch_cfg<256, 256, 2, 4, MODE, W_FP8>(p, max_rows, s);
+    case 2:
+      return launch_cfg<256, 128, 2, 2, MODE, W_FP8>(p, max_rows, s);
+    default:
+      return launch_cfg<128, 128, 2, 2, MODE, W_FP8>(p, max_rows, s);
+  }
+}
+
+}  // namespace
+
+int launch_grouped_gemm_bf16(const GemmParams &p, int mode, int w_dtype, int64_t max_rows,
+                             hipStream_t s) {
+  if (p.k % kBK != 0) return fail(DICE_ERR_UNSUPPORTED, "bf16 expert GEMM: k %d %% %d != 0", p.k, kBK);
+  if (p.n % 8 != 0) return fail(DICE_ERR_UNSUPPORTED, "bf16 expert GEMM: n %d %% 8 != 0", p.n);
+  const bool fp8 = w_dtype == DICE_FP8_E4M3;
+  const int cfg = mode == kFc2 ? g_cfg_fc2 : g_cfg_fc1;
+  switch (mode) {
+    case kFc1Swiglu:
+      return fp8 ? launch_mode<kFc1Swiglu, true>(p, cfg, max_rows, s)
+                 : launch_mode<kFc1Swiglu, false>(p, cfg, max_rows, s);
+    case kFc1Gelu:
+      return fp8 ? launch_mode<kFc1Gelu, true>(p, cfg, max_rows, s)
+                 : launch_mode<kFc1Gelu, false>(p, cfg, max_rows, s);
+    default:
+      return fp8 ? launch_mode<kFc2, true>(p, cfg, max_rows, s)
+                 : launch_mode<kFc2, false>(p, cfg, max_rows, s);
+  }
+}
+
+}  // namespace dice
+
+// Tuning hook: selects the tile configuration (0: 128x128x64 / 4 waves,
+// 1: 256x256x64 / 8 waves, 2: 256x128x64 / 4 waves) per GEMM.  Not part of the
+// drop-in surface; used by the benchmark to compare tilings.
+extern "C" int dice_set_gemm_config(int fc1_cfg, int fc2_cfg) {
+  dice::g_cfg_fc1 = fc1_cfg;
+  dice::g_cfg_fc2 = fc2_cfg;
+  return DICE_OK;
+}

@@ -1,0 +1,218 @@
+// C entry points of the expert MLP and of the whole layer.
+#include "gemm_common.h"
+
+namespace dice {
+namespace {
+
+int run_gemm(const GemmParams &p, int mode, int act_dtype, int w_dtype, int64_t max_rows,
+             hipStream_t s) {
+  if (act_dtype == DICE_F32) return launch_grouped_gemm_f32(p, mode, max_rows, s);
+  return launch_grouped_gemm_bf16(p, mode, w_dtype, max_rows, s);
+}
+
+struct Carve {
+  unsigned char *base;
+  size_t used;
+  template <typename T> T *take(size_t count) {
+    T *ptr = reinterpret_cast<T *>(base ? base + used : nullptr);
+    used += align_up(count * sizeof(T), 256);
+    return ptr;
+  }
+  void *take_bytes(size_t bytes) { return take<unsigned char>(bytes); }
+};
+
+struct LayerWorkspace {
+  int32_t *topk_idx;
+  float *topk_weight;
+  int32_t *counts, *offsets, *perm, *inv_perm;
+  void *dispatch_ws;
+  size_t dispatch_ws_bytes;
+  void *h, *slot_out, *shared_h, *shared_out;
+  int32_t *shared_offsets;
+  size_t total;
+};
+
+LayerWorkspace carve_layer(const dice_moe_layer_t *L, int64_t n_tokens, void *ws) {
+  LayerWorkspace w;
+  Carve c{(unsigned char *)ws, 0};
+  const size_t es = dtype_size(L->act_dtype);
+  const size_t slots = (size_t)n_tokens * L->top_k;
+  w.topk_idx = c.take<int32_t>(slots);
+  w.topk_weight = c.take<float>(slots);
+  w.counts = c.take<int32_t>(L->n_experts);
+  w.offsets = c.take<int32_t>(L->n_experts + 1);
+  w.perm = c.take<int32_t>(slots);
+  w.inv_perm = c.take<int32_t>(slots);
+  w.dispatch_ws_bytes = dice_dispatch_workspace_bytes((int64_t)slots, L->n_experts);
+  w.dispatch_ws = c.take_bytes(w.dispatch_ws_bytes);
+  w.h = c.take_bytes(slots * L->inter * es);
+  w.slot_out = c.take_bytes(slots * L->hidden * es);
+  w.shared_offsets = c.take<int32_t>(2);
+  if (L->shared_inter > 0) {
+    w.shared_h = c.take_bytes((size_t)n_tokens * L->shared_inter * es);
+    w.shared_out = c.take_bytes((size_t)n_tokens * L->hidden * es);
+  } else {
+    w.shared_h = w.shared_out = nullptr;
+  }
+  w.total = c.used;
+  return w;
+}
+
+__global__ void set_range_kernel(int32_t *offsets, int32_t n) {
+  if (threadIdx.x == 0) {
+    offsets[0] = 0;
+    offsets[1] = n;
+  }
+}
+
+int check_mlp_shape(const char *who, int act_dtype, int w_dtype, int act_variant, int hidden,
+                    int inter, int n_experts) {
+  DICE_REQUIRE(act_dtype == DICE_BF16 || act_dtype == DICE_F32, DICE_ERR_UNSUPPORTED,
+               "%s: act_dtype %d (BF16 or F32)", who, act_dtype);
+  DICE_REQUIRE(w_dtype == act_dtype || (w_dtype == DICE_FP8_E4M3 && act_dtype == DICE_BF16),
+               DICE_ERR_UNSUPPORTED, "%s: w_dtype %d with act_dtype %d", who, w_dtype, act_dtype);
+  DICE_REQUIRE(act_variant == DICE_ACT_SWIGLU || act_variant == DICE_ACT_GELU_TANH,
+               DICE_ERR_BAD_ARG, "%s: act_variant %d", who, act_variant);
+  DICE_REQUIRE(hidden > 0 && hidden % 64 == 0 && inter > 0 && inter % 64 == 0, DICE_ERR_UNSUPPORTED,
+               "%s: hidden %d and inter %d must be positive multiples of 64", who, hidden, inter);
+  DICE_REQUIRE(n_experts >= 1 && n_experts <= 256, DICE_ERR_UNSUPPORTED,
+               "%s: n_experts %d outside [1, 256]", who, n_experts);
+  return DICE_OK;
+}
+
+}  // namespace
+}  // namespace dice
+
+extern "C" int dice_grouped_mlp(const void *x, int act_dtype, const int32_t *perm,
+                                int slots_per_token, const int32_t *offsets, int n_experts,
+                                int64_t max_rows, int hidden, int inter, const void *w1,
+                                const float *b1, const void *w2, const float *b2,
+                                const float *w1_scale, const float *w2_scale, int w_dtype,
+                                int act_variant, void *h, void *out, int scatter_to_slots,
+                                void *stream) {
+  using namespace dice;
+  DICE_REQUIRE(x && offsets && w1 && w2 && h && out, DICE_ERR_BAD_ARG, "dice_grouped_mlp: null pointer");
+  int rc = check_mlp_shape("dice_grouped_mlp", act_dtype, w_dtype, act_variant, hidden, inter, n_experts);
+  if (rc) return rc;
+  DICE_REQUIRE(max_rows >= 0 && max_rows < (1ll << 31), DICE_ERR_BAD_ARG,
+               "dice_grouped_mlp: max_rows %lld", (long long)max_rows);
+  DICE_REQUIRE(!perm || slots_per_token >= 1, DICE_ERR_BAD_ARG,
+               "dice_grouped_mlp: slots_per_token %d < 1", slots_per_token);
+  DICE_REQUIRE(!scatter_to_slots || perm, DICE_ERR_BAD_ARG,
+               "dice_grouped_mlp: scatter_to_slots needs perm");
+  if (w_dtype == DICE_FP8_E4M3)
+    DICE_REQUIRE(w1_scale && w2_scale, DICE_ERR_BAD_ARG, "dice_grouped_mlp: fp8 weights need scales");
+  DICE_REQUIRE(max_rows * (int64_t)(inter > hidden ? inter : hidden) < (1ll << 31),
+               DICE_ERR_UNSUPPORTED, "dice_grouped_mlp: max_rows * row length exceeds 2^31 elements");
+  if (max_rows == 0) return DICE_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const bool swiglu = act_variant == DICE_ACT_SWIGLU;
+
+  GemmParams p1{};
+  p1.a = x;
+  p1.a_perm = perm;
+  p1.a_div = perm ? slots_per_token : 1;
+  p1.lda = hidden;
+  p1.offsets = offsets;
+  p1.n_experts = n_experts;
+  p1.w = w1;
+  p1.w_rows = swiglu ? 2 * inter : inter;
+  p1.up_offset = inter;
+  p1.bias = swiglu ? nullptr : b1;
+  p1.w_scale = w_dtype == DICE_FP8_E4M3 ? w1_scale : nullptr;
+  p1.c = h;
+  p1.ldc = inter;
+  p1.c_perm = nullptr;
+  p1.n = inter;
+  p1.k = hidden;
+  rc = run_gemm(p1, swiglu ? kFc1Swiglu : kFc1Gelu, act_dtype, w_dtype, max_rows, s);
+  if (rc) return rc;
+
+  GemmParams p2{};
+  p2.a = h;
+  p2.a_perm = nullptr;
+  p2.a_div = 1;
+  p2.lda = inter;
+  p2.offsets = offsets;
+  p2.n_experts = n_experts;
+  p2.w = w2;
+  p2.w_rows = hidden;
+  p2.up_offset = 0;
+  p2.bias = swiglu ? nullptr : b2;
+  p2.w_scale = w_dtype == DICE_FP8_E4M3 ? w2_scale : nullptr;
+  p2.c = out;
+  p2.ldc = hidden;
+  p2.c_perm = scatter_to_slots ? perm : nullptr;
+  p2.n = hidden;
+  p2.k = inter;
+  return run_gemm(p2, kFc2, act_dtype, w_dtype, max_rows, s);
+}
+
+extern "C" size_t dice_moe_workspace_bytes(const dice_moe_layer_t *layer, int64_t n_tokens) {
+  if (!layer || n_tokens < 0) return 0;
+  return dice::carve_layer(layer, n_tokens, nullptr).total;
+}
+
+extern "C" int dice_moe_forward(const dice_moe_layer_t *L, const void *x, int64_t n_tokens,
+                                int mode, const uint8_t *skip_mask, const void *cache_in,
+                                void *cache_out, void *y, int32_t *topk_idx_out,
+                                float *topk_weight_out, void *workspace, size_t workspace_bytes,
+                                void *stream) {
+  using namespace dice;
+  DICE_REQUIRE(L && x && y, DICE_ERR_BAD_ARG, "dice_moe_forward: null pointer");
+  DICE_REQUIRE(mode >= 0 && mode <= 2, DICE_ERR_BAD_ARG, "dice_moe_forward: mode %d", mode);
+  DICE_REQUIRE(L->gate_w && L->w1 && L->w2, DICE_ERR_BAD_ARG, "dice_moe_forward: null weights");
+  DICE_REQUIRE(L->top_k >= 1 && L->top_k <= 8 && L->top_k <= L->n_experts, DICE_ERR_BAD_ARG,
+               "dice_moe_forward: top_k %d", L->top_k);
+  int rc = check_mlp_shape("dice_moe_forward", L->act_dtype, L->w_dtype, L->act_variant, L->hidden,
+                           L->inter, L->n_experts);
+  if (rc) return rc;
+  DICE_REQUIRE(L->n_experts <= 64, DICE_ERR_UNSUPPORTED, "dice_moe_forward: n_experts %d > 64",
+               L->n_experts);
+  if (L->shared_inter > 0) {
+    DICE_REQUIRE(L->shared_w1 && L->shared_w2 && L->shared_inter % 64 == 0, DICE_ERR_BAD_ARG,
+                 "dice_moe_forward: shared expert weights / shared_inter %d", L->shared_inter);
+  }
+  if (mode == 1) DICE_REQUIRE(skip_mask && cache_out, DICE_ERR_BAD_ARG,
+                              "dice_moe_forward: a put step needs skip_mask and cache_out");
+  if (mode == 2) {
+    DICE_REQUIRE(skip_mask && cache_in, DICE_ERR_BAD_ARG,
+                 "dice_moe_forward: a skip step needs skip_mask and cache_in");
+    DICE_REQUIRE(L->top_k == 2, DICE_ERR_UNSUPPORTED,
+                 "dice_moe_forward: skipping supports top_k == 2 only (got %d)", L->top_k);
+  }
+  DICE_REQUIRE(n_tokens >= 0 && n_tokens * L->top_k < (1ll << 31), DICE_ERR_BAD_ARG,
+               "dice_moe_forward: n_tokens %lld", (long long)n_tokens);
+  if (n_tokens == 0) return DICE_OK;
+  LayerWorkspace w = carve_layer(L, n_tokens, workspace);
+  DICE_REQUIRE(workspace && workspace_bytes >= w.total, DICE_ERR_WORKSPACE,
+               "dice_moe_forward: workspace %zu < %zu bytes", workspace_bytes, w.total);
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t slots = n_tokens * L->top_k;
+  int32_t *idx = topk_idx_out ? topk_idx_out : w.topk_idx;
+  float *wt = topk_weight_out ? topk_weight_out : w.topk_weight;
+
+  rc = dice_gate_topk(x, L->act_dtype, L->gate_w, L->gate_w_dtype, L->gate_bias, n_tokens, L->hidden,
+                      L->n_experts, L->top_k, L->norm_topk_prob, idx, nullptr, wt, nullptr, stream);
+  if (rc) return rc;
+  rc = dice_dispatch(idx, mode == 2 ? skip_mask : nullptr, slots, L->n_experts, w.counts, w.offsets,
+                     w.perm, w.inv_perm, w.dispatch_ws, w.dispatch_ws_bytes, stream);
+  if (rc) return rc;
+  // A skip step recomputes one slot per token.
+  const int64_t max_rows = mode == 2 ? n_tokens * (L->top_k - 1) : slots;
+  rc = dice_grouped_mlp(x, L->act_dtype, w.perm, L->top_k, w.offsets, L->n_experts, max_rows,
+                        L->hidden, L->inter, L->w1, L->b1, L->w2, L->b2, L->w1_scale, L->w2_scale,
+                        L->w_dtype, L->act_variant, w.h, w.slot_out, 1, stream);
+  if (rc) return rc;
+  if (L->shared_inter > 0) {
+    hipLaunchKernelGGL(set_range_kernel, dim3(1), dim3(64), 0, s, w.shared_offsets, (int32_t)n_tokens);
+    rc = dice_grouped_mlp(x, L->act_dtype, nullptr, 1, w.shared_offsets, 1, n_tokens, L->hidden,
+                          L->shared_inter, L->shared_w1, L->shared_b1, L->shared_w2, L->shared_b2,
+                          nullptr, nullptr, L->act_dtype, L->act_variant, w.shared_h, w.shared_out, 0,
+                          stream);
+    if (rc) return rc;
+  }
+  return dice_combine(w.slot_out, nullptr, wt, w.shared_out, mode == 0 ? nullptr : skip_mask,
+                      mode == 2 ? cache_in : nullptr, mode == 1 ? cache_out : nullptr, y,
+                      L->act_dtype, n_tokens, L->top_k, L->hidden, stream);
+}

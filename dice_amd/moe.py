@@ -1,0 +1,309 @@
+"""Drop-in modules for the reference's MoE layer, running on the HIP library.
+
+``MoEGate``, ``MoeMLP`` and ``SparseMoeBlock`` keep the constructor arguments,
+sub-module names, parameter names/shapes (state-dict keys) and ``forward``
+signatures of the reference classes (models.py:159-217, 240-273, 276-382), so a
+checkpoint of the reference loads unchanged and ``DiTBlock`` can call the block
+as before.  Only the inference branch exists; there is no training path and no
+CPU path - every forward runs the gfx950 kernels.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from typing import Optional
+
+import torch
+import torch.nn as nn
+
+from . import diep, ops
+from .lib import (DICE_ACT_GELU_TANH, DICE_ACT_SWIGLU, MODE_PLAIN, MODE_PUT, MODE_SKIP, DiceError,
+                  MoeLayerDesc, check, dtype_code, load, ptr, stream_ptr)
+
+
+class ParaMode:
+    """Value object of the reference (models.py:34-55), reduced to what the MoE
+    block reads: ``ep`` selects the ``moe_infer_ep`` data flow (and with it the
+    staleness cache); anything that needs a second GPU is refused."""
+
+    def __init__(self, ep=False, ep_async=False, sp=False, sp_async=False, **kwargs):
+        if ep_async or sp or sp_async:
+            raise DiceError("async expert parallelism and sequence parallelism need several GPUs "
+                            "and are outside this single-GPU build")
+        self.ep = ep
+        self.ep_async = False
+        self.sp = False
+        self.sp_async = False
+        self.dp = not ep
+        for k, v in kwargs.items():
+            setattr(self, k, v)
+
+    def verbose(self):
+        return "DP" if self.dp else "EP"
+
+
+class MoEGate(nn.Module):
+    """Router (reference models.py:159-217, inference branch)."""
+
+    def __init__(self, embed_dim, num_experts=16, num_experts_per_tok=2, aux_loss_alpha=0.01):
+        super().__init__()
+        self.top_k = num_experts_per_tok
+        self.n_routed_experts = num_experts
+        self.scoring_func = "softmax"
+        self.alpha = aux_loss_alpha
+        self.seq_aux = False
+        self.norm_topk_prob = False
+        self.gating_dim = embed_dim
+        self.weight = nn.Parameter(torch.empty((self.n_routed_experts, self.gating_dim)))
+        self.bias = None  # extension: optional fp32 [E] router bias (not in the reference)
+        self.reset_parameters()
+
+    def reset_parameters(self) -> None:
+        nn.init.kaiming_uniform_(self.weight, a=math.sqrt(5))
+
+    @torch.no_grad()
+    def forward(self, hidden_states):
+        if self.training:
+            raise DiceError("MoEGate: only the inference branch is implemented (call .eval())")
+        idx, wt, _, idx64 = ops.gate_topk(hidden_states.contiguous(), self.weight, self.top_k,
+                                          self.norm_topk_prob, self.bias, want_int64=True)
+        return idx64, wt.to(hidden_states.dtype), None
+
+
+class MoeMLP(nn.Module):
+    """SwiGLU expert (reference models.py:240-273).  ``pretraining_tp`` is
+    accepted for interface parity; the slice/cat/sum path it selects in the
+    reference is algebraically the same product, which is what runs here."""
+
+    def __init__(self, hidden_size, intermediate_size, pretraining_tp=2):
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.gate_proj = nn.Linear(hidden_size, intermediate_size, bias=False)
+        self.up_proj = nn.Linear(hidden_size, intermediate_size, bias=False)
+        self.down_proj = nn.Linear(intermediate_size, hidden_size, bias=False)
+        self.pretraining_tp = pretraining_tp
+
+    @torch.no_grad()
+    def forward(self, x):
+        shape = x.shape
+        x2 = x.reshape(-1, shape[-1]).contiguous()
+        n = x2.shape[0]
+        w1 = torch.cat([self.gate_proj.weight, self.up_proj.weight], 0).unsqueeze(0).contiguous()
+        w2 = self.down_proj.weight.unsqueeze(0).contiguous()
+        offsets = torch.tensor([0, n], dtype=torch.int32, device=x.device)
+        out = ops.grouped_mlp(x2, None, 1, offsets, n, w1, w2, "swiglu")
+        return out.view(shape)
+
+
+class GeluMLP(nn.Module):
+    """Two-matrix tanh-GELU expert, ``fc2(gelu_tanh(fc1(x)))`` with biases: the
+    MLP the benchmark configurations name (the reference keeps it only as a
+    commented-out dense ``Mlp``, models.py:496-497)."""
+
+    def __init__(self, hidden_size, intermediate_size):
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.fc1 = nn.Linear(hidden_size, intermediate_size, bias=True)
+        self.fc2 = nn.Linear(intermediate_size, hidden_size, bias=True)
+
+
+class _Packed:
+    """Expert weights in the layout the grouped GEMM reads."""
+
+    def __init__(self):
+        self.w1 = self.w2 = self.b1 = self.b2 = None
+        self.w1_scale = self.w2_scale = None
+        self.sw1 = self.sw2 = self.sb1 = self.sb2 = None
+
+
+class SparseMoeBlock(nn.Module):
+    """Mixture-of-experts block with a shared expert (reference models.py:276-382).
+
+    Extra keyword ``variant`` ("swiglu" = reference, "gelu_tanh" = two-matrix
+    experts) and ``n_shared_experts`` are extensions with reference defaults.
+    """
+
+    def __init__(self, embed_dim, mlp_ratio=4, num_experts=16, num_experts_per_tok=2,
+                 pretraining_tp=2, layer_idx=None, total_layers=None, para_mode: ParaMode = None,
+                 variant: str = "swiglu", n_shared_experts: Optional[int] = 2):
+        super().__init__()
+        assert para_mode is not None
+        self.num_experts_per_tok = num_experts_per_tok
+        self.variant = variant
+        inter = int(mlp_ratio * embed_dim)
+        if variant == "swiglu":
+            mk = lambda i: MoeMLP(embed_dim, i, pretraining_tp)
+        elif variant == "gelu_tanh":
+            mk = lambda i: GeluMLP(embed_dim, i)
+        else:
+            raise DiceError(f"unknown expert variant {variant}")
+        self.experts = nn.ModuleList([mk(inter) for _ in range(num_experts)])
+        self.gate = MoEGate(embed_dim, num_experts, num_experts_per_tok)
+        self.n_shared_experts = n_shared_experts
+        if self.n_shared_experts is not None:
+            self.shared_experts = mk(embed_dim * self.n_shared_experts)
+        self.layer_idx = layer_idx
+        self.total_layers = total_layers
+        self.para_mode = para_mode
+        self.embed_dim = embed_dim
+        self.inter = inter
+        self._packed: Optional[_Packed] = None
+        self._fp8 = False
+        self._desc = None
+        self._ws = None
+
+    # ------------------------------------------------------------------ #
+    # weight packing
+    # ------------------------------------------------------------------ #
+    def _apply(self, fn, *args, **kwargs):
+        self._packed = None
+        self._desc = None
+        self._ws = None
+        return super()._apply(fn, *args, **kwargs)
+
+    def load_state_dict(self, *args, **kwargs):
+        self._packed = None
+        self._desc = None
+        return super().load_state_dict(*args, **kwargs)
+
+    @torch.no_grad()
+    def pack_weights(self, fp8: bool = False) -> _Packed:
+        """Builds ``w1 [E, 2I, D]`` = rows ``[gate_proj; up_proj]`` and
+        ``w2 [E, D, I]`` from the per-expert parameters, then re-points every
+        parameter at its slice of the packed storage so the weights exist once.
+        ``fp8=True`` additionally quantises the routed experts to e4m3 with
+        per-output-channel scales (shared expert stays in the module dtype)."""
+        p = _Packed()
+        ex = list(self.experts)
+        if self.variant == "swiglu":
+            p.w1 = torch.stack([torch.cat([e.gate_proj.weight, e.up_proj.weight], 0) for e in ex]).contiguous()
+            p.w2 = torch.stack([e.down_proj.weight for e in ex]).contiguous()
+            inter = self.inter
+            for i, e in enumerate(ex):
+                e.gate_proj.weight.data = p.w1[i, :inter]
+                e.up_proj.weight.data = p.w1[i, inter:]
+                e.down_proj.weight.data = p.w2[i]
+            if self.n_shared_experts is not None:
+                s = self.shared_experts
+                p.sw1 = torch.cat([s.gate_proj.weight, s.up_proj.weight], 0).unsqueeze(0).contiguous()
+                p.sw2 = s.down_proj.weight.data.unsqueeze(0).contiguous()
+                si = s.intermediate_size
+                s.gate_proj.weight.data = p.sw1[0, :si]
+                s.up_proj.weight.data = p.sw1[0, si:]
+                s.down_proj.weight.data = p.sw2[0]
+        else:
+            p.w1 = torch.stack([e.fc1.weight for e in ex]).contiguous()
+            p.w2 = torch.stack([e.fc2.weight for e in ex]).contiguous()
+            p.b1 = torch.stack([e.fc1.bias for e in ex]).float().contiguous()
+            p.b2 = torch.stack([e.fc2.bias for e in ex]).float().contiguous()
+            for i, e in enumerate(ex):
+                e.fc1.weight.data = p.w1[i]
+                e.fc2.weight.data = p.w2[i]
+            if self.n_shared_experts is not None:
+                s = self.shared_experts
+                p.sw1 = s.fc1.weight.data.unsqueeze(0).contiguous()
+                p.sw2 = s.fc2.weight.data.unsqueeze(0).contiguous()
+                p.sb1 = s.fc1.bias.data.float().unsqueeze(0).contiguous()
+                p.sb2 = s.fc2.bias.data.float().unsqueeze(0).contiguous()
+                s.fc1.weight.data = p.sw1[0]
+                s.fc2.weight.data = p.sw2[0]
+        if fp8:
+            p.w1, p.w1_scale = ops.quantize_fp8_rowwise(p.w1)
+            p.w2, p.w2_scale = ops.quantize_fp8_rowwise(p.w2)
+        self._packed = p
+        self._fp8 = fp8
+        self._desc = None
+        return p
+
+    def quantize_fp8(self):
+        """Switches the routed experts to e4m3 weights (build-defined path)."""
+        self.pack_weights(fp8=True)
+        return self
+
+    def _ensure(self, x: torch.Tensor):
+        if self._packed is None:
+            self.pack_weights(self._fp8)
+        if self._desc is None:
+            p = self._packed
+            d = MoeLayerDesc()
+            d.hidden, d.inter = self.embed_dim, self.inter
+            d.n_experts, d.top_k = len(self.experts), self.num_experts_per_tok
+            d.act_dtype = dtype_code(x.dtype)
+            d.w_dtype = dtype_code(p.w1.dtype)
+            d.act_variant = DICE_ACT_SWIGLU if self.variant == "swiglu" else DICE_ACT_GELU_TANH
+            d.norm_topk_prob = int(self.gate.norm_topk_prob)
+            d.gate_w_dtype = dtype_code(self.gate.weight.dtype)
+            d.shared_inter = 0 if p.sw1 is None else p.sw2.shape[-1]
+            d.gate_w = ptr(self.gate.weight)
+            d.gate_bias = ptr(self.gate.bias)
+            d.w1, d.w2 = ptr(p.w1), ptr(p.w2)
+            d.b1, d.b2 = ptr(p.b1), ptr(p.b2)
+            d.w1_scale, d.w2_scale = ptr(p.w1_scale), ptr(p.w2_scale)
+            d.shared_w1, d.shared_w2 = ptr(p.sw1), ptr(p.sw2)
+            d.shared_b1, d.shared_b2 = ptr(p.sb1), ptr(p.sb2)
+            self._desc = d
+        return self._desc
+
+    def _workspace(self, desc, n_tokens: int, device):
+        need = load().dice_moe_workspace_bytes(ctypes.byref(desc), n_tokens)
+        if self._ws is None or self._ws.numel() < need or self._ws.device != device:
+            self._ws = torch.empty(need, dtype=torch.uint8, device=device)
+        return self._ws
+
+    # ------------------------------------------------------------------ #
+    # forward
+    # ------------------------------------------------------------------ #
+    @torch.no_grad()
+    def forward(self, hidden_states):
+        """``[B, T, D] -> [B, T, D]`` (reference models.py:302-358)."""
+        if self.training:
+            raise DiceError("SparseMoeBlock: only the inference branch is implemented (call .eval())")
+        orig_shape = hidden_states.shape
+        x = hidden_states.reshape(-1, orig_shape[-1]).contiguous()
+        mode, mask, cache_in, cache_out = MODE_PLAIN, None, None, None
+        if self.para_mode.ep and diep.ep_skip_enabled():
+            # conditional communication: reference models.py:342-353, ep_fwd.py:49-66,176-188
+            mask = diep.ep_skip_mask(x.shape[0] * self.num_experts_per_tok).to(x.device)
+            if diep.ep_skip_now(self.layer_idx):
+                mode, cache_in = MODE_SKIP, diep.ep_skip_get(self.layer_idx)
+            else:
+                mode = MODE_PUT
+                cache_out = torch.empty_like(x)
+        y = self.run(x, mode, mask, cache_in, cache_out)
+        if mode == MODE_PUT:
+            diep.ep_skip_put(self.layer_idx, cache_out)
+        return y.view(*orig_shape)
+
+    @torch.no_grad()
+    def run(self, x, mode=MODE_PLAIN, skip_mask=None, cache_in=None, cache_out=None,
+            topk_idx_out=None, topk_weight_out=None, y=None):
+        """One call of ``dice_moe_forward`` on ``x [N, D]``."""
+        desc = self._ensure(x)
+        n = x.shape[0]
+        ws = self._workspace(desc, n, x.device)
+        if y is None:
+            y = torch.empty_like(x)
+        if skip_mask is not None and skip_mask.dtype == torch.bool:
+            skip_mask = skip_mask.view(torch.uint8)
+        check(load().dice_moe_forward(ctypes.byref(desc), ptr(x), n, mode, ptr(skip_mask), ptr(cache_in),
+                                      ptr(cache_out), ptr(y), ptr(topk_idx_out), ptr(topk_weight_out),
+                                      ptr(ws), ws.numel(), stream_ptr()))
+        return y
+
+    @torch.no_grad()
+    def moe_infer(self, x, flat_expert_indices, flat_expert_weights):
+        """Routed experts only, from given routing (reference models.py:361-382)."""
+        if self._packed is None:
+            self.pack_weights(self._fp8)
+        p = self._packed
+        k = self.num_experts_per_tok
+        n = x.shape[0]
+        idx = flat_expert_indices.to(torch.int32).contiguous()
+        _, offsets, perm, _ = ops.dispatch(idx, len(self.experts))
+        slot_out = ops.grouped_mlp(x.contiguous(), perm, k, offsets, n * k, p.w1, p.w2, self.variant,
+                                   p.b1, p.b2, p.w1_scale, p.w2_scale, scatter_to_slots=True,
+                                   n_out_rows=n * k)
+        w = flat_expert_weights.reshape(n, k).float().contiguous()
+        return ops.combine(slot_out, w, n, k)

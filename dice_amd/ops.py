@@ -1,0 +1,124 @@
+"""Tensor-level wrappers over the C ABI, one per stage of the layer.
+
+Every function enqueues HIP kernels on torch's current stream and returns
+device tensors; none of them synchronises with the host.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import lib as _l
+from .lib import DICE_ACT_GELU_TANH, DICE_ACT_SWIGLU, check, dtype_code, load, ptr, stream_ptr
+
+VARIANTS = {"swiglu": DICE_ACT_SWIGLU, "gelu_tanh": DICE_ACT_GELU_TANH}
+
+
+def gate_topk(x: torch.Tensor, weight: torch.Tensor, top_k: int, norm_topk_prob: bool = False,
+              bias: Optional[torch.Tensor] = None, want_logits: bool = False,
+              want_int64: bool = False):
+    """Router (reference ``MoEGate.forward`` models.py:179-196).
+
+    Returns ``(topk_idx int32 [N,k], topk_weight fp32 [N,k], logits fp32 [N,E] | None,
+    topk_idx int64 | None)``; slot 0 is the arg-max."""
+    x2 = x.reshape(-1, x.shape[-1])
+    n, d = x2.shape
+    e = weight.shape[0]
+    dev = x2.device
+    idx = torch.empty((n, top_k), dtype=torch.int32, device=dev)
+    idx64 = torch.empty((n, top_k), dtype=torch.int64, device=dev) if want_int64 else None
+    wt = torch.empty((n, top_k), dtype=torch.float32, device=dev)
+    logits = torch.empty((n, e), dtype=torch.float32, device=dev) if want_logits else None
+    if bias is not None and bias.dtype != torch.float32:
+        raise _l.DiceError("router bias must be fp32")
+    check(load().dice_gate_topk(ptr(x2), dtype_code(x2.dtype), ptr(weight), dtype_code(weight.dtype),
+                                ptr(bias), n, d, e, top_k, int(bool(norm_topk_prob)), ptr(idx),
+                                ptr(idx64), ptr(wt), ptr(logits), stream_ptr()))
+    return idx, wt, logits, idx64
+
+
+def dispatch(flat_idx: torch.Tensor, n_experts: int, skip_mask: Optional[torch.Tensor] = None):
+    """Dispatch tables (reference models.py:365-367, ep_fwd.py:57-76,100-106).
+
+    ``flat_idx`` int32 [S]; ``skip_mask`` uint8/bool [S] marks dropped slots.
+    Returns ``(counts [E], offsets [E+1], perm [S], inv_perm [S])`` int32."""
+    if flat_idx.dtype != torch.int32:
+        raise _l.DiceError("dispatch needs int32 expert indices")
+    s = flat_idx.numel()
+    dev = flat_idx.device
+    counts = torch.empty(n_experts, dtype=torch.int32, device=dev)
+    offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=dev)
+    perm = torch.empty(s, dtype=torch.int32, device=dev)
+    inv_perm = torch.empty(s, dtype=torch.int32, device=dev)
+    ws_bytes = load().dice_dispatch_workspace_bytes(s, n_experts)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    if skip_mask is not None:
+        skip_mask = skip_mask.view(torch.uint8) if skip_mask.dtype == torch.bool else skip_mask
+    check(load().dice_dispatch(ptr(flat_idx), ptr(skip_mask), s, n_experts, ptr(counts), ptr(offsets),
+                               ptr(perm), ptr(inv_perm), ptr(ws), ws_bytes, stream_ptr()))
+    return counts, offsets, perm, inv_perm
+
+
+def gather_rows(x: torch.Tensor, perm: torch.Tensor, slots_per_token: int, n_rows: int):
+    """``out[r] = x[perm[r] // slots_per_token]`` (reference ``_local_dispatch``
+    ep_fwd.py:345-347)."""
+    out = torch.zeros((n_rows, x.shape[-1]), dtype=x.dtype, device=x.device)
+    check(load().dice_gather_rows(ptr(x), dtype_code(x.dtype), ptr(perm), slots_per_token, n_rows,
+                                  x.shape[-1], ptr(out), stream_ptr()))
+    return out
+
+
+def grouped_mlp(x: torch.Tensor, perm: Optional[torch.Tensor], slots_per_token: int,
+                offsets: torch.Tensor, max_rows: int, w1: torch.Tensor, w2: torch.Tensor,
+                variant: str = "swiglu", b1=None, b2=None, w1_scale=None, w2_scale=None,
+                scatter_to_slots: bool = False, n_out_rows: Optional[int] = None,
+                h: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None):
+    """Grouped expert MLP (reference models.py:368-377 with MoeMLP :252-273).
+
+    ``w1`` is ``[E, 2I, D]`` (SwiGLU, rows ``[gate_proj; up_proj]``) or
+    ``[E, I, D]`` (GELU); ``w2`` is ``[E, D, I]``.  Returns ``out``: row
+    ``perm[r]`` of ``[n_out_rows, D]`` when ``scatter_to_slots`` else row ``r``
+    of ``[max_rows, D]``.  Outputs are not scaled by the routing weights."""
+    e, d, inter = w2.shape
+    if n_out_rows is None:
+        n_out_rows = max_rows
+    if h is None:
+        h = torch.empty((max(max_rows, 1), inter), dtype=x.dtype, device=x.device)
+    if out is None:
+        out = torch.zeros((n_out_rows, d), dtype=x.dtype, device=x.device)
+    check(load().dice_grouped_mlp(
+        ptr(x), dtype_code(x.dtype), ptr(perm), slots_per_token, ptr(offsets), e, max_rows, d, inter,
+        ptr(w1), ptr(b1), ptr(w2), ptr(b2), ptr(w1_scale), ptr(w2_scale), dtype_code(w1.dtype),
+        VARIANTS[variant], ptr(h), ptr(out), int(bool(scatter_to_slots)), stream_ptr()))
+    return out
+
+
+def combine(slot_out: torch.Tensor, topk_weight: torch.Tensor, n_tokens: int, top_k: int,
+            inv_perm: Optional[torch.Tensor] = None, shared_out: Optional[torch.Tensor] = None,
+            skip_mask: Optional[torch.Tensor] = None, cache_in: Optional[torch.Tensor] = None,
+            cache_out: Optional[torch.Tensor] = None):
+    """Weighted sum over a token's slots + shared add + cache blend / put
+    (reference models.py:377-381,355-357; ep_fwd.py:176-195)."""
+    d = slot_out.shape[-1]
+    y = torch.empty((n_tokens, d), dtype=slot_out.dtype, device=slot_out.device)
+    if skip_mask is not None and skip_mask.dtype == torch.bool:
+        skip_mask = skip_mask.view(torch.uint8)
+    if topk_weight.dtype != torch.float32:
+        raise _l.DiceError("combine needs fp32 routing weights")
+    check(load().dice_combine(ptr(slot_out), ptr(inv_perm), ptr(topk_weight), ptr(shared_out),
+                              ptr(skip_mask), ptr(cache_in), ptr(cache_out), ptr(y),
+                              dtype_code(slot_out.dtype), n_tokens, top_k, d, stream_ptr()))
+    return y
+
+
+def quantize_fp8_rowwise(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-output-channel e4m3fn quantisation of a ``[..., rows, cols]`` weight.
+    Returns ``(q float8_e4m3fn same shape, scale fp32 [..., rows])``."""
+    cols = w.shape[-1]
+    rows = w.numel() // cols
+    q = torch.empty(w.shape, dtype=torch.uint8, device=w.device)
+    scale = torch.empty(w.shape[:-1], dtype=torch.float32, device=w.device)
+    check(load().dice_quantize_fp8_rowwise(ptr(w), dtype_code(w.dtype), rows, cols, ptr(q), ptr(scale),
+                                           stream_ptr()))
+    return q.view(torch.float8_e4m3fn), scale

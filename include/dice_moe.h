@@ -1,0 +1,202 @@
+/*
+ * dice_moe.h - C ABI of the MI355X (gfx950) DiT-MoE sparse expert layer.
+ *
+ * The reference (Cobalt-27/DICE) is pure Python on torch and has no FFI of its
+ * own; every entry point below names the reference function whose work it
+ * replaces.  Paths are relative to the reference tree.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its name ends in _host;
+ *   - the caller owns every buffer; the library never allocates, frees or
+ *     synchronises; all work is enqueued on `stream` (a hipStream_t passed as
+ *     void*; NULL = the default stream);
+ *   - return value 0 = ok, negative = error (see DICE_ERR_*); the text of the
+ *     last error on the calling thread is available from dice_last_error();
+ *   - matrices are row-major and contiguous; "slot" s = k*token + j is entry j
+ *     of token's top-k list (token-major, as models.py:311-312 flattens it).
+ */
+#ifndef DICE_MOE_H
+#define DICE_MOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DICE_MOE_ABI_VERSION 1
+
+/* element types */
+#define DICE_F32 0
+#define DICE_BF16 1
+#define DICE_F16 2
+#define DICE_FP8_E4M3 3 /* OCP e4m3fn, weights only */
+
+/* expert MLP variants */
+#define DICE_ACT_SWIGLU 0    /* down(silu(gate(x)) * up(x)), models.py:271 */
+#define DICE_ACT_GELU_TANH 1 /* fc2(gelu_tanh(fc1(x)+b1))+b2, models.py:496 */
+
+/* errors */
+#define DICE_OK 0
+#define DICE_ERR_BAD_ARG (-1)
+#define DICE_ERR_UNSUPPORTED (-2)
+#define DICE_ERR_WORKSPACE (-3)
+#define DICE_ERR_LAUNCH (-4)
+
+int dice_abi_version(void);
+const char *dice_last_error(void);
+
+/*
+ * Router.  Replaces MoEGate.forward, inference branch (models.py:179-196):
+ * logits = x W^T (+ bias, an extension; NULL = reference), fp32 softmax over
+ * experts, top-k in descending score order (slot 0 = arg-max; ties -> lower
+ * expert id), optional renormalisation by (sum + 1e-20) (models.py:194-196).
+ *   x        [n_tokens, hidden]   x_dtype in {F32, BF16, F16}
+ *   w        [n_experts, hidden]  w_dtype in {F32, BF16, F16}
+ *   bias     [n_experts] fp32 or NULL
+ *   topk_idx   [n_tokens, top_k] int32   (required)
+ *   topk_idx64 [n_tokens, top_k] int64   (optional, the reference's dtype)
+ *   topk_weight[n_tokens, top_k] fp32
+ *   logits     [n_tokens, n_experts] fp32 (optional, for tie audits)
+ * Limits: n_experts <= 64, top_k <= 8, hidden % 8 == 0.
+ */
+int dice_gate_topk(const void *x, int x_dtype, const void *w, int w_dtype,
+                   const float *bias, int64_t n_tokens, int hidden,
+                   int n_experts, int top_k, int norm_topk_prob,
+                   int32_t *topk_idx, int64_t *topk_idx64, float *topk_weight,
+                   float *logits, void *stream);
+
+/*
+ * Dispatch tables.  Replaces argsort + bincount + cumsum of
+ * SparseMoeBlock.moe_infer (models.py:365-367) and of moe_infer_ep
+ * (expertpara/ep_fwd.py:70-76,100-106), including the slot drop of a skip
+ * step (ep_fwd.py:57-66): slots whose skip_mask byte is non-zero are left out.
+ *   flat_idx  [n_slots] int32 expert id per slot
+ *   skip_mask [n_slots] uint8 or NULL
+ *   counts    [n_experts] int32      rows per expert
+ *   offsets   [n_experts+1] int32    exclusive scan of counts
+ *   perm      [n_slots] int32        grouped row -> slot (stable: ascending
+ *                                    slot inside each expert); entries past
+ *                                    offsets[n_experts] are set to -1
+ *   inv_perm  [n_slots] int32        slot -> grouped row, -1 for dropped slots
+ *   workspace: dice_dispatch_workspace_bytes(n_slots, n_experts) bytes
+ */
+size_t dice_dispatch_workspace_bytes(int64_t n_slots, int n_experts);
+int dice_dispatch(const int32_t *flat_idx, const uint8_t *skip_mask,
+                  int64_t n_slots, int n_experts, int32_t *counts,
+                  int32_t *offsets, int32_t *perm, int32_t *inv_perm,
+                  void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Row gather.  Replaces _local_dispatch (expertpara/ep_fwd.py:345-347) and
+ * x[exp_token_idx] (models.py:373): out[r] = x[perm[r] / slots_per_token] for
+ * r < n_rows with perm[r] >= 0.  The fused expert path below reads x through
+ * perm directly and does not need this copy; it exists for callers that want
+ * the grouped activations themselves.
+ */
+int dice_gather_rows(const void *x, int dtype, const int32_t *perm,
+                     int slots_per_token, int64_t n_rows, int hidden,
+                     void *out, void *stream);
+
+/*
+ * Grouped expert MLP.  Replaces the per-expert loop of moe_infer
+ * (models.py:368-377) / proc_experts (expertpara/ep_fwd.py:200-211) with
+ * MoeMLP.forward (models.py:252-273) as the expert, in two grouped GEMMs:
+ *   fc1: h[r] = act(A[r] W1[e]^T)     fc2: out[dst(r)] = h[r] W2[e]^T
+ * for grouped rows r in [offsets[e], offsets[e+1]).
+ *   x        [n_tokens, hidden] activations (act_dtype in {BF16, F32})
+ *   perm     [>= max_rows] int32 grouped row -> slot, or NULL (row r = token r)
+ *   slots_per_token  divisor turning a slot into its token row of x
+ *   offsets  [n_experts+1] int32 (device)
+ *   max_rows host upper bound of offsets[n_experts] (sizes the launch)
+ *   w1       SWIGLU: [n_experts, 2, inter, hidden] = row-concatenated
+ *            [gate_proj; up_proj]; GELU_TANH: [n_experts, inter, hidden]
+ *   b1       GELU_TANH: [n_experts, inter] fp32 or NULL
+ *   w2       [n_experts, hidden, inter]
+ *   b2       GELU_TANH: [n_experts, hidden] fp32 or NULL
+ *   w1_scale [n_experts, (2*)inter], w2_scale [n_experts, hidden] fp32 per
+ *            output channel, required iff w_dtype == FP8_E4M3
+ *   h        [max_rows, inter] workspace in act_dtype
+ *   out      act_dtype; scatter_to_slots != 0: row perm[r] of [n_slots, hidden]
+ *            (this is _local_combine, ep_fwd.py:350-354, fused into the fc2
+ *            epilogue); else row r of [max_rows, hidden]
+ * Expert outputs are NOT scaled by the routing weight here (the skip cache
+ * stores them unscaled, ep_fwd.py:188); dice_combine applies the weights.
+ * Limits: hidden % 64 == 0, inter % 64 == 0, n_experts <= 256.
+ */
+int dice_grouped_mlp(const void *x, int act_dtype, const int32_t *perm,
+                     int slots_per_token, const int32_t *offsets,
+                     int n_experts, int64_t max_rows, int hidden, int inter,
+                     const void *w1, const float *b1, const void *w2,
+                     const float *b2, const float *w1_scale,
+                     const float *w2_scale, int w_dtype, int act_variant,
+                     void *h, void *out, int scatter_to_slots, void *stream);
+
+/*
+ * Combine.  Replaces mul_ by the routing weight + scatter_reduce_ of moe_infer
+ * (models.py:377-381), i.e. final.mul_(w).view(N,k,h).sum(1) of moe_infer_ep
+ * (expertpara/ep_fwd.py:190-195), the shared-expert add (models.py:355-357)
+ * and the skip-cache blend / put (ep_fwd.py:176-188):
+ *   y[t] = sum_j w[t,j] * row(t,j) (+ shared[t])
+ *   row(t,j) = cache_in[t]               if skip_mask[k*t+j] and cache_in
+ *            = slot_out[src(k*t+j)]      otherwise
+ *   src(s) = inv_perm[s] if inv_perm else s
+ *   cache_out[t] = slot_out[src(s)] for the slot s of token t with
+ *                  skip_mask[s] != 0     (if cache_out; the "put" of a full step)
+ * skip_mask must mark exactly one slot per token when a cache pointer is given.
+ * Deterministic: fp32 accumulation in slot order, one rounding to `dtype`.
+ */
+int dice_combine(const void *slot_out, const int32_t *inv_perm,
+                 const float *topk_weight, const void *shared_out,
+                 const uint8_t *skip_mask, const void *cache_in,
+                 void *cache_out, void *y, int dtype, int64_t n_tokens,
+                 int top_k, int hidden, void *stream);
+
+/*
+ * Per-output-channel fp8 quantiser for expert weights (build-defined, the
+ * reference has no fp8 path): scale[r] = amax(|w[r,:]|)/448 (1 if the row is
+ * all zero), q[r,c] = e4m3fn(rne(w[r,c]/scale[r])).
+ *   w [rows, cols] in_dtype in {BF16, F32};  q [rows, cols] uint8;  scale [rows]
+ */
+int dice_quantize_fp8_rowwise(const void *w, int in_dtype, int64_t rows,
+                              int64_t cols, uint8_t *q, float *scale,
+                              void *stream);
+
+/*
+ * Whole layer.  Replaces SparseMoeBlock.forward, inference branch
+ * (models.py:302-312,321-358) with moe_infer / moe_infer_ep as above:
+ * gate -> dispatch -> grouped MLP (+ shared expert MLP) -> combine, enqueued
+ * back to back on `stream` with no host synchronisation (the reference's
+ * .cpu() at models.py:366 disappears: offsets stay on the device).
+ */
+typedef struct dice_moe_layer {
+  int32_t hidden, inter, n_experts, top_k;
+  int32_t act_dtype;      /* DICE_BF16 or DICE_F32 */
+  int32_t w_dtype;        /* act_dtype, or DICE_FP8_E4M3 for routed experts */
+  int32_t act_variant;    /* DICE_ACT_* */
+  int32_t norm_topk_prob; /* models.py:170: 0 in the reference */
+  int32_t gate_w_dtype;
+  int32_t shared_inter;   /* 0 = no shared expert */
+  const void *gate_w;     /* [n_experts, hidden] */
+  const float *gate_bias; /* NULL in the reference */
+  const void *w1, *w2;    /* routed experts, layout of dice_grouped_mlp */
+  const float *b1, *b2, *w1_scale, *w2_scale;
+  const void *shared_w1, *shared_w2; /* one expert, act_dtype */
+  const float *shared_b1, *shared_b2;
+} dice_moe_layer_t;
+
+/* mode: 0 = plain step; 1 = full step that also writes cache_out ("put");
+ *       2 = skip step: slots with skip_mask != 0 are not recomputed and take
+ *           cache_in instead. */
+size_t dice_moe_workspace_bytes(const dice_moe_layer_t *layer, int64_t n_tokens);
+int dice_moe_forward(const dice_moe_layer_t *layer, const void *x,
+                     int64_t n_tokens, int mode, const uint8_t *skip_mask,
+                     const void *cache_in, void *cache_out, void *y,
+                     int32_t *topk_idx_out, float *topk_weight_out,
+                     void *workspace, size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DICE_MOE_H */

@@ -1,0 +1,489 @@
+"""CPU oracle for the DiT-MoE sparse expert layer of Cobalt-27/DICE.
+
+TEST INFRASTRUCTURE ONLY.  This file is a plain-torch CPU restatement of the
+reference algorithm.  It is imported by ``tests/``, by
+``__graft_entry__.smoke()`` and by the ``cpu_baseline`` leg of ``bench.py`` as
+the checker / the timed CPU baseline.  The product package never imports it:
+the HIP path raises when its shared library is missing instead of falling
+back to anything in this directory.
+
+Each function cites the reference lines it restates (paths are relative to
+the reference tree).  All arithmetic lives in stock torch calls, exactly as in
+the reference, which ships no native code.
+
+Pinning status (what independently fixes each function's result):
+
+* ``gate_forward``      - brute-force numpy restatement on tiny inputs,
+                          ordering/invariant checks (descending weights,
+                          distinct indices, sum<=1, renorm sums to 1).
+* ``moe_mlp``           - closed form ``down(silu(g)*u)`` evaluated in float64
+                          numpy; ``pretraining_tp`` split path must agree.
+* ``gelu_mlp``          - float64 numpy closed form of the tanh GELU.
+* ``moe_infer``         - per-token double loop (``dense_moe``), the reference's
+                          own fixture recipe (tests/test_ep.py:54-90, seeds
+                          42/43, atol 1e-6) committed under tests/golden.
+* ``moe_infer_ep_local``- must equal ``moe_infer`` on that same recipe, which
+                          is the property tests/test_ep.py:124 asserts.
+* skip path             - closed form of the blend, the "cache := own outputs
+                          reproduces the full step" identity, high/low slot
+                          swap symmetry.  The reference never tests its skip
+                          path, so beyond these identities it is
+                          "parity unpinned" by any reference-held vector.
+* bf16 / fp8 variants   - no reference code or vector exists for them
+                          ("parity unpinned" by the reference); they are the
+                          same functions evaluated in that dtype.
+"""
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+import torch.nn.functional as F
+
+
+# --------------------------------------------------------------------------- #
+# Router
+# --------------------------------------------------------------------------- #
+def gate_forward(
+    hidden_states: torch.Tensor,
+    weight: torch.Tensor,
+    top_k: int = 2,
+    norm_topk_prob: bool = False,
+    bias: Optional[torch.Tensor] = None,
+    fp32_gate: bool = True,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Restates ``MoEGate.forward`` inference branch (models.py:179-196,215-217).
+
+    ``logits = x W^T`` (no bias in the reference, models.py:184) -> softmax over
+    experts (:186) -> ``topk(k, sorted=False)`` (:191) -> optional renorm with
+    divisor ``sum + 1e-20`` (:194-196; off in the reference, :170).
+
+    ``fp32_gate`` upcasts x and W to fp32 first: the build fixes the router to
+    fp32 arithmetic for every activation dtype (exact for bf16/fp16 inputs).
+    With ``fp32_gate=False`` the linear runs in the tensors' own dtype as a
+    literal ``.to(dtype)`` of the reference module would.
+
+    torch's CPU ``topk`` for k*64 > E returns slot 0 = arg-max, slot 1 = runner
+    up even with ``sorted=False``; ``sorted=True`` is used here so the slot
+    order is explicit rather than an implementation accident.
+    Returns (topk_idx int64 [N,k], topk_weight [N,k], logits [N,E]).
+    """
+    h = hidden_states.shape[-1]
+    x = hidden_states.reshape(-1, h)
+    w = weight
+    if fp32_gate:
+        x = x.float()
+        w = w.float()
+        bias = None if bias is None else bias.float()
+    logits = F.linear(x, w, bias)
+    scores = logits.softmax(dim=-1)
+    topk_weight, topk_idx = torch.topk(scores, k=top_k, dim=-1, sorted=True)
+    if top_k > 1 and norm_topk_prob:
+        denominator = topk_weight.sum(dim=-1, keepdim=True) + 1e-20
+        topk_weight = topk_weight / denominator
+    return topk_idx, topk_weight, logits
+
+
+def gate_tie_rows(logits: torch.Tensor, top_k: int, tol: float = 1e-6) -> torch.Tensor:
+    """Rows whose top-(k+1) logits contain a gap <= tol.
+
+    On those rows an implementation with a different fp32 summation order may
+    legitimately pick another expert or slot order; everywhere else the indices
+    must match bit-exactly.
+    """
+    E = logits.shape[-1]
+    kk = min(top_k + 1, E)
+    top = torch.topk(logits.double(), k=kk, dim=-1, sorted=True).values
+    gaps = top[:, :-1] - top[:, 1:]
+    return (gaps <= tol).any(dim=-1)
+
+
+# --------------------------------------------------------------------------- #
+# Expert MLPs
+# --------------------------------------------------------------------------- #
+def moe_mlp(
+    x: torch.Tensor,
+    gate_proj: torch.Tensor,
+    up_proj: torch.Tensor,
+    down_proj: torch.Tensor,
+    pretraining_tp: int = 1,
+) -> torch.Tensor:
+    """Restates ``MoeMLP.forward`` (models.py:252-273): bias-free SwiGLU.
+
+    ``gate_proj``/``up_proj`` are ``[I, D]``, ``down_proj`` is ``[D, I]``.
+    ``pretraining_tp > 1`` follows the slice / cat / sum path (:253-269).
+    """
+    if pretraining_tp > 1:
+        inter = gate_proj.shape[0]
+        sl = inter // pretraining_tp
+        g_slices = gate_proj.split(sl, dim=0)
+        u_slices = up_proj.split(sl, dim=0)
+        d_slices = down_proj.split(sl, dim=1)
+        g = torch.cat([F.linear(x, g_slices[i]) for i in range(pretraining_tp)], dim=-1)
+        u = torch.cat([F.linear(x, u_slices[i]) for i in range(pretraining_tp)], dim=-1)
+        inter_states = (F.silu(g) * u).split(sl, dim=-1)
+        outs = [F.linear(inter_states[i], d_slices[i]) for i in range(pretraining_tp)]
+        return sum(outs)
+    return F.linear(F.silu(F.linear(x, gate_proj)) * F.linear(x, up_proj), down_proj)
+
+
+def gelu_mlp(
+    x: torch.Tensor,
+    fc1_w: torch.Tensor,
+    fc1_b: Optional[torch.Tensor],
+    fc2_w: torch.Tensor,
+    fc2_b: Optional[torch.Tensor],
+) -> torch.Tensor:
+    """``fc2(gelu_tanh(fc1(x)))``: the two-matrix MLP the benchmark configs name.
+
+    The reference only holds this as the activation of a commented-out dense
+    ``Mlp`` (models.py:496-497); the closed form is torch's
+    ``gelu(approximate='tanh')``.
+    """
+    return F.linear(F.gelu(F.linear(x, fc1_w, fc1_b), approximate="tanh"), fc2_w, fc2_b)
+
+
+class SwiGLUExpert:
+    """One reference ``MoeMLP`` (models.py:240-273) as plain tensors."""
+
+    def __init__(self, gate_proj, up_proj, down_proj, pretraining_tp: int = 1):
+        self.gate_proj = gate_proj
+        self.up_proj = up_proj
+        self.down_proj = down_proj
+        self.pretraining_tp = pretraining_tp
+
+    def __call__(self, x):
+        return moe_mlp(x, self.gate_proj, self.up_proj, self.down_proj, self.pretraining_tp)
+
+
+class GeluExpert:
+    def __init__(self, fc1_w, fc1_b, fc2_w, fc2_b):
+        self.fc1_w, self.fc1_b, self.fc2_w, self.fc2_b = fc1_w, fc1_b, fc2_w, fc2_b
+
+    def __call__(self, x):
+        return gelu_mlp(x, self.fc1_w, self.fc1_b, self.fc2_w, self.fc2_b)
+
+
+# --------------------------------------------------------------------------- #
+# Dispatch / combine
+# --------------------------------------------------------------------------- #
+def dispatch_tables(flat_expert_indices: torch.Tensor, num_experts: int):
+    """Counts, offsets and the canonical (stable) permutation.
+
+    ``bincount`` padded to E (ep_fwd.py:70-76), ``offsets = [0, cumsum]``
+    (models.py:366), ``perm = argsort(flat_idx, stable=True)``.  The reference
+    calls the default (unstable) ``argsort`` (models.py:365, ep_fwd.py:100), so
+    its order inside one expert's group is an artefact of torch's sort; the
+    layer output does not depend on it.  Canonical order = ascending flat slot
+    index inside each group.
+    Returns (counts [E], offsets [E+1], perm [S], inv_perm [S]) as int64.
+    """
+    counts = torch.bincount(flat_expert_indices, minlength=num_experts)
+    offsets = torch.zeros(num_experts + 1, dtype=torch.int64)
+    offsets[1:] = counts.cumsum(0)
+    perm = torch.argsort(flat_expert_indices, stable=True)
+    inv_perm = torch.empty_like(perm)
+    inv_perm[perm] = torch.arange(perm.numel(), dtype=perm.dtype)
+    return counts, offsets, perm, inv_perm
+
+
+@torch.no_grad()
+def moe_infer(
+    x: torch.Tensor,
+    experts: Sequence,
+    flat_expert_indices: torch.Tensor,
+    flat_expert_weights: torch.Tensor,
+    num_experts_per_tok: int,
+) -> torch.Tensor:
+    """Restates ``SparseMoeBlock.moe_infer`` (models.py:361-382).
+
+    sort slots by expert (:365) -> cumulative counts (:366) -> token = slot//k
+    (:367) -> per non-empty expert: gather, run expert, scale by the routing
+    weight of each slot (:373-377) -> ``scatter_reduce_('sum')`` into a
+    zero-initialised buffer that takes the expert output dtype (:380-381).
+    """
+    expert_cache = torch.zeros_like(x)
+    idxs = flat_expert_indices.argsort(stable=True)
+    tokens_per_expert = flat_expert_indices.bincount().cumsum(0).tolist()
+    token_idxs = idxs // num_experts_per_tok
+    for i, end_idx in enumerate(tokens_per_expert):
+        start_idx = 0 if i == 0 else tokens_per_expert[i - 1]
+        if start_idx == end_idx:
+            continue
+        exp_token_idx = token_idxs[start_idx:end_idx]
+        expert_out = experts[i](x[exp_token_idx])
+        expert_out = expert_out * flat_expert_weights[idxs[start_idx:end_idx]]
+        expert_cache = expert_cache.to(expert_out.dtype)
+        expert_cache.scatter_reduce_(
+            0, exp_token_idx.view(-1, 1).repeat(1, x.shape[-1]), expert_out, reduce="sum"
+        )
+    return expert_cache
+
+
+class EPSkipCache:
+    """Restates ``EPSkipCache`` (expertpara/ep_cache.py:188-235): one slot per
+    layer; ``get`` empties the slot (:215-220)."""
+
+    def __init__(self, capacity: int):
+        self.capacity = capacity
+        self.cache: List[Optional[torch.Tensor]] = [None] * capacity
+
+    def clear(self):
+        self.cache = [None] * self.capacity
+
+    def put(self, key: int, tensor: torch.Tensor):
+        assert isinstance(key, int)
+        self.cache[key] = tensor
+
+    def get(self, key: int):
+        value = self.cache[key]
+        self.cache[key] = None
+        return value
+
+    def contains(self, key: int) -> bool:
+        return self.cache[key] is not None
+
+    def tensors_size(self) -> int:
+        return sum(t.element_size() * t.numel() for t in self.cache if t is not None)
+
+
+def skip_mask(length: int, mode: str, rand_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Restates ``ep_skip_mask`` (expertpara/diep.py:72-90).
+
+    'high' marks slot 0 of every token pair (the higher router score), 'low'
+    slot 1, 'rand' one random slot per pair.  The reference draws the random
+    mask once per process and reuses it; here the caller owns it (pass the
+    same ``rand_mask`` back in to reuse it).
+    """
+    mask = torch.zeros(length, dtype=torch.bool)
+    if mode == "high":
+        mask[::2] = True
+    elif mode == "low":
+        mask[1::2] = True
+    elif mode == "rand":
+        if rand_mask is not None:
+            return rand_mask
+        n = length // 2
+        m2 = torch.zeros((n, 2), dtype=torch.bool)
+        m2[torch.arange(n), torch.randint(0, 2, (n,))] = True
+        mask = m2.view(-1)
+    else:
+        raise ValueError(f"Unknown skip mode: {mode}")
+    return mask
+
+
+def skip_now(enabled: bool, cache: EPSkipCache, layer: int, step: int, noskip_interval: int) -> bool:
+    """Restates ``ep_skip_now`` (expertpara/diep.py:61-68)."""
+    if not enabled or not cache.contains(layer):
+        return False
+    return step % noskip_interval != 0
+
+
+@torch.no_grad()
+def moe_infer_ep_local(
+    inp: torch.Tensor,
+    experts: Sequence,
+    flat_expert_indices: torch.Tensor,
+    flat_expert_weights: torch.Tensor,
+    num_experts_per_tok: int,
+    skip_mask_: Optional[torch.Tensor] = None,
+    skip_now_: Optional[bool] = None,
+    cache: Optional[EPSkipCache] = None,
+    cache_key: int = 0,
+) -> torch.Tensor:
+    """Restates ``moe_infer_ep`` at world_size 1, ``async_op=False``
+    (expertpara/ep_fwd.py:19-197) with the collectives reduced to identity.
+
+    skip step: keep only the retained slots (:57-66) -> bincount padded to E
+    (:70-76) -> sort, ``//k`` (:100-106) -> ``index_select`` (:345-347) -> per
+    expert MLP over contiguous row ranges (:200-211) -> un-permute with
+    ``index_copy_`` into zeros (:350-354) -> blend with / put into the skip
+    cache (:176-188) -> scale by the routing weights and sum the k slots of a
+    token (:190-195).
+    """
+    num_total_experts = len(experts)
+    partial_skip = skip_mask_ is not None
+    retain_mask = ~skip_mask_ if partial_skip else None
+    if skip_now_:
+        assert partial_skip, "skip is not enabled"
+        assert num_experts_per_tok == 2, "only support num_experts_per_tok == 2"
+        original_k = num_experts_per_tok
+        num_experts_per_tok //= 2
+        flat_expert_indices = flat_expert_indices[retain_mask]
+        assert flat_expert_indices.size(0) == inp.size(0) * num_experts_per_tok
+    else:
+        original_k = num_experts_per_tok
+
+    counts = flat_expert_indices.bincount()
+    if counts.size(0) != num_total_experts:
+        expanded = torch.zeros(num_total_experts, dtype=counts.dtype)
+        expanded[: counts.size(0)] = counts
+        counts = expanded
+
+    grouped_idx_dup = flat_expert_indices.argsort(stable=True)
+    grouped_idx = grouped_idx_dup // num_experts_per_tok
+    grouped_dup_inp = torch.index_select(inp, 0, grouped_idx)
+
+    mlp_outp = torch.empty_like(grouped_dup_inp)
+    start = 0
+    for e in range(num_total_experts):
+        c = int(counts[e])
+        if c:
+            mlp_outp[start:start + c] = experts[e](grouped_dup_inp[start:start + c])
+        start += c
+    assert start == grouped_dup_inp.size(0)
+
+    outp_dup = torch.zeros(mlp_outp.size(0), inp.shape[-1], dtype=mlp_outp.dtype)
+    outp_dup.index_copy_(0, grouped_idx_dup, mlp_outp)
+
+    final_outp = outp_dup
+    if partial_skip:
+        if outp_dup.size(0) != inp.size(0) * original_k:
+            assert outp_dup.size(0) == inp.size(0) * original_k // 2
+            dropped = cache.get(cache_key)
+            final_outp = outp_dup.new_empty((outp_dup.size(0) * 2, outp_dup.size(1)))
+            final_outp[retain_mask] = outp_dup
+            final_outp[skip_mask_] = dropped
+        else:
+            cache.put(cache_key, outp_dup[skip_mask_])
+    final_outp = final_outp * flat_expert_weights
+    expert_out = final_outp.view(inp.size(0), original_k, inp.size(1)).sum(dim=1)
+    assert expert_out.shape == inp.shape
+    return expert_out
+
+
+@torch.no_grad()
+def dense_moe(x, experts, topk_idx, topk_weight):
+    """Per-token brute force: ``y[t] = sum_j w[t,j] * E_{idx[t,j]}(x[t])``.
+
+    This is the training-branch formulation (models.py:314-319) evaluated one
+    token at a time; used to pin ``moe_infer`` on small inputs.
+    """
+    n, k = topk_idx.shape
+    rows = []
+    for t in range(n):
+        acc = None
+        for j in range(k):
+            o = experts[int(topk_idx[t, j])](x[t:t + 1])[0] * topk_weight[t, j]
+            acc = o if acc is None else acc + o
+        rows.append(acc)
+    return torch.stack(rows, 0)
+
+
+# --------------------------------------------------------------------------- #
+# Whole block
+# --------------------------------------------------------------------------- #
+class MoEBlockParams:
+    """Plain-tensor parameter set with the reference's state-dict layout
+    (models.py:280-300, expertpara/etrim.py:44): ``gate.weight [E,D]``,
+    ``experts.{e}.{gate,up,down}_proj.weight`` and
+    ``shared_experts.{gate,up,down}_proj.weight`` (intermediate
+    ``D * n_shared_experts``, models.py:292-296)."""
+
+    def __init__(self, gate_weight, experts, shared=None, top_k=2, norm_topk_prob=False,
+                 gate_bias=None):
+        self.gate_weight = gate_weight
+        self.experts = list(experts)
+        self.shared = shared
+        self.top_k = top_k
+        self.norm_topk_prob = norm_topk_prob
+        self.gate_bias = gate_bias
+
+
+def xavier_uniform(out_f: int, in_f: int, gen: torch.Generator) -> torch.Tensor:
+    """Xavier-uniform as ``DiT.initialize_weights`` applies to every Linear
+    (models.py:604-609)."""
+    a = math.sqrt(6.0 / (in_f + out_f))
+    return (torch.rand(out_f, in_f, generator=gen) * 2 - 1) * a
+
+
+def make_block_params(D, E, top_k=2, mlp_ratio=4, n_shared=2, seed=0, dtype=torch.float32,
+                      variant="swiglu", gate_std=0.02, pretraining_tp=1, gate_bias=None,
+                      norm_topk_prob=False) -> MoEBlockParams:
+    """Seeded synthetic weights of the benchmark configurations: router
+    ~N(0, 0.02), experts Xavier-uniform, zero biases."""
+    g = torch.Generator().manual_seed(seed)
+    gate_w = (torch.randn(E, D, generator=g) * gate_std).to(dtype)
+    inter = mlp_ratio * D
+    experts = []
+    for _ in range(E):
+        if variant == "swiglu":
+            experts.append(SwiGLUExpert(
+                xavier_uniform(inter, D, g).to(dtype), xavier_uniform(inter, D, g).to(dtype),
+                xavier_uniform(D, inter, g).to(dtype), pretraining_tp))
+        else:
+            experts.append(GeluExpert(
+                xavier_uniform(inter, D, g).to(dtype), torch.zeros(inter, dtype=dtype),
+                xavier_uniform(D, inter, g).to(dtype), torch.zeros(D, dtype=dtype)))
+    shared = None
+    if n_shared:
+        si = D * n_shared
+        if variant == "swiglu":
+            shared = SwiGLUExpert(
+                xavier_uniform(si, D, g).to(dtype), xavier_uniform(si, D, g).to(dtype),
+                xavier_uniform(D, si, g).to(dtype), pretraining_tp)
+        else:
+            shared = GeluExpert(
+                xavier_uniform(si, D, g).to(dtype), torch.zeros(si, dtype=dtype),
+                xavier_uniform(D, si, g).to(dtype), torch.zeros(D, dtype=dtype))
+    return MoEBlockParams(gate_w, experts, shared, top_k, norm_topk_prob, gate_bias)
+
+
+@torch.no_grad()
+def sparse_moe_block_forward(
+    params: MoEBlockParams,
+    hidden_states: torch.Tensor,
+    use_ep_path: bool = False,
+    skip_mask_: Optional[torch.Tensor] = None,
+    skip_now_: Optional[bool] = None,
+    cache: Optional[EPSkipCache] = None,
+    cache_key: int = 0,
+    fp32_gate: bool = True,
+):
+    """Restates ``SparseMoeBlock.forward`` inference branch
+    (models.py:302-312,321-358): gate -> flatten -> ``moe_infer`` (or the EP
+    data flow) -> reshape -> ``+ shared_experts(identity)``.
+
+    Routing weights are cast to the activation dtype before they scale expert
+    outputs, as the reference module does when it runs in one dtype.
+    Returns (y, topk_idx, topk_weight_fp32, logits).
+    """
+    identity = hidden_states
+    orig_shape = hidden_states.shape
+    topk_idx, topk_weight, logits = gate_forward(
+        hidden_states, params.gate_weight, params.top_k, params.norm_topk_prob,
+        params.gate_bias, fp32_gate)
+    x = hidden_states.reshape(-1, orig_shape[-1])
+    flat_idx = topk_idx.reshape(-1)
+    flat_w = topk_weight.to(x.dtype).reshape(-1, 1)
+    if use_ep_path or skip_mask_ is not None:
+        y = moe_infer_ep_local(x, params.experts, flat_idx, flat_w, params.top_k,
+                               skip_mask_, skip_now_, cache, cache_key)
+    else:
+        y = moe_infer(x, params.experts, flat_idx, flat_w, params.top_k)
+    y = y.view(*orig_shape)
+    if params.shared is not None:
+        y = y + params.shared(identity)
+    return y, topk_idx, topk_weight, logits
+
+
+# --------------------------------------------------------------------------- #
+# fp8 weight quantisation (build-defined; the reference has no fp8 code)
+# --------------------------------------------------------------------------- #
+E4M3_MAX = 448.0
+
+
+def quantize_fp8_rowwise(w: torch.Tensor):
+    """Per-output-channel (row) symmetric quantisation to OCP e4m3fn:
+    ``scale = amax(row)/448`` (1.0 for an all-zero row), ``q = rne(w/scale)``.
+    Returns (q float8_e4m3fn [rows, cols], scale fp32 [rows])."""
+    wf = w.float()
+    amax = wf.abs().amax(dim=1)
+    scale = torch.where(amax > 0, amax / E4M3_MAX, torch.ones_like(amax))
+    q = (wf / scale[:, None]).clamp(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn)
+    return q, scale
+
+
+def dequantize_fp8_rowwise(q: torch.Tensor, scale: torch.Tensor, dtype=torch.float32):
+    return (q.float() * scale[:, None]).to(dtype)

@@ -1,0 +1,50 @@
+"""Shared helpers of the GPU parity tests."""
+import torch
+
+from oracle import dice_oracle as O
+
+
+def rel_l2(a: torch.Tensor, b: torch.Tensor) -> float:
+    a, b = a.double().cpu(), b.double().cpu()
+    return float((a - b).norm() / b.norm().clamp_min(1e-30))
+
+
+def block_from_params(p: O.MoEBlockParams, D, variant="swiglu", dtype=torch.float32, device="cuda",
+                      ep=False, layer_idx=0):
+    """Builds the product module and loads the oracle's weights through the
+    reference's state-dict key layout."""
+    from dice_amd import ParaMode, SparseMoeBlock
+    E = len(p.experts)
+    inter = p.experts[0].gate_proj.shape[0] if variant == "swiglu" else p.experts[0].fc1_w.shape[0]
+    n_shared = None
+    if p.shared is not None:
+        si = p.shared.gate_proj.shape[0] if variant == "swiglu" else p.shared.fc1_w.shape[0]
+        n_shared = si // D
+    blk = SparseMoeBlock(D, mlp_ratio=inter // D, num_experts=E, num_experts_per_tok=p.top_k,
+                         pretraining_tp=1, layer_idx=layer_idx, total_layers=1,
+                         para_mode=ParaMode(ep=ep), variant=variant, n_shared_experts=n_shared)
+    sd = {"gate.weight": p.gate_weight}
+    def put(prefix, ex):
+        if variant == "swiglu":
+            sd[prefix + "gate_proj.weight"] = ex.gate_proj
+            sd[prefix + "up_proj.weight"] = ex.up_proj
+            sd[prefix + "down_proj.weight"] = ex.down_proj
+        else:
+            sd[prefix + "fc1.weight"], sd[prefix + "fc1.bias"] = ex.fc1_w, ex.fc1_b
+            sd[prefix + "fc2.weight"], sd[prefix + "fc2.bias"] = ex.fc2_w, ex.fc2_b
+    for e, ex in enumerate(p.experts):
+        put(f"experts.{e}.", ex)
+    if p.shared is not None:
+        put("shared_experts.", p.shared)
+    blk.load_state_dict(sd)
+    blk = blk.to(device=device, dtype=dtype).eval()
+    blk.gate.norm_topk_prob = p.norm_topk_prob
+    if p.gate_bias is not None:
+        blk.gate.bias = p.gate_bias.float().to(device)
+    return blk
+
+
+def zipf_bias(E, s=1.2):
+    pr = torch.tensor([(e + 1.0) ** -s for e in range(E)])
+    pr = pr / pr.sum()
+    return pr.log()

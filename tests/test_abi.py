@@ -1,0 +1,133 @@
+"""CPU-side checks of the C boundary and the host logic (no kernel launches)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "dice_moe.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dice_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from dice_amd import lib
+    cdll = lib.load()
+    names = _declared_symbols()
+    assert len(names) >= 11
+    for n in names:
+        assert hasattr(cdll, n), f"{n} declared in include/dice_moe.h but not exported"
+    for n in lib.EXPORTS:
+        assert n in names, f"{n} bound in python but not declared in the header"
+    assert cdll.dice_abi_version() == 1
+
+
+def test_layer_struct_matches_header_layout():
+    from dice_amd.lib import MoeLayerDesc
+    # 10 int32 fields then 12 pointers, naturally aligned.
+    assert MoeLayerDesc.gate_w.offset == 40
+    assert ctypes.sizeof(MoeLayerDesc) == 40 + 12 * 8
+
+
+def test_bad_arguments_are_reported_without_touching_a_gpu():
+    from dice_amd import lib
+    cdll = lib.load()
+    rc = cdll.dice_gate_topk(None, 0, None, 0, None, 4, 64, 8, 2, 0, None, None, None, None, None)
+    assert rc == -1 and b"null pointer" in cdll.dice_last_error()
+    one = ctypes.c_void_p(16)
+    rc = cdll.dice_gate_topk(one, 0, one, 0, None, 4, 63, 8, 2, 0, one, None, one, None, None)
+    assert rc == -1 and b"multiple of 8" in cdll.dice_last_error()
+    rc = cdll.dice_gate_topk(one, 0, one, 0, None, 4, 64, 65, 2, 0, one, None, one, None, None)
+    assert rc == -2
+    rc = cdll.dice_dispatch(one, None, 10, 300, one, one, one, one, None, 0, None)
+    assert rc == -2
+    rc = cdll.dice_combine(one, None, one, None, None, one, None, one, 1, 8, 2, 64, None)
+    assert rc == -1 and b"skip_mask" in cdll.dice_last_error()
+    rc = cdll.dice_grouped_mlp(one, 1, None, 1, one, 8, 16, 100, 256, one, None, one, None, None, None,
+                               1, 0, one, one, 0, None)
+    assert rc == -2 and b"multiples of 64" in cdll.dice_last_error()
+    with pytest.raises(lib.DiceError):
+        lib.check(rc)
+
+
+def test_cpu_tensors_are_refused():
+    from dice_amd import lib, ops
+    with pytest.raises(lib.DiceError, match="no CPU path"):
+        ops.gate_topk(torch.zeros(4, 64), torch.zeros(8, 64), 2)
+
+
+def test_module_interface_and_state_dict_keys():
+    """Same constructor, sub-module names and parameter shapes as the reference
+    block (models.py:280-300; key format expertpara/etrim.py:44)."""
+    from dice_amd import ParaMode, SparseMoeBlock
+    blk = SparseMoeBlock(128, mlp_ratio=4, num_experts=8, num_experts_per_tok=2, pretraining_tp=1,
+                         layer_idx=0, total_layers=1, para_mode=ParaMode())
+    sd = blk.state_dict()
+    assert sd["gate.weight"].shape == (8, 128)
+    for e in range(8):
+        assert sd[f"experts.{e}.gate_proj.weight"].shape == (512, 128)
+        assert sd[f"experts.{e}.up_proj.weight"].shape == (512, 128)
+        assert sd[f"experts.{e}.down_proj.weight"].shape == (128, 512)
+    assert sd["shared_experts.gate_proj.weight"].shape == (256, 128)
+    assert sd["shared_experts.down_proj.weight"].shape == (128, 256)
+    assert len(sd) == 1 + 8 * 3 + 3
+    blk.train()
+    with pytest.raises(Exception):
+        blk(torch.zeros(1, 4, 128))
+
+
+def test_multi_gpu_modes_are_refused():
+    from dice_amd import DiceError, ParaMode
+    with pytest.raises(DiceError):
+        ParaMode(ep=True, ep_async=True)
+    with pytest.raises(DiceError):
+        ParaMode(sp=True)
+
+
+def test_skip_policy_matches_oracle():
+    """dice_amd.diep mirrors the reference's control functions; the oracle's
+    restatement of diep.py:61-90 is the checker."""
+    from dice_amd import diep
+    from oracle import dice_oracle as O
+    for mode in ("high", "low"):
+        diep.ep_cache_init(cache_capacity=2, noskip_step=2, skip_mode=mode)
+        assert diep.ep_skip_enabled()
+        assert torch.equal(diep.ep_skip_mask(64), O.skip_mask(64, mode))
+    diep.ep_cache_init(cache_capacity=2, noskip_step=2, skip_mode="rand")
+    diep.ep_set_rand_mask(None)
+    m = diep.ep_skip_mask(64)
+    assert m.view(32, 2).sum(1).eq(1).all() and diep.ep_skip_mask(64) is m
+
+    ocache = O.EPSkipCache(2)
+    for i in range(50, 0, -1):
+        diep.ep_set_step(i)
+        if i == 50:
+            diep.ep_cache_clear()
+            ocache.clear()
+        for layer in (0, 1):
+            now = diep.ep_skip_now(layer)
+            assert now == O.skip_now(True, ocache, layer, i, 2)
+            if now:
+                assert diep.ep_skip_get(layer) is not None
+                ocache.get(layer)
+            else:
+                diep.ep_skip_put(layer, torch.zeros(3))
+                ocache.put(layer, torch.zeros(3))
+    assert diep.ep_cached_tensors_size() == ocache.tensors_size()
+    diep.ep_cache_init(cache_capacity=2, noskip_step=1)
+    assert not diep.ep_skip_enabled() and not diep.ep_skip_now(0)
+
+
+def test_forced_sync_schedule():
+    from dice_amd import diep
+    assert diep.ep_forced_sync(50, 50)
+    assert not diep.ep_forced_sync(49, 50)
+    assert diep.ep_forced_sync(48, 50, ep_async_warm_up=2)
+    assert not diep.ep_forced_sync(47, 50, ep_async_warm_up=2)
+    assert diep.ep_forced_sync(40, 50, strided_sync=10)
+    assert diep.ep_forced_sync(2, 50, strided_sync=100, ep_async_cool_down=3)

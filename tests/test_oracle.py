@@ -1,0 +1,231 @@
+"""Pins the CPU oracle: golden fixtures, closed forms, invariants, brute force.
+
+None of these tests retype an oracle formula in torch; each compares against a
+float64 numpy definition, a fixture computed without the oracle, or a property
+the mathematics fixes.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import dice_oracle as O
+
+
+class LinearExpert:
+    def __init__(self, w, b):
+        self.w, self.b = torch.from_numpy(w), torch.from_numpy(b)
+
+    def __call__(self, x):
+        return torch.nn.functional.linear(x, self.w, self.b)
+
+
+@pytest.mark.parametrize("seed", [42, 43])
+def test_moe_infer_matches_reference_recipe(golden_dir, seed):
+    """tests/test_ep.py's recipe: single-node and EP data flows agree with the
+    per-token float64 definition within the reference's own tolerance."""
+    z = np.load(os.path.join(golden_dir, f"ep_recipe_seed{seed}.npz"))
+    experts = [LinearExpert(z["expert_w"][e], z["expert_b"][e]) for e in range(8)]
+    for it in range(4):
+        x = torch.from_numpy(z[f"inp{it}"])
+        idx = torch.from_numpy(z[f"idx{it}"])
+        w = torch.from_numpy(z[f"w{it}"])
+        want = torch.from_numpy(z[f"y{it}"]).float()
+        got = O.moe_infer(x, experts, idx, w, 2)
+        got_ep = O.moe_infer_ep_local(x, experts, idx, w, 2)
+        assert torch.allclose(got, want, atol=1e-6, rtol=1e-5)
+        assert torch.allclose(got_ep, want, atol=1e-6, rtol=1e-5)
+        assert torch.allclose(got_ep, got, atol=1e-6)
+
+
+def test_gate_against_bruteforce_fixture(golden_dir):
+    z = np.load(os.path.join(golden_dir, "gate_small.npz"))
+    idx, w, logits = O.gate_forward(torch.from_numpy(z["x"]), torch.from_numpy(z["w"]), 2)
+    assert torch.equal(idx, torch.from_numpy(z["idx"]))
+    np.testing.assert_allclose(w.numpy(), z["weight"], rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(logits.numpy(), z["logits"], rtol=1e-5, atol=1e-6)
+    _, wn, _ = O.gate_forward(torch.from_numpy(z["x"]), torch.from_numpy(z["w"]), 2, norm_topk_prob=True)
+    np.testing.assert_allclose(wn.numpy(), z["weight_norm"], rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("E,k", [(8, 2), (16, 2), (16, 4), (5, 3)])
+def test_gate_invariants(E, k):
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(301, 64, generator=g)
+    w = torch.randn(E, 64, generator=g) * 0.2
+    idx, wt, logits = O.gate_forward(x, w, k)
+    assert idx.dtype == torch.int64 and idx.shape == (301, k)
+    assert (wt[:, :-1] >= wt[:, 1:]).all(), "slot order must be descending score"
+    assert all(len(set(r.tolist())) == k for r in idx), "experts of a token are distinct"
+    assert (wt.sum(-1) <= 1 + 1e-6).all() and (wt > 0).all()
+    # slot 0 is the arg-max of the logits; the top-k set equals numpy's.
+    assert torch.equal(idx[:, 0], logits.argmax(-1))
+    want = np.argsort(-logits.double().numpy(), axis=-1, kind="stable")[:, :k]
+    assert np.array_equal(np.sort(idx.numpy(), -1), np.sort(want, -1))
+    _, wn, _ = O.gate_forward(x, w, k, norm_topk_prob=True)
+    assert torch.allclose(wn.sum(-1), torch.ones(301), atol=1e-6)
+    # bias extension shifts logits
+    b = torch.randn(E, generator=g)
+    _, _, lb = O.gate_forward(x, w, k, bias=b)
+    assert torch.allclose(lb, logits + b, atol=1e-6)
+
+
+def test_gate_bf16_inputs_use_fp32_arithmetic():
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(64, 128, generator=g).bfloat16()
+    w = (torch.randn(8, 128, generator=g) * 0.02).bfloat16()
+    _, _, logits = O.gate_forward(x, w, 2)
+    ref = x.double() @ w.double().T
+    assert logits.dtype == torch.float32
+    assert torch.allclose(logits.double(), ref, atol=1e-6)
+
+
+def test_tie_rows_flags_small_gaps():
+    logits = torch.tensor([[3.0, 2.0, 1.0, 0.0], [3.0, 3.0 - 5e-7, 1.0, 0.0], [3.0, 2.0, 2.0, 0.0],
+                           [3.0, 2.0, 1.0, 1.0]])
+    assert O.gate_tie_rows(logits, 2).tolist() == [False, True, True, False]
+
+
+def _np_silu(v):
+    return v / (1.0 + np.exp(-v))
+
+
+@pytest.mark.parametrize("tp", [1, 2])
+def test_swiglu_closed_form(tp):
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((19, 32))
+    wg, wu = rng.standard_normal((64, 32)) * 0.2, rng.standard_normal((64, 32)) * 0.2
+    wd = rng.standard_normal((32, 64)) * 0.2
+    want = (_np_silu(x @ wg.T) * (x @ wu.T)) @ wd.T
+    got = O.moe_mlp(*(torch.from_numpy(a).float() for a in (x, wg, wu, wd)), pretraining_tp=tp)
+    np.testing.assert_allclose(got.numpy(), want, rtol=1e-4, atol=1e-5)
+    # a transposed down_proj or swapped gate/up must not pass
+    swapped = O.moe_mlp(*(torch.from_numpy(a).float() for a in (x, wu, wg, wd)), pretraining_tp=tp)
+    assert not np.allclose(swapped.numpy(), want, rtol=1e-2, atol=1e-3)
+
+
+def test_gelu_closed_form():
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((11, 16))
+    w1, b1 = rng.standard_normal((48, 16)) * 0.3, rng.standard_normal(48) * 0.1
+    w2, b2 = rng.standard_normal((16, 48)) * 0.3, rng.standard_normal(16) * 0.1
+    a = x @ w1.T + b1
+    gelu = 0.5 * a * (1 + np.tanh(np.sqrt(2 / np.pi) * (a + 0.044715 * a ** 3)))
+    want = gelu @ w2.T + b2
+    got = O.gelu_mlp(*(torch.from_numpy(v).float() for v in (x, w1, b1, w2, b2)))
+    np.testing.assert_allclose(got.numpy(), want, rtol=1e-4, atol=1e-5)
+
+
+def test_dispatch_tables_invariants():
+    g = torch.Generator().manual_seed(5)
+    idx = torch.randint(0, 8, (2048,), generator=g)
+    idx[idx == 3] = 4  # an empty expert
+    counts, offsets, perm, inv = O.dispatch_tables(idx, 8)
+    assert counts.tolist() == np.bincount(idx.numpy(), minlength=8).tolist()
+    assert counts[3] == 0
+    assert offsets.tolist() == [0] + np.cumsum(counts.numpy()).tolist()
+    assert sorted(perm.tolist()) == list(range(2048))
+    grouped = idx[perm]
+    assert (grouped[1:] >= grouped[:-1]).all()
+    assert torch.equal(inv[perm], torch.arange(2048))
+    for e in range(8):
+        seg = perm[offsets[e]:offsets[e + 1]]
+        assert (seg[1:] > seg[:-1]).all(), "stable: ascending slot inside a group"
+    # group membership equals the reference's unstable argsort
+    ref = idx.argsort()
+    for e in range(8):
+        assert set(ref[offsets[e]:offsets[e + 1]].tolist()) == set(perm[offsets[e]:offsets[e + 1]].tolist())
+
+
+def _small_block(dtype=torch.float32, variant="swiglu", seed=0, E=8, D=64):
+    return O.make_block_params(D, E, top_k=2, mlp_ratio=2, n_shared=2, seed=seed, dtype=dtype,
+                               variant=variant, gate_std=0.5)
+
+
+@pytest.mark.parametrize("variant", ["swiglu", "gelu_tanh"])
+def test_block_equals_dense_definition(variant):
+    p = _small_block(variant=variant)
+    x = torch.randn(2, 24, 64, generator=torch.Generator().manual_seed(6))
+    y, idx, wt, _ = O.sparse_moe_block_forward(p, x)
+    y_ep, _, _, _ = O.sparse_moe_block_forward(p, x, use_ep_path=True)
+    dense = O.dense_moe(x.view(-1, 64), p.experts, idx, wt) + p.shared(x.view(-1, 64))
+    assert torch.allclose(y.view(-1, 64), dense, atol=1e-5)
+    assert torch.allclose(y_ep, y, atol=1e-5)
+
+
+def test_skip_identities():
+    """(i) a skip step that blends with THIS step's own unscaled outputs equals
+    the full step; (ii) closed form of the blend with a foreign cache;
+    (iii) 'high' and 'low' exchange roles when the two slots are swapped."""
+    p = _small_block(seed=9)
+    g = torch.Generator().manual_seed(10)
+    x = torch.randn(40, 64, generator=g)
+    idx, wt, _ = O.gate_forward(x, p.gate_weight, 2)
+    flat_idx, flat_w = idx.reshape(-1), wt.reshape(-1, 1)
+    full = O.moe_infer_ep_local(x, p.experts, flat_idx, flat_w, 2)
+    for mode in ("high", "low", "rand"):
+        mask = O.skip_mask(80, mode)
+        assert mask.view(40, 2).sum(1).eq(1).all()
+        cache = O.EPSkipCache(1)
+        put = O.moe_infer_ep_local(x, p.experts, flat_idx, flat_w, 2, mask, False, cache, 0)
+        assert torch.allclose(put, full, atol=1e-6), "a put step returns the full result"
+        assert cache.contains(0) and cache.cache[0].shape == (40, 64)
+        skipped = O.moe_infer_ep_local(x, p.experts, flat_idx, flat_w, 2, mask, True, cache, 0)
+        assert torch.allclose(skipped, full, atol=1e-5)
+        assert not cache.contains(0), "get empties the entry"
+        # foreign cache: closed form per token
+        C = torch.randn(40, 64, generator=g)
+        cache.put(0, C)
+        got = O.moe_infer_ep_local(x, p.experts, flat_idx, flat_w, 2, mask, True, cache, 0)
+        m2 = mask.view(40, 2)
+        for t in range(40):
+            s = int(m2[t].nonzero()[0])
+            r = 1 - s
+            want = wt[t, s] * C[t] + wt[t, r] * p.experts[int(idx[t, r])](x[t:t + 1])[0]
+            assert torch.allclose(got[t], want, atol=1e-5)
+    # slot swap symmetry
+    C = torch.randn(40, 64, generator=g)
+    sw_idx, sw_w = idx.flip(1).reshape(-1), wt.flip(1).reshape(-1, 1)
+    c1, c2 = O.EPSkipCache(1), O.EPSkipCache(1)
+    c1.put(0, C)
+    c2.put(0, C)
+    a = O.moe_infer_ep_local(x, p.experts, flat_idx, flat_w, 2, O.skip_mask(80, "high"), True, c1, 0)
+    b = O.moe_infer_ep_local(x, p.experts, sw_idx, sw_w, 2, O.skip_mask(80, "low"), True, c2, 0)
+    assert torch.allclose(a, b, atol=1e-6)
+
+
+def test_skip_schedule_interval_two():
+    """Reference schedule (rectified_flow.py:83-105, diep.py:61-68): steps count
+    down 50..1, the first is full, then odd steps skip and even steps are full."""
+    cache = O.EPSkipCache(1)
+    pattern = []
+    for i in range(50, 0, -1):
+        if i == 50:
+            cache.clear()
+        now = O.skip_now(True, cache, 0, i, 2)
+        pattern.append(now)
+        if now:
+            assert cache.get(0) is not None
+        else:
+            cache.put(0, torch.zeros(1))
+    assert pattern[0] is False
+    assert pattern[1:] == [(i % 2 != 0) for i in range(49, 0, -1)]
+    assert not any(a and b for a, b in zip(pattern, pattern[1:])), "never two skips in a row"
+
+
+def test_fp8_rowwise_quantiser_properties():
+    g = torch.Generator().manual_seed(11)
+    w = O.xavier_uniform(96, 64, g)
+    w[5] = 0
+    q, s = O.quantize_fp8_rowwise(w)
+    assert q.dtype == torch.float8_e4m3fn and s.shape == (96,)
+    assert s[5] == 1.0 and (q[5].float() == 0).all()
+    deq = O.dequantize_fp8_rowwise(q, s)
+    amax = w.abs().amax(1)
+    # the row maximum maps to +-448 exactly; e4m3 keeps 3 mantissa bits
+    assert torch.allclose(deq.abs().amax(1)[amax > 0], amax[amax > 0], rtol=1e-6)
+    rel = (deq - w).abs() / amax[:, None].clamp_min(1e-30)
+    assert rel.max() <= 2 ** -4 + 1e-6
+    big = w.abs() > amax[:, None] / 16
+    assert ((deq - w).abs()[big] <= w.abs()[big] * 2 ** -4 + 1e-9).all()
