@@ -83,14 +83,13 @@ int check_mlp_shape(const char *who, int act_dtype, int w_dtype, int act_variant
 }  // namespace
 }  // namespace dice
 
-extern "C" int dice_grouped_mlp(const void *x, int act_dtype, const int32_t *perm,
-                                int slots_per_token, const int32_t *offsets, int n_experts,
-                                int64_t max_rows, int hidden, int inter, const void *w1,
-                                const float *b1, const void *w2, const float *b2,
-                                const float *w1_scale, const float *w2_scale, int w_dtype,
-                                int act_variant, void *h, void *out, int scatter_to_slots,
-                                void *stream) {
-  using namespace dice;
+namespace dice {
+namespace {
+int grouped_mlp_impl(int stages, const void *x, int act_dtype, const int32_t *perm,
+                     int slots_per_token, const int32_t *offsets, int n_experts, int64_t max_rows,
+                     int hidden, int inter, const void *w1, const float *b1, const void *w2,
+                     const float *b2, const float *w1_scale, const float *w2_scale, int w_dtype,
+                     int act_variant, void *h, void *out, int scatter_to_slots, void *stream) {
   DICE_REQUIRE(x && offsets && w1 && w2 && h && out, DICE_ERR_BAD_ARG, "dice_grouped_mlp: null pointer");
   int rc = check_mlp_shape("dice_grouped_mlp", act_dtype, w_dtype, act_variant, hidden, inter, n_experts);
   if (rc) return rc;
@@ -125,8 +124,11 @@ extern "C" int dice_grouped_mlp(const void *x, int act_dtype, const int32_t *per
   p1.c_perm = nullptr;
   p1.n = inter;
   p1.k = hidden;
-  rc = run_gemm(p1, swiglu ? kFc1Swiglu : kFc1Gelu, act_dtype, w_dtype, max_rows, s);
-  if (rc) return rc;
+  if (stages & 1) {
+    rc = run_gemm(p1, swiglu ? kFc1Swiglu : kFc1Gelu, act_dtype, w_dtype, max_rows, s);
+    if (rc) return rc;
+  }
+  if (!(stages & 2)) return DICE_OK;
 
   GemmParams p2{};
   p2.a = h;
@@ -146,6 +148,34 @@ extern "C" int dice_grouped_mlp(const void *x, int act_dtype, const int32_t *per
   p2.n = hidden;
   p2.k = inter;
   return run_gemm(p2, kFc2, act_dtype, w_dtype, max_rows, s);
+}
+}  // namespace
+}  // namespace dice
+
+extern "C" int dice_grouped_mlp(const void *x, int act_dtype, const int32_t *perm,
+                                int slots_per_token, const int32_t *offsets, int n_experts,
+                                int64_t max_rows, int hidden, int inter, const void *w1,
+                                const float *b1, const void *w2, const float *b2,
+                                const float *w1_scale, const float *w2_scale, int w_dtype,
+                                int act_variant, void *h, void *out, int scatter_to_slots,
+                                void *stream) {
+  return dice::grouped_mlp_impl(3, x, act_dtype, perm, slots_per_token, offsets, n_experts, max_rows,
+                                hidden, inter, w1, b1, w2, b2, w1_scale, w2_scale, w_dtype,
+                                act_variant, h, out, scatter_to_slots, stream);
+}
+
+extern "C" int dice_grouped_mlp_stage(int stage, const void *x, int act_dtype, const int32_t *perm,
+                                      int slots_per_token, const int32_t *offsets, int n_experts,
+                                      int64_t max_rows, int hidden, int inter, const void *w1,
+                                      const float *b1, const void *w2, const float *b2,
+                                      const float *w1_scale, const float *w2_scale, int w_dtype,
+                                      int act_variant, void *h, void *out, int scatter_to_slots,
+                                      void *stream) {
+  if (stage != 1 && stage != 2)
+    return dice::fail(DICE_ERR_BAD_ARG, "dice_grouped_mlp_stage: stage %d (1 = fc1, 2 = fc2)", stage);
+  return dice::grouped_mlp_impl(stage, x, act_dtype, perm, slots_per_token, offsets, n_experts,
+                                max_rows, hidden, inter, w1, b1, w2, b2, w1_scale, w2_scale, w_dtype,
+                                act_variant, h, out, scatter_to_slots, stream);
 }
 
 extern "C" size_t dice_moe_workspace_bytes(const dice_moe_layer_t *layer, int64_t n_tokens) {

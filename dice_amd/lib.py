@@ -34,6 +34,8 @@ EXPORTS = [
     "dice_dispatch",
     "dice_gather_rows",
     "dice_grouped_mlp",
+    "dice_grouped_mlp_stage",
+    "dice_set_gemm_config",
     "dice_combine",
     "dice_quantize_fp8_rowwise",
     "dice_moe_workspace_bytes",
@@ -89,6 +91,8 @@ def load() -> ctypes.CDLL:
     lib.dice_grouped_mlp.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int64, c_int,
                                      c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]
+    lib.dice_grouped_mlp_stage.restype = c_int
+    lib.dice_grouped_mlp_stage.argtypes = [c_int] + lib.dice_grouped_mlp.argtypes
     lib.dice_combine.restype = c_int
     lib.dice_combine.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_void_p, c_int, c_int64, c_int, c_int, c_void_p]

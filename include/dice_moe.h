@@ -134,6 +134,22 @@ int dice_grouped_mlp(const void *x, int act_dtype, const int32_t *perm,
                      void *h, void *out, int scatter_to_slots, void *stream);
 
 /*
+ * One stage of dice_grouped_mlp on its own, same arguments: stage 1 = fc1 with
+ * its activation (writes h), stage 2 = fc2 (reads h, writes out).  For callers
+ * that schedule the two GEMMs themselves (other streams, per-kernel timing as
+ * the reference's CudaProfiler scopes do around "moe.mlp", models.py:375).
+ */
+int dice_grouped_mlp_stage(int stage, const void *x, int act_dtype,
+                           const int32_t *perm, int slots_per_token,
+                           const int32_t *offsets, int n_experts,
+                           int64_t max_rows, int hidden, int inter,
+                           const void *w1, const float *b1, const void *w2,
+                           const float *b2, const float *w1_scale,
+                           const float *w2_scale, int w_dtype, int act_variant,
+                           void *h, void *out, int scatter_to_slots,
+                           void *stream);
+
+/*
  * Combine.  Replaces mul_ by the routing weight + scatter_reduce_ of moe_infer
  * (models.py:377-381), i.e. final.mul_(w).view(N,k,h).sum(1) of moe_infer_ep
  * (expertpara/ep_fwd.py:190-195), the shared-expert add (models.py:355-357)
@@ -195,6 +211,13 @@ int dice_moe_forward(const dice_moe_layer_t *layer, const void *x,
                      const void *cache_in, void *cache_out, void *y,
                      int32_t *topk_idx_out, float *topk_weight_out,
                      void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Tuning hook, no counterpart in the reference: selects the tile shape of the
+ * bf16/fp8 expert GEMMs per stage (0 = library default).  Process-wide; meant
+ * for benchmarks that compare tilings, not for the drop-in path.
+ */
+int dice_set_gemm_config(int fc1_cfg, int fc2_cfg);
 
 #ifdef __cplusplus
 }
