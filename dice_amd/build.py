@@ -25,6 +25,7 @@ SOURCES = [
     "quant.hip",
     "grouped_gemm_f32.hip",
     "grouped_gemm_bf16.hip",
+    "grouped_gemm_persist.hip",
     "grouped_mlp.hip",
 ]
 

@@ -19,8 +19,22 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+// LDS staging is written as packed bf16 and read back as raw 16-byte chunks;
+// these views may alias anything.
+typedef u32x4_t __attribute__((may_alias)) u32x4_any_t;
+typedef u32x2_t __attribute__((may_alias)) u32x2_any_t;
 
 constexpr int kWave = 64;
+
+// Orders LDS traffic between the lanes of one wavefront: everything written
+// before is visible to every lane after.  (Lanes exchange data through LDS in
+// the GEMM epilogues; without this the compiler may run one side of a
+// divergent branch's reads ahead of the other side's writes.)
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
 
 // Records a printf-style message for dice_last_error() and returns `code`.
 int fail(int code, const char *fmt, ...);

@@ -105,6 +105,43 @@ __device__ __forceinline__ float gelu_tanh_f(float x) {
   return 0.5f * x * (1.0f + tanhf(inner));
 }
 
+// Hardware-transcendental forms for the bf16 kernels (v_exp_f32 / v_rcp_f32,
+// about 1 ulp each, far below bf16 resolution): sigmoid(z) = 1/(1 + 2^(-z log2 e)).
+__device__ __forceinline__ float sigmoid_fast(float z) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * z));
+}
+__device__ __forceinline__ float silu_fast(float g) { return g * sigmoid_fast(g); }
+// 0.5 x (1 + tanh(u)) = x sigmoid(2u)
+__device__ __forceinline__ float gelu_tanh_fast(float x) {
+  const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+  return x * sigmoid_fast(2.0f * k0 * (x + k1 * x * x * x));
+}
+
+// One grouped GEMM of a persistent launch: contiguous grouped activation rows
+// (row r of expert e = a + (offsets[e] + r) * lda), bf16 weights
+// [n_experts, w_rows, k], output rows in the same grouped order.
+struct PersistProblem {
+  const void *a;
+  int lda;
+  const int32_t *offsets;  // [n_experts + 1], device
+  int n_experts;
+  const void *w;
+  int w_rows;
+  int up_offset;           // SwiGLU: first up_proj row of an expert's block
+  const float *bias;       // [n_experts, n] or NULL
+  void *c;
+  int ldc;
+  int n, k;
+};
+constexpr int kMaxPersistProblems = 3;
+struct PersistBatch {
+  int n_problems;
+  PersistProblem prob[kMaxPersistProblems];
+};
+bool persist_supported(const PersistBatch &b, int mode);
+bool gemm_config_wants_persistent();  // tuning hook state: both stages set to the persistent kernel
+int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s);
+
 int launch_grouped_gemm_f32(const GemmParams &p, int mode, int64_t max_rows, hipStream_t s);
 int launch_grouped_gemm_bf16(const GemmParams &p, int mode, int w_dtype, int64_t max_rows,
                              hipStream_t s);

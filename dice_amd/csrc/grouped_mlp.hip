@@ -107,6 +107,27 @@ int grouped_mlp_impl(int stages, const void *x, int act_dtype, const int32_t *pe
   hipStream_t s = (hipStream_t)stream;
   const bool swiglu = act_variant == DICE_ACT_SWIGLU;
 
+  // Contiguous grouped rows + bf16 weights: the persistent kernel applies.
+  if (!perm && act_dtype == DICE_BF16 && w_dtype == DICE_BF16 && gemm_config_wants_persistent()) {
+    PersistBatch pb1{};
+    pb1.n_problems = 1;
+    pb1.prob[0] = PersistProblem{x, hidden, offsets, n_experts, w1, swiglu ? 2 * inter : inter, inter,
+                                 swiglu ? nullptr : b1, h, inter, inter, hidden};
+    PersistBatch pb2{};
+    pb2.n_problems = 1;
+    pb2.prob[0] = PersistProblem{h, inter, offsets, n_experts, w2, hidden, 0, swiglu ? nullptr : b2,
+                                 out, hidden, hidden, inter};
+    const int m1 = swiglu ? kFc1Swiglu : kFc1Gelu;
+    if (persist_supported(pb1, m1) && persist_supported(pb2, kFc2)) {
+      if (stages & 1) {
+        rc = launch_grouped_gemm_persist(pb1, m1, s);
+        if (rc) return rc;
+      }
+      if (stages & 2) return launch_grouped_gemm_persist(pb2, kFc2, s);
+      return DICE_OK;
+    }
+  }
+
   GemmParams p1{};
   p1.a = x;
   p1.a_perm = perm;
@@ -230,6 +251,44 @@ extern "C" int dice_moe_forward(const dice_moe_layer_t *L, const void *x, int64_
   if (rc) return rc;
   // A skip step recomputes one slot per token.
   const int64_t max_rows = mode == 2 ? n_tokens * (L->top_k - 1) : slots;
+  const uint8_t *mask = mode == 0 ? nullptr : skip_mask;
+
+  // bf16 path: gather the grouped rows once, then two persistent launches,
+  // each covering the routed experts and the shared expert together.
+  if (L->act_dtype == DICE_BF16 && L->w_dtype == DICE_BF16) {
+    const bool swiglu = L->act_variant == DICE_ACT_SWIGLU;
+    const int m1 = swiglu ? kFc1Swiglu : kFc1Gelu;
+    PersistBatch f1{}, f2{};
+    void *xg = w.slot_out;  // the gathered rows die before fc2 writes its outputs there
+    f1.prob[0] = PersistProblem{xg, L->hidden, w.offsets, L->n_experts, L->w1,
+                                swiglu ? 2 * L->inter : L->inter, L->inter, swiglu ? nullptr : L->b1,
+                                w.h, L->inter, L->inter, L->hidden};
+    f2.prob[0] = PersistProblem{w.h, L->inter, w.offsets, L->n_experts, L->w2, L->hidden, 0,
+                                swiglu ? nullptr : L->b2, w.slot_out, L->hidden, L->hidden, L->inter};
+    f1.n_problems = f2.n_problems = 1;
+    if (L->shared_inter > 0) {
+      const int si = L->shared_inter;
+      f1.prob[1] = PersistProblem{x, L->hidden, w.shared_offsets, 1, L->shared_w1, swiglu ? 2 * si : si, si,
+                                  swiglu ? nullptr : L->shared_b1, w.shared_h, si, si, L->hidden};
+      f2.prob[1] = PersistProblem{w.shared_h, si, w.shared_offsets, 1, L->shared_w2, L->hidden, 0,
+                                  swiglu ? nullptr : L->shared_b2, w.shared_out, L->hidden, L->hidden, si};
+      f1.n_problems = f2.n_problems = 2;
+    }
+    if (persist_supported(f1, m1) && persist_supported(f2, kFc2)) {
+      rc = dice_gather_rows(x, L->act_dtype, w.perm, L->top_k, max_rows, L->hidden, xg, stream);
+      if (rc) return rc;
+      if (L->shared_inter > 0)
+        hipLaunchKernelGGL(set_range_kernel, dim3(1), dim3(64), 0, s, w.shared_offsets, (int32_t)n_tokens);
+      rc = launch_grouped_gemm_persist(f1, m1, s);
+      if (rc) return rc;
+      rc = launch_grouped_gemm_persist(f2, kFc2, s);
+      if (rc) return rc;
+      return dice_combine(w.slot_out, w.inv_perm, wt, w.shared_out, mask, mode == 2 ? cache_in : nullptr,
+                          mode == 1 ? cache_out : nullptr, y, L->act_dtype, n_tokens, L->top_k, L->hidden,
+                          stream);
+    }
+  }
+
   rc = dice_grouped_mlp(x, L->act_dtype, w.perm, L->top_k, w.offsets, L->n_experts, max_rows,
                         L->hidden, L->inter, L->w1, L->b1, L->w2, L->b2, L->w1_scale, L->w2_scale,
                         L->w_dtype, L->act_variant, w.h, w.slot_out, 1, stream);
