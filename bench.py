@@ -22,6 +22,8 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
+# HBM bytes of one fc1 launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/); None until measured.
+FC1_HBM_TRAFFIC_BYTES = None
 
 N_TOKENS, D, E, TOPK, RATIO = 8192, 1152, 8, 2, 4
 
@@ -73,54 +75,28 @@ def time_layer(blk, x, steps, warmup):
 
 
 def time_stages(blk, x, steps):
-    """Runs the layer stage by stage through the C ABI with a HIP event after
-    every launch (torch's current stream is the stream the library launches on)
-    and returns the mean duration of each kernel in ms."""
-    from dice_amd import ops
-    from dice_amd.lib import check, dtype_code, load, ptr, stream_ptr
-    p = blk._packed
-    n, k = x.shape[0], TOPK
-    dev = x.device
+    """Mean duration of every launch of the layer in ms, from the library's own
+    stage timers: HIP events recorded between the launches of dice_moe_forward
+    on the stream it launches on (torch's current stream)."""
+    import ctypes
+    from dice_amd.lib import check, load
     lib = load()
-    names = ["gate", "dispatch", "fc1", "fc2", "shared_fc1", "shared_fc2", "combine"]
-    acc = {s: 0.0 for s in names}
-    h = torch.empty((n * k, blk.inter), dtype=x.dtype, device=dev)
-    slot_out = torch.empty((n * k, D), dtype=x.dtype, device=dev)
-    si = p.sw2.shape[-1]
-    sh = torch.empty((n, si), dtype=x.dtype, device=dev)
-    sout = torch.empty((n, D), dtype=x.dtype, device=dev)
-    soff = torch.tensor([0, n], dtype=torch.int32, device=dev)
-    variant = ops.VARIANTS[blk.variant]
-
-    def stage(which, xin, perm, spt, off, ne, rows, inter, w1, b1, w2, b2, hbuf, out, scatter):
-        check(lib.dice_grouped_mlp_stage(which, ptr(xin), dtype_code(x.dtype), ptr(perm), spt, ptr(off), ne,
-                                         rows, D, inter, ptr(w1), ptr(b1), ptr(w2), ptr(b2), None, None,
-                                         dtype_code(w1.dtype), variant, ptr(hbuf), ptr(out), scatter,
-                                         stream_ptr()))
-
-    for it in range(steps + 1):
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(len(names) + 1)]
-        ev[0].record()
-        idx, wt, _, _ = ops.gate_topk(x, blk.gate.weight, k)
-        ev[1].record()
-        _, off, perm, _ = ops.dispatch(idx.view(-1), E)
-        ev[2].record()
-        stage(1, x, perm, k, off, E, n * k, blk.inter, p.w1, p.b1, p.w2, p.b2, h, slot_out, 1)
-        ev[3].record()
-        stage(2, x, perm, k, off, E, n * k, blk.inter, p.w1, p.b1, p.w2, p.b2, h, slot_out, 1)
-        ev[4].record()
-        stage(1, x, None, 1, soff, 1, n, si, p.sw1, p.sb1, p.sw2, p.sb2, sh, sout, 0)
-        ev[5].record()
-        stage(2, x, None, 1, soff, 1, n, si, p.sw1, p.sb1, p.sw2, p.sb2, sh, sout, 0)
-        ev[6].record()
-        ops.combine(slot_out, wt, n, k, shared_out=sout)
-        ev[7].record()
-        torch.cuda.synchronize()
-        if it == 0:
-            continue  # first pass warms allocator and caches
-        for i, s in enumerate(names):
-            acc[s] += ev[i].elapsed_time(ev[i + 1])
-    return {s: v / steps for s, v in acc.items()}
+    check(lib.dice_profile_enable(1))
+    n = lib.dice_profile_stage_count()
+    names = [lib.dice_profile_stage_name(i).decode() for i in range(n)]
+    buf = (ctypes.c_float * n)()
+    acc = [0.0] * n
+    y = torch.empty_like(x)
+    try:
+        for it in range(steps + 2):
+            blk.run(x, y=y)
+            check(lib.dice_profile_read(buf, n))
+            if it >= 2:
+                for i in range(n):
+                    acc[i] += buf[i]
+    finally:
+        check(lib.dice_profile_enable(0))
+    return {names[i]: acc[i] / steps for i in range(n)}
 
 
 def cpu_baseline(variant, budget_s=20.0):
@@ -140,15 +116,20 @@ def cpu_baseline(variant, budget_s=20.0):
     sample = int(min(N_TOKENS, max(256, (budget_s / 4) / max(per_tok, 1e-9))))
     sample = max(256, sample // 256 * 256)
     xs = torch.randn(1, sample, D, generator=g).bfloat16()
+    t0 = time.perf_counter()
+    O.sparse_moe_block_forward(p, xs)
+    first = time.perf_counter() - t0
+    reps = int(max(3, min(200, (budget_s / 2) / max(first, 1e-6))))
     times = []
-    for _ in range(3):
+    for _ in range(reps):
         t0 = time.perf_counter()
         O.sparse_moe_block_forward(p, xs)
         times.append(time.perf_counter() - t0)
     t = statistics.median(times)
     return {"value": sample / t, "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": f"{sample} of {N_TOKENS} tokens (tokens are independent), bf16 torch oracle, "
-                      f"median of 3 after 1 warm-up, {t:.2f} s each"}
+            "sample": f"{sample} of {N_TOKENS} tokens per call (tokens are independent), bf16 torch oracle of the "
+                      f"reference block, median of {reps} calls after 2 warm-ups, {t:.3f} s each, "
+                      f"{sum(times):.1f} s of CPU work"}
 
 
 def main():
@@ -204,20 +185,27 @@ def main():
         "layer_frac_of_bf16_peak": total_flops / sec / 1e12 / PEAK_BF16_TFLOPS,
     }
     if not args.no_stages:
-        st = time_stages(blk, x, max(5, min(args.steps, 20)))
-        dom = "fc1"
-        ach = flops[dom] / (st[dom] * 1e-3) / 1e12
-        out["roofline"] = {"bound": "mfma", "kernel": "grouped_gemm_bf16_kernel (routed fc1 + activation)",
+        st = time_stages(blk, x, max(5, min(args.steps, 30)))
+        # Dominant kernel: the persistent fc1 launch (routed experts + shared expert, activation fused).
+        dom_flops = flops["fc1"] + flops["shared_fc1"]
+        dom_ms = st["moe.mlp.fc1"]
+        ach = dom_flops / (dom_ms * 1e-3) / 1e12
+        out["roofline"] = {"bound": "mfma",
+                           "kernel": "gemm_persist_kernel<fc1> (routed + shared expert fc1, activation fused)",
                            "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                           "frac": ach / PEAK_BF16_TFLOPS, "traffic": None,
-                           "flop_per_launch": flops[dom], "ms_per_launch": st[dom]}
-        gemm_ms = st["fc1"] + st["fc2"] + st["shared_fc1"] + st["shared_fc2"]
+                           "frac": ach / PEAK_BF16_TFLOPS, "traffic": FC1_HBM_TRAFFIC_BYTES,
+                           "flop_per_launch": dom_flops, "ms_per_launch": dom_ms}
+        gemm_ms = st["moe.mlp.fc1"] + st["moe.mlp.fc2"]
         out["mfma_util_pct_of_peak"] = 100.0 * total_flops / (gemm_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS
         out["stage_ms"] = st
         bf = 2
-        hbm = {"gate": N_TOKENS * D * bf + N_TOKENS * TOPK * 8,
-               "combine": (N_TOKENS * TOPK * D + 2 * N_TOKENS * D) * bf + N_TOKENS * TOPK * 4}
+        slots = N_TOKENS * TOPK
+        hbm = {"moe.gate": N_TOKENS * D * bf + slots * 8,
+               "moe.dispatch": slots * 12,
+               "moe.gather": (N_TOKENS + slots) * D * bf,
+               "moe.combine": (slots * D + 2 * N_TOKENS * D) * bf + slots * 8}
         out["hbm_stage_gbs"] = {s: hbm[s] / (st[s] * 1e-3) / 1e9 for s in hbm}
+        out["hbm_stage_frac_of_peak"] = {s: v / PEAK_HBM_GBS for s, v in out["hbm_stage_gbs"].items()}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.variant)
     print(json.dumps(out))

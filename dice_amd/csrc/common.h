@@ -26,14 +26,15 @@ typedef u32x2_t __attribute__((may_alias)) u32x2_any_t;
 
 constexpr int kWave = 64;
 
-// Orders LDS traffic between the lanes of one wavefront: everything written
-// before is visible to every lane after.  (Lanes exchange data through LDS in
-// the GEMM epilogues; without this the compiler may run one side of a
-// divergent branch's reads ahead of the other side's writes.)
+// Orders LDS traffic between the lanes of one wavefront: LDS writes issued
+// before are complete and visible to every lane after.  (Lanes exchange data
+// through LDS in the GEMM epilogues; without a barrier here the compiler may
+// run one side of a divergent branch's reads ahead of the other side's
+// writes.)  Deliberately not a fence: a fence would also wait for every
+// outstanding global load and store.
 __device__ __forceinline__ void wave_lds_sync() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 // Records a printf-style message for dice_last_error() and returns `code`.

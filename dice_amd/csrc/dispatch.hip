@@ -91,6 +91,12 @@ __device__ __forceinline__ void rank_span(const int32_t *idx, const uint8_t *ski
   }
 }
 
+// Single-workgroup path.  Each wave first pulls its whole span into registers
+// (MAXR independent loads in flight: one memory latency instead of one per
+// round), then counts, then ranks out of those registers.
+// Slot codes: expert id >= 0 = live slot, -1 = dropped (skip mask / illegal id),
+// -2 = past the end.
+template <int MAXR>
 __global__ __launch_bounds__(kFusedWaves *kWave) void dispatch_fused_kernel(
     const int32_t *__restrict__ idx, const uint8_t *__restrict__ skip, int64_t n_slots,
     int n_experts, int nbits, int rounds, int32_t *__restrict__ counts,
@@ -102,9 +108,31 @@ __global__ __launch_bounds__(kFusedWaves *kWave) void dispatch_fused_kernel(
   const int64_t span = (int64_t)rounds * kWave;
   const int64_t begin = wave * span;
 
+  int code[MAXR];
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r) {
+    const int64_t slot = begin + (int64_t)r * kWave + lane;
+    code[r] = -2;
+    if (r < rounds && slot < n_slots) {
+      const int e = idx[slot];
+      const bool dropped = skip && skip[slot];
+      code[r] = (!dropped && e >= 0 && e < n_experts) ? e : -1;
+    }
+  }
+
   for (int e = lane; e < n_experts; e += kWave) wrow[wave][e] = 0;
   __syncthreads();
-  count_span(idx, skip, n_slots, n_experts, nbits, begin, rounds, wrow[wave], lane);
+  volatile int32_t *row = wrow[wave];
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r) {
+    if (r < rounds) {
+      const bool valid = code[r] >= 0;
+      const int e = valid ? code[r] : 0;
+      const uint64_t m = peers_of(e, valid, nbits);
+      if (valid && (__ffsll((unsigned long long)m) - 1) == lane) row[e] += __popcll(m);
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
   __syncthreads();
 
   // Exclusive scan of the per-expert totals by the first wave.
@@ -144,7 +172,25 @@ __global__ __launch_bounds__(kFusedWaves *kWave) void dispatch_fused_kernel(
     }
   }
   __syncthreads();
-  rank_span(idx, skip, n_slots, n_experts, nbits, begin, rounds, wrow[wave], lane, perm, inv_perm);
+  const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r) {
+    if (r < rounds) {
+      const bool valid = code[r] >= 0;
+      const int e = valid ? code[r] : 0;
+      const int64_t slot = begin + (int64_t)r * kWave + lane;
+      const uint64_t m = peers_of(e, valid, nbits);
+      int pos = -1;
+      if (valid) pos = row[e] + __popcll(m & below);
+      __builtin_amdgcn_wave_barrier();
+      if (valid) {
+        perm[pos] = (int32_t)slot;
+        if ((__ffsll((unsigned long long)m) - 1) == lane) row[e] += __popcll(m);
+      }
+      if (code[r] != -2) inv_perm[slot] = pos;
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
   const int total = eoff[n_experts];
   for (int64_t i = total + threadIdx.x; i < n_slots; i += blockDim.x) perm[i] = -1;
 }
@@ -227,12 +273,20 @@ __global__ __launch_bounds__(kTileWaves *kWave) void dispatch_rank_kernel(
   }
 }
 
+// `range_out` (optional) receives {0, range_n}: the one-group offset table of
+// the shared expert, written here so the layer needs no extra launch for it.
 template <typename V>
 __global__ __launch_bounds__(256) void gather_rows_kernel(const V *__restrict__ x,
                                                           const int32_t *__restrict__ perm,
                                                           int slots_per_token, int64_t n_rows,
-                                                          int vec_per_row, V *__restrict__ out) {
+                                                          int vec_per_row, V *__restrict__ out,
+                                                          int32_t *__restrict__ range_out,
+                                                          int32_t range_n) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (range_out && i == 0) {
+    range_out[0] = 0;
+    range_out[1] = range_n;
+  }
   if (i >= n_rows * vec_per_row) return;
   const int64_t r = i / vec_per_row;
   const int c = (int)(i - r * vec_per_row);
@@ -272,8 +326,15 @@ extern "C" int dice_dispatch(const int32_t *flat_idx, const uint8_t *skip_mask, 
   const int nbits = bits_for(n_experts);
   if (n_slots <= kFusedMaxSlots) {
     int rounds = (int)((n_slots + kFusedWaves * kWave - 1) / (kFusedWaves * kWave));
-    hipLaunchKernelGGL(dispatch_fused_kernel, dim3(1), dim3(kFusedWaves * kWave), 0, s, flat_idx,
-                       skip_mask, n_slots, n_experts, nbits, rounds, counts, offsets, perm, inv_perm);
+    if (rounds <= 16)
+      hipLaunchKernelGGL(dispatch_fused_kernel<16>, dim3(1), dim3(kFusedWaves * kWave), 0, s, flat_idx,
+                         skip_mask, n_slots, n_experts, nbits, rounds, counts, offsets, perm, inv_perm);
+    else if (rounds <= 32)
+      hipLaunchKernelGGL(dispatch_fused_kernel<32>, dim3(1), dim3(kFusedWaves * kWave), 0, s, flat_idx,
+                         skip_mask, n_slots, n_experts, nbits, rounds, counts, offsets, perm, inv_perm);
+    else
+      hipLaunchKernelGGL(dispatch_fused_kernel<64>, dim3(1), dim3(kFusedWaves * kWave), 0, s, flat_idx,
+                         skip_mask, n_slots, n_experts, nbits, rounds, counts, offsets, perm, inv_perm);
     return launch_status("dice_dispatch");
   }
   const int64_t units64 = (n_slots + kTileRounds * kWave - 1) / (kTileRounds * kWave);
@@ -292,9 +353,10 @@ extern "C" int dice_dispatch(const int32_t *flat_idx, const uint8_t *skip_mask, 
   return launch_status("dice_dispatch");
 }
 
-extern "C" int dice_gather_rows(const void *x, int dtype, const int32_t *perm, int slots_per_token,
-                                int64_t n_rows, int hidden, void *out, void *stream) {
-  using namespace dice;
+namespace dice {
+int gather_rows_impl(const void *x, int dtype, const int32_t *perm, int slots_per_token,
+                     int64_t n_rows, int hidden, void *out, int32_t *range_out, int32_t range_n,
+                     void *stream) {
   DICE_REQUIRE(x && perm && out, DICE_ERR_BAD_ARG, "dice_gather_rows: null pointer");
   DICE_REQUIRE(slots_per_token >= 1, DICE_ERR_BAD_ARG, "dice_gather_rows: slots_per_token %d < 1",
                slots_per_token);
@@ -309,6 +371,12 @@ extern "C" int dice_gather_rows(const void *x, int dtype, const int32_t *perm, i
   const int64_t blocks = (total + 255) / 256;
   hipLaunchKernelGGL(gather_rows_kernel<u32x4_t>, dim3((unsigned)blocks), dim3(256), 0,
                      (hipStream_t)stream, (const u32x4_t *)x, perm, slots_per_token, n_rows,
-                     vec_per_row, (u32x4_t *)out);
+                     vec_per_row, (u32x4_t *)out, range_out, range_n);
   return launch_status("dice_gather_rows");
+}
+}  // namespace dice
+
+extern "C" int dice_gather_rows(const void *x, int dtype, const int32_t *perm, int slots_per_token,
+                                int64_t n_rows, int hidden, void *out, void *stream) {
+  return dice::gather_rows_impl(x, dtype, perm, slots_per_token, n_rows, hidden, out, nullptr, 0, stream);
 }

@@ -3,7 +3,7 @@
 // Replaces MoEGate.forward, inference branch (reference models.py:179-196).
 // HBM-bound: the only large operand is x, read exactly once (n_tokens*hidden
 // elements); the router matrix is staged once per workgroup in LDS.  Each wave
-// keeps TOK tokens in flight so one LDS read of a router chunk feeds TOK
+// keeps 64/E tokens in flight so one LDS read of a router chunk feeds that many
 // dot-product updates.
 #include "common.h"
 
@@ -32,14 +32,58 @@ __device__ __forceinline__ Vec8<T> load8(const T *p) {
 
 constexpr int kGateWaves = 4;
 
-// EP = experts padded to a compile-time bound so accumulators stay in
-// registers; TOK = tokens per wave per pass.
-template <typename XT, typename WT, int EP, int TOK, bool W_IN_LDS>
+// 8-element dot product accumulate.  bf16 x bf16 uses the packed
+// v_dot2_f32_bf16 (exact products, fp32 accumulation); everything else widens
+// to fp32 FMAs.
+template <typename XT, typename WT>
+__device__ __forceinline__ float dot8(const Vec8<XT> &x, const Vec8<WT> &w, float acc) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc = fmaf(x.get(i), w.get(i), acc);
+  return acc;
+}
+template <>
+__device__ __forceinline__ float dot8<bf16_t, bf16_t>(const Vec8<bf16_t> &x, const Vec8<bf16_t> &w,
+                                                      float acc) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const bf16x2_t a = {x.v[2 * i], x.v[2 * i + 1]};
+    const bf16x2_t b = {w.v[2 * i], w.v[2 * i + 1]};
+    acc = __builtin_amdgcn_fdot2_f32_bf16(a, b, acc, false);
+  }
+  return acc;
+}
+
+// Sums v[0..63] across the 64 lanes; lane l returns the total of v[l].  Each
+// step halves the values a lane keeps (the partner takes the other half), so
+// the whole reduction costs 63 lane exchanges instead of 64 x 6, and the
+// summation order is fixed.
+__device__ __forceinline__ float reduce_transpose64(float (&v)[64], int lane) {
+#pragma unroll
+  for (int step = 0; step < 6; ++step) {
+    const int mask = 32 >> step;   // partner distance
+    const int half = 32 >> step;   // values kept after this step
+    const bool upper = lane & mask;
+#pragma unroll
+    for (int i = 0; i < half; ++i) {
+      const float keep = upper ? v[i + half] : v[i];
+      const float send = upper ? v[i] : v[i + half];
+      v[i] = keep + __shfl_xor(send, mask, kWave);
+    }
+  }
+  return v[0];
+}
+
+// One wavefront routes TOK = 64 / EP tokens at a time: lanes split the hidden
+// dimension, every lane accumulates all TOK x EP dot products, the transposing
+// reduction leaves lane t*EP + e with logit (t, e), and softmax / top-k then
+// run inside each group of EP lanes for all TOK tokens at once.
+template <typename XT, typename WT, int EP, bool W_IN_LDS>
 __global__ __launch_bounds__(kGateWaves *kWave) void gate_topk_kernel(
     const XT *__restrict__ x, const WT *__restrict__ w, const float *__restrict__ bias,
     int64_t n_tokens, int hidden, int n_experts, int top_k, int norm_topk,
     int32_t *__restrict__ topk_idx, int64_t *__restrict__ topk_idx64,
     float *__restrict__ topk_weight, float *__restrict__ logits_out) {
+  constexpr int TOK = kWave / EP;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
@@ -55,23 +99,21 @@ __global__ __launch_bounds__(kGateWaves *kWave) void gate_topk_kernel(
     wsrc = wl;
   }
 
+  const int my_tok = lane / EP, my_e = lane % EP;
+  const bool live = my_e < n_experts;
   const int64_t groups = (n_tokens + TOK - 1) / TOK;
   for (int64_t g = (int64_t)blockIdx.x * kGateWaves + wave; g < groups;
        g += (int64_t)gridDim.x * kGateWaves) {
     const int64_t t0 = g * TOK;
-    float acc[TOK][EP];
+    float acc[64];
 #pragma unroll
-    for (int t = 0; t < TOK; ++t)
-#pragma unroll
-      for (int e = 0; e < EP; ++e) acc[t][e] = 0.f;
-
+    for (int i = 0; i < 64; ++i) acc[i] = 0.f;
     const XT *xrow[TOK];
 #pragma unroll
     for (int t = 0; t < TOK; ++t) {
-      int64_t tt = t0 + t < n_tokens ? t0 + t : n_tokens - 1;
+      const int64_t tt = t0 + t < n_tokens ? t0 + t : n_tokens - 1;
       xrow[t] = x + tt * hidden;
     }
-
     for (int c = lane; c < chunks; c += kWave) {
       Vec8<XT> xv[TOK];
 #pragma unroll
@@ -79,81 +121,72 @@ __global__ __launch_bounds__(kGateWaves *kWave) void gate_topk_kernel(
 #pragma unroll
       for (int e = 0; e < EP; ++e) {
         if (e < n_experts) {
-          Vec8<WT> wv = load8(wsrc + ((size_t)e * chunks + c) * 8);
+          const Vec8<WT> wv = load8(wsrc + ((size_t)e * chunks + c) * 8);
 #pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            const float wf = wv.get(i);
-#pragma unroll
-            for (int t = 0; t < TOK; ++t) acc[t][e] = fmaf(xv[t].get(i), wf, acc[t][e]);
-          }
+          for (int t = 0; t < TOK; ++t) acc[t * EP + e] = dot8<XT, WT>(xv[t], wv, acc[t * EP + e]);
         }
       }
     }
+    float logit = reduce_transpose64(acc, lane);
+    if (live && bias) logit += bias[my_e];
+    if (!live) logit = -INFINITY;
+    const int64_t tok = t0 + my_tok;
+    const bool tok_ok = tok < n_tokens;
+    if (logits_out && live && tok_ok) logits_out[tok * n_experts + my_e] = logit;
 
+    // softmax inside the EP-lane group
+    float m = logit;
 #pragma unroll
-    for (int t = 0; t < TOK; ++t) {
-      // Lane e ends up owning expert e's logit.
-      float logit = -INFINITY;
+    for (int o = EP / 2; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, kWave));
+    const float p = live ? expf(logit - m) : 0.f;
+    float denom = p;
 #pragma unroll
-      for (int e = 0; e < EP; ++e) {
-        float s = wave_sum(acc[t][e]);
-        if (lane == e) logit = s;
-      }
-      const bool live = lane < n_experts;
-      if (live && bias) logit += bias[lane];
-      if (!live) logit = -INFINITY;
-      const int64_t tok = t0 + t;
-      if (tok >= n_tokens) continue;  // uniform across the wave
-      if (logits_out && live) logits_out[tok * n_experts + lane] = logit;
+    for (int o = EP / 2; o > 0; o >>= 1) denom += __shfl_xor(denom, o, kWave);
+    float score = live ? p / denom : -1.f;
 
-      const float m = wave_max(logit);
-      const float p = live ? expf(logit - m) : 0.f;
-      const float denom = wave_sum(p);
-      float score = live ? p / denom : -1.f;
-
-      float sel_w = 0.f;  // lane j < top_k keeps the j-th pick
-      int sel_i = 0;
-      float picked_sum = 0.f;
-      for (int j = 0; j < top_k; ++j) {
-        float bv = score;
-        int bi = lane;
+    float sel_w = 0.f;  // lane j of the group keeps the j-th pick
+    int sel_i = 0;
+    float picked_sum = 0.f;
+    for (int j = 0; j < top_k; ++j) {
+      float bv = score;
+      int bi = my_e;
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-          float ov = __shfl_xor(bv, o, kWave);
-          int oi = __shfl_xor(bi, o, kWave);
-          if (ov > bv || (ov == bv && oi < bi)) {
-            bv = ov;
-            bi = oi;
-          }
+      for (int o = EP / 2; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, kWave);
+        const int oi = __shfl_xor(bi, o, kWave);
+        if (ov > bv || (ov == bv && oi < bi)) {
+          bv = ov;
+          bi = oi;
         }
-        if (lane == j) {
-          sel_w = bv;
-          sel_i = bi;
-        }
-        picked_sum += bv;
-        if (lane == bi) score = -1.f;
       }
-      if (norm_topk && top_k > 1) sel_w = sel_w / (picked_sum + 1e-20f);
-      if (lane < top_k) {
-        topk_idx[tok * top_k + lane] = sel_i;
-        if (topk_idx64) topk_idx64[tok * top_k + lane] = sel_i;
-        topk_weight[tok * top_k + lane] = sel_w;
+      if (my_e == j) {
+        sel_w = bv;
+        sel_i = bi;
       }
+      picked_sum += bv;
+      if (my_e == bi) score = -1.f;
+    }
+    if (norm_topk && top_k > 1) sel_w = sel_w / (picked_sum + 1e-20f);
+    if (tok_ok && my_e < top_k) {
+      topk_idx[tok * top_k + my_e] = sel_i;
+      if (topk_idx64) topk_idx64[tok * top_k + my_e] = sel_i;
+      topk_weight[tok * top_k + my_e] = sel_w;
     }
   }
 }
 
-template <typename XT, typename WT, int EP, int TOK>
+template <typename XT, typename WT, int EP>
 int launch_gate(const void *x, const void *w, const float *bias, int64_t n_tokens, int hidden,
                 int n_experts, int top_k, int norm, int32_t *idx, int64_t *idx64, float *wt,
                 float *logits, hipStream_t stream) {
+  constexpr int TOK = kWave / EP;
   const size_t w_bytes = (size_t)n_experts * hidden * sizeof(WT);
   const int64_t groups = (n_tokens + TOK - 1) / TOK;
   int64_t blocks = (groups + kGateWaves - 1) / kGateWaves;
   if (blocks > 512) blocks = 512;
   if (blocks < 1) blocks = 1;
   if (w_bytes <= 160 * 1024 - 1024) {
-    auto kern = gate_topk_kernel<XT, WT, EP, TOK, true>;
+    auto kern = gate_topk_kernel<XT, WT, EP, true>;
     if (w_bytes > 48 * 1024) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)w_bytes);
@@ -163,7 +196,7 @@ int launch_gate(const void *x, const void *w, const float *bias, int64_t n_token
                        (const XT *)x, (const WT *)w, bias, n_tokens, hidden, n_experts, top_k, norm,
                        idx, idx64, wt, logits);
   } else {
-    auto kern = gate_topk_kernel<XT, WT, EP, TOK, false>;
+    auto kern = gate_topk_kernel<XT, WT, EP, false>;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kGateWaves * kWave), 0, stream,
                        (const XT *)x, (const WT *)w, bias, n_tokens, hidden, n_experts, top_k, norm,
                        idx, idx64, wt, logits);
@@ -176,12 +209,12 @@ int dispatch_experts(const void *x, const void *w, const float *bias, int64_t n_
                      int n_experts, int top_k, int norm, int32_t *idx, int64_t *idx64, float *wt,
                      float *logits, hipStream_t s) {
   if (n_experts <= 8)
-    return launch_gate<XT, WT, 8, 4>(x, w, bias, n_tokens, hidden, n_experts, top_k, norm, idx, idx64, wt, logits, s);
+    return launch_gate<XT, WT, 8>(x, w, bias, n_tokens, hidden, n_experts, top_k, norm, idx, idx64, wt, logits, s);
   if (n_experts <= 16)
-    return launch_gate<XT, WT, 16, 4>(x, w, bias, n_tokens, hidden, n_experts, top_k, norm, idx, idx64, wt, logits, s);
+    return launch_gate<XT, WT, 16>(x, w, bias, n_tokens, hidden, n_experts, top_k, norm, idx, idx64, wt, logits, s);
   if (n_experts <= 32)
-    return launch_gate<XT, WT, 32, 2>(x, w, bias, n_tokens, hidden, n_experts, top_k, norm, idx, idx64, wt, logits, s);
-  return launch_gate<XT, WT, 64, 1>(x, w, bias, n_tokens, hidden, n_experts, top_k, norm, idx, idx64, wt, logits, s);
+    return launch_gate<XT, WT, 32>(x, w, bias, n_tokens, hidden, n_experts, top_k, norm, idx, idx64, wt, logits, s);
+  return launch_gate<XT, WT, 64>(x, w, bias, n_tokens, hidden, n_experts, top_k, norm, idx, idx64, wt, logits, s);
 }
 
 // The router matrix is either fp32 or stored in the activation dtype.

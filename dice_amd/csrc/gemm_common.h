@@ -142,6 +142,10 @@ bool persist_supported(const PersistBatch &b, int mode);
 bool gemm_config_wants_persistent();  // tuning hook state: both stages set to the persistent kernel
 int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s);
 
+int gather_rows_impl(const void *x, int dtype, const int32_t *perm, int slots_per_token,
+                     int64_t n_rows, int hidden, void *out, int32_t *range_out, int32_t range_n,
+                     void *stream);
+
 int launch_grouped_gemm_f32(const GemmParams &p, int mode, int64_t max_rows, hipStream_t s);
 int launch_grouped_gemm_bf16(const GemmParams &p, int mode, int w_dtype, int64_t max_rows,
                              hipStream_t s);

@@ -49,6 +49,13 @@ __device__ __forceinline__ int pring_off(int row, int chunk) {
   return row * 64 + ((chunk ^ pswizzle(row)) << 4);
 }
 
+// Workgroup barrier that instructions may not be scheduled across.
+__device__ __forceinline__ void phase_barrier() {
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+}
+
 template <int N> __device__ __forceinline__ void pwait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
@@ -113,7 +120,10 @@ struct Tile {
   bool valid;
 };
 
-template <int MODE>
+// HAS_BIAS is a compile-time switch so that the bias-free (reference SwiGLU)
+// instantiations carry no bias loads: a vector load in the epilogue makes the
+// compiler wait for every outstanding copy and store.
+template <int MODE, bool HAS_BIAS>
 __global__ __launch_bounds__(kPWaves *kWave, 1) void gemm_persist_kernel(PersistBatch batch) {
   constexpr bool SWIGLU = MODE == kFc1Swiglu;
   constexpr int BN_OUT = SWIGLU ? kPBN / 2 : kPBN;
@@ -129,7 +139,7 @@ __global__ __launch_bounds__(kPWaves *kWave, 1) void gemm_persist_kernel(Persist
   constexpr int PASSES = BAND / ROWS_PER_PASS;
   static_assert(PASSES >= 1, "band smaller than one store pass");
   constexpr int STORES = (WTM / BAND) * PASSES;  // buffer stores per wave per tile
-  constexpr int WAIT_STEADY = (kPStages - 3) * kPCopies;
+  constexpr int WAIT_STEADY = (kPAhead - 1) * kPCopies;  // copies of the two newest steps
   constexpr int WAIT_AFTER_EPILOGUE = WAIT_STEADY + STORES;
   static_assert(WAIT_AFTER_EPILOGUE < 64, "vmcnt is a 6-bit counter");
 
@@ -296,7 +306,7 @@ __global__ __launch_bounds__(kPWaves *kWave, 1) void gemm_persist_kernel(Persist
   next_id += wgs_per_xcd;
   if (!ld.valid) return;                         // nothing to do for this workgroup
   Tile cp = ld;                                  // tile being multiplied
-  int ld_kt = 0, cp_kt = 0;
+  int ld_kt = 0;
   int cslot = 0;                                 // ring slot of the step being multiplied
 
   // Advances the copy side by one step (wave-uniform control flow only).
@@ -316,46 +326,65 @@ __global__ __launch_bounds__(kPWaves *kWave, 1) void gemm_persist_kernel(Persist
   }
   zero_acc();
   pwait_vmcnt<WAIT_STEADY>();
-  __builtin_amdgcn_s_barrier();
-  read_frags(0, 0, 0);
+  phase_barrier();                      // everyone's copies of steps 0 and 1 have landed
   int since_epilogue = 2;
 
   const int stage_base = kPRingBytes + wave * (BAND * PITCH);
   const int rd_row = lane / LANES_PER_ROW, rd_chunk = lane % LANES_PER_ROW;
   const int wave_col0 = SWIGLU ? wn * (WTN / 2) : wn * WTN;
 
-  while (true) {
-    const int lslot = (cslot + kPAhead) & (kPStages - 1);  // = slot read during the previous step
-    const int nslot = (cslot + 1) & (kPStages - 1);
-    // This wave's copies for the current and the next step have landed ...
+  // Two groups of four waves (one wave of each group per SIMD) alternate between
+  // a memory phase (fragment reads of one k step + this wave's share of the
+  // copies three steps ahead) and a compute phase (the step's 16 MFMAs), one
+  // phase apart: while one group multiplies the other one loads, so the matrix
+  // pipe only idles for the barrier hand-over between phases.
+  const int group = wm;
+  // Waits until at most the copies of the two newest steps (plus the stores of an
+  // epilogue that was issued in between) are still in flight.
+  auto copies_landed = [&]() {
     if (since_epilogue < 2) pwait_vmcnt<WAIT_AFTER_EPILOGUE>();
     else pwait_vmcnt<WAIT_STEADY>();
     ++since_epilogue;
-    // ... everyone's have, and nobody still reads the slot about to be refilled.
-    __builtin_amdgcn_s_barrier();
-
-    read_frags(cslot, 1, 1);
+  };
+  while (true) {  // one tile per iteration
+    if (group == 1) phase_barrier();
+    for (int s = 0; s < cp.steps; ++s) {
+      // ---- memory phase ----
+      const int lslot = (cslot + kPAhead) & (kPStages - 1);  // slot of the step before this one
+      read_frags(cslot, 0, 0);
+      read_frags(cslot, 1, 1);
 #pragma unroll
-    for (int l = 0; l < kPCopies / 2; ++l) issue_copy(ld, ld_kt, lslot, l);
+      for (int l = 0; l < kPCopies; ++l) issue_copy(ld, ld_kt, lslot, l);
+      advance_copy();
+      // The first reader of step s+1 is the first group, right after the barrier
+      // that ends this phase pair.  Each wave therefore confirms that its own
+      // copies of step s+1 have landed at the last barrier before that point:
+      // the second group at the end of its memory phase, the first group at the
+      // end of its compute phase.  Copies get four to five phases to land.
+      if (group == 1) copies_landed();
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // slot fully read before anyone may refill it
+      phase_barrier();
+      // ---- compute phase ----
+#ifndef DICE_PRIO_COMPUTE
+#define DICE_PRIO_COMPUTE 0
+#endif
+#ifndef DICE_PRIO_MEMORY
+#define DICE_PRIO_MEMORY 0
+#endif
+      __builtin_amdgcn_s_setprio(DICE_PRIO_COMPUTE);
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+      for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[0][j], af[0][i], acc[i][j], 0, 0, 0);
-    read_frags(nslot, 0, 0);
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int l = kPCopies / 2; l < kPCopies; ++l) issue_copy(ld, ld_kt, lslot, l);
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[1][j], af[1][i], acc[i][j], 0, 0, 0);
-    psched_half<TM * TN, TM + TN, kPCopies / 2>();
-    psched_half<TM * TN, TM + TN, kPCopies - kPCopies / 2>();
-
-    advance_copy();
-    cslot = nslot;
-    if (++cp_kt < cp.steps) continue;
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[kk][j], af[kk][i], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_s_setprio(DICE_PRIO_MEMORY);
+      if (group == 0) copies_landed();
+      phase_barrier();
+      cslot = (cslot + 1) & (kPStages - 1);
+    }
+    if (group == 0) phase_barrier();  // let the other group finish the tile's last step
 
     // ---- epilogue of tile `cp` ----
     {
@@ -363,6 +392,23 @@ __global__ __launch_bounds__(kPWaves *kWave, 1) void gemm_persist_kernel(Persist
           __builtin_amdgcn_make_buffer_rsrc((void *)cp.c, 0, cp.c_bytes, kRsrcFlags);
       unsigned char *stage = lds_raw + stage_base;
       const int col_base = cp.n0 + wave_col0;
+      // Bias of this lane's columns, fetched in one batch (one wait instead of one per element).
+      float bias_v[OUT_BLOCKS][16];
+      if (HAS_BIAS) {
+#pragma unroll
+        for (int j = 0; j < OUT_BLOCKS; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) bias_v[j][e] = 0.f;
+        if (cp.bias) {
+#pragma unroll
+          for (int j = 0; j < OUT_BLOCKS; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+              const int cn = col_base + j * 32 + frag_half * 4 + (e >> 2) * 8 + (e & 3);
+              bias_v[j][e] = cp.bias[cn < cp.n ? cn : 0];
+            }
+        }
+      }
 #pragma unroll
       for (int band = 0; band < WTM / BAND; ++band) {
         const int i = band * BAND / 32;             // 32-row block the band lies in
@@ -381,10 +427,7 @@ __global__ __launch_bounds__(kPWaves *kWave, 1) void gemm_persist_kernel(Persist
                 if (SWIGLU) {
                   v = silu_fast(v) * acc[i][j + OUT_BLOCKS][q * 4 + r];
                 } else {
-                  if (cp.bias) {
-                    const int cn = col_base + col + r;
-                    v += cp.bias[cn < cp.n ? cn : 0];
-                  }
+                  if (HAS_BIAS) v += bias_v[j][q * 4 + r];
                   if (MODE == kFc1Gelu) v = gelu_tanh_fast(v);
                 }
                 o[r] = (bf16_t)v;
@@ -410,7 +453,6 @@ __global__ __launch_bounds__(kPWaves *kWave, 1) void gemm_persist_kernel(Persist
     // tile ahead here: the tile it is working on is the one to multiply next.
     cp = ld;
     if (!cp.valid) break;
-    cp_kt = 0;
     since_epilogue = 0;
     zero_acc();
   }
@@ -443,29 +485,25 @@ int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s) 
       return fail(DICE_ERR_LAUNCH, "persistent expert GEMM: cannot query the CU count");
     grid = cus / kNumXcd * kNumXcd;
   }
-  const void *kern = nullptr;
+  bool has_bias = false;
+  for (int i = 0; i < b.n_problems; ++i) has_bias = has_bias || b.prob[i].bias != nullptr;
+  if (mode == kFc1Swiglu) has_bias = false;
+  void (*kern)(PersistBatch) = nullptr;
   switch (mode) {
-    case kFc1Swiglu: kern = reinterpret_cast<const void *>(gemm_persist_kernel<kFc1Swiglu>); break;
-    case kFc1Gelu: kern = reinterpret_cast<const void *>(gemm_persist_kernel<kFc1Gelu>); break;
-    default: kern = reinterpret_cast<const void *>(gemm_persist_kernel<kFc2>); break;
+    case kFc1Swiglu: kern = gemm_persist_kernel<kFc1Swiglu, false>; break;
+    case kFc1Gelu: kern = has_bias ? gemm_persist_kernel<kFc1Gelu, true> : gemm_persist_kernel<kFc1Gelu, false>; break;
+    default: kern = has_bias ? gemm_persist_kernel<kFc2, true> : gemm_persist_kernel<kFc2, false>; break;
   }
-  static thread_local bool configured[3] = {false, false, false};
-  if (!configured[mode]) {
-    hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, kPLdsBytes);
+  const int slot = mode * 2 + (has_bias ? 1 : 0);
+  static thread_local bool configured[6] = {false, false, false, false, false, false};
+  if (!configured[slot]) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kPLdsBytes);
     if (e != hipSuccess)
       return fail(DICE_ERR_LAUNCH, "persistent expert GEMM: LDS attribute: %s", hipGetErrorString(e));
-    configured[mode] = true;
+    configured[slot] = true;
   }
-  switch (mode) {
-    case kFc1Swiglu:
-      hipLaunchKernelGGL(gemm_persist_kernel<kFc1Swiglu>, dim3(grid), dim3(kPWaves * kWave), kPLdsBytes, s, b);
-      break;
-    case kFc1Gelu:
-      hipLaunchKernelGGL(gemm_persist_kernel<kFc1Gelu>, dim3(grid), dim3(kPWaves * kWave), kPLdsBytes, s, b);
-      break;
-    default:
-      hipLaunchKernelGGL(gemm_persist_kernel<kFc2>, dim3(grid), dim3(kPWaves * kWave), kPLdsBytes, s, b);
-  }
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kPWaves * kWave), kPLdsBytes, s, b);
   return launch_status("grouped_gemm_persist");
 }
 

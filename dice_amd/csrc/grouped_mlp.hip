@@ -65,6 +65,29 @@ __global__ void set_range_kernel(int32_t *offsets, int32_t n) {
   }
 }
 
+// Stage timers of dice_moe_forward: HIP events recorded on the caller's stream
+// between the launches, the counterpart of the reference's CudaProfiler scopes
+// "moe.gate" / "moe.mlp" / "moe.mlp_shared" (models.py:305,356,375;
+// cudaprof/prof.py:19-60).  Off by default; events are host objects created on
+// first use.
+constexpr int kStages = 6;
+const char *const kStageNames[kStages] = {"moe.gate", "moe.dispatch", "moe.gather", "moe.mlp.fc1",
+                                          "moe.mlp.fc2", "moe.combine"};
+struct StageTimers {
+  bool enabled = false;
+  bool have_events = false;
+  bool recorded = false;
+  hipEvent_t ev[kStages + 1];
+};
+StageTimers g_timers;
+
+void stamp(int i, hipStream_t s) {
+  if (g_timers.enabled && g_timers.have_events) {
+    (void)hipEventRecord(g_timers.ev[i], s);
+    if (i == kStages) g_timers.recorded = true;
+  }
+}
+
 int check_mlp_shape(const char *who, int act_dtype, int w_dtype, int act_variant, int hidden,
                     int inter, int n_experts) {
   DICE_REQUIRE(act_dtype == DICE_BF16 || act_dtype == DICE_F32, DICE_ERR_UNSUPPORTED,
@@ -243,12 +266,16 @@ extern "C" int dice_moe_forward(const dice_moe_layer_t *L, const void *x, int64_
   int32_t *idx = topk_idx_out ? topk_idx_out : w.topk_idx;
   float *wt = topk_weight_out ? topk_weight_out : w.topk_weight;
 
+  g_timers.recorded = false;
+  stamp(0, s);
   rc = dice_gate_topk(x, L->act_dtype, L->gate_w, L->gate_w_dtype, L->gate_bias, n_tokens, L->hidden,
                       L->n_experts, L->top_k, L->norm_topk_prob, idx, nullptr, wt, nullptr, stream);
   if (rc) return rc;
+  stamp(1, s);
   rc = dice_dispatch(idx, mode == 2 ? skip_mask : nullptr, slots, L->n_experts, w.counts, w.offsets,
                      w.perm, w.inv_perm, w.dispatch_ws, w.dispatch_ws_bytes, stream);
   if (rc) return rc;
+  stamp(2, s);
   // A skip step recomputes one slot per token.
   const int64_t max_rows = mode == 2 ? n_tokens * (L->top_k - 1) : slots;
   const uint8_t *mask = mode == 0 ? nullptr : skip_mask;
@@ -275,17 +302,21 @@ extern "C" int dice_moe_forward(const dice_moe_layer_t *L, const void *x, int64_
       f1.n_problems = f2.n_problems = 2;
     }
     if (persist_supported(f1, m1) && persist_supported(f2, kFc2)) {
-      rc = dice_gather_rows(x, L->act_dtype, w.perm, L->top_k, max_rows, L->hidden, xg, stream);
+      rc = gather_rows_impl(x, L->act_dtype, w.perm, L->top_k, max_rows, L->hidden, xg,
+                            L->shared_inter > 0 ? w.shared_offsets : nullptr, (int32_t)n_tokens, stream);
       if (rc) return rc;
-      if (L->shared_inter > 0)
-        hipLaunchKernelGGL(set_range_kernel, dim3(1), dim3(64), 0, s, w.shared_offsets, (int32_t)n_tokens);
+      stamp(3, s);
       rc = launch_grouped_gemm_persist(f1, m1, s);
       if (rc) return rc;
+      stamp(4, s);
       rc = launch_grouped_gemm_persist(f2, kFc2, s);
       if (rc) return rc;
-      return dice_combine(w.slot_out, w.inv_perm, wt, w.shared_out, mask, mode == 2 ? cache_in : nullptr,
-                          mode == 1 ? cache_out : nullptr, y, L->act_dtype, n_tokens, L->top_k, L->hidden,
-                          stream);
+      stamp(5, s);
+      rc = dice_combine(w.slot_out, w.inv_perm, wt, w.shared_out, mask, mode == 2 ? cache_in : nullptr,
+                        mode == 1 ? cache_out : nullptr, y, L->act_dtype, n_tokens, L->top_k, L->hidden,
+                        stream);
+      stamp(6, s);
+      return rc;
     }
   }
 
@@ -304,4 +335,38 @@ extern "C" int dice_moe_forward(const dice_moe_layer_t *L, const void *x, int64_
   return dice_combine(w.slot_out, nullptr, wt, w.shared_out, mode == 0 ? nullptr : skip_mask,
                       mode == 2 ? cache_in : nullptr, mode == 1 ? cache_out : nullptr, y,
                       L->act_dtype, n_tokens, L->top_k, L->hidden, stream);
+}
+
+extern "C" int dice_profile_enable(int on) {
+  using namespace dice;
+  if (on && !g_timers.have_events) {
+    for (int i = 0; i <= kStages; ++i) {
+      hipError_t e = hipEventCreate(&g_timers.ev[i]);
+      if (e != hipSuccess) return fail(DICE_ERR_LAUNCH, "dice_profile_enable: %s", hipGetErrorString(e));
+    }
+    g_timers.have_events = true;
+  }
+  g_timers.enabled = on != 0;
+  g_timers.recorded = false;
+  return DICE_OK;
+}
+
+extern "C" int dice_profile_stage_count(void) { return dice::kStages; }
+
+extern "C" const char *dice_profile_stage_name(int i) {
+  return i >= 0 && i < dice::kStages ? dice::kStageNames[i] : "";
+}
+
+extern "C" int dice_profile_read(float *ms_out, int n) {
+  using namespace dice;
+  DICE_REQUIRE(ms_out && n >= kStages, DICE_ERR_BAD_ARG, "dice_profile_read: need room for %d stages", kStages);
+  DICE_REQUIRE(g_timers.enabled && g_timers.recorded, DICE_ERR_BAD_ARG,
+               "dice_profile_read: no timed dice_moe_forward call (bf16 path) since dice_profile_enable");
+  hipError_t e = hipEventSynchronize(g_timers.ev[kStages]);
+  if (e != hipSuccess) return fail(DICE_ERR_LAUNCH, "dice_profile_read: %s", hipGetErrorString(e));
+  for (int i = 0; i < kStages; ++i) {
+    e = hipEventElapsedTime(&ms_out[i], g_timers.ev[i], g_timers.ev[i + 1]);
+    if (e != hipSuccess) return fail(DICE_ERR_LAUNCH, "dice_profile_read: %s", hipGetErrorString(e));
+  }
+  return DICE_OK;
 }

@@ -36,6 +36,10 @@ EXPORTS = [
     "dice_grouped_mlp",
     "dice_grouped_mlp_stage",
     "dice_set_gemm_config",
+    "dice_profile_enable",
+    "dice_profile_stage_count",
+    "dice_profile_stage_name",
+    "dice_profile_read",
     "dice_combine",
     "dice_quantize_fp8_rowwise",
     "dice_moe_workspace_bytes",
@@ -103,6 +107,13 @@ def load() -> ctypes.CDLL:
     lib.dice_moe_forward.restype = c_int
     lib.dice_moe_forward.argtypes = [POINTER(MoeLayerDesc), c_void_p, c_int64, c_int, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]
+    lib.dice_profile_enable.restype = c_int
+    lib.dice_profile_enable.argtypes = [c_int]
+    lib.dice_profile_stage_count.restype = c_int
+    lib.dice_profile_stage_name.restype = c_char_p
+    lib.dice_profile_stage_name.argtypes = [c_int]
+    lib.dice_profile_read.restype = c_int
+    lib.dice_profile_read.argtypes = [POINTER(c_float), c_int]
     lib.dice_set_gemm_config.restype = c_int
     lib.dice_set_gemm_config.argtypes = [c_int, c_int]
     if lib.dice_abi_version() != 1:

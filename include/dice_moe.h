@@ -213,6 +213,19 @@ int dice_moe_forward(const dice_moe_layer_t *layer, const void *x,
                      void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Stage timers.  Replace the reference's CudaProfiler scopes around the MoE
+ * layer ("moe.gate", "moe.mlp", "moe.mlp_shared": models.py:305,356,375;
+ * cudaprof/prof.py:19-60, expertpara/prof_analyse.py:3-17).  When enabled,
+ * dice_moe_forward (bf16 path) records HIP events on the caller's stream
+ * between its launches; dice_profile_read waits for the last one and returns
+ * the elapsed milliseconds of every stage of the most recent call.
+ */
+int dice_profile_enable(int on);
+int dice_profile_stage_count(void);
+const char *dice_profile_stage_name(int i);
+int dice_profile_read(float *ms_out, int n);
+
+/*
  * Tuning hook, no counterpart in the reference: selects the tile shape of the
  * bf16/fp8 expert GEMMs per stage (0 = library default).  Process-wide; meant
  * for benchmarks that compare tilings, not for the drop-in path.
