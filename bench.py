@@ -22,8 +22,9 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
-# HBM bytes of one fc1 launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/); None until measured.
-FC1_HBM_TRAFFIC_BYTES = None
+# Bytes one fc1 launch moves past the L2 (Infinity Cache + HBM), from rocprofv3 --pmc FETCH_SIZE (x2.0, the
+# factor a plain 256 MiB copy needs) + WRITE_SIZE (x1.0): profiles/layer_c2_bf16_hbm_traffic.txt.
+FC1_HBM_TRAFFIC_BYTES = 1.272e9
 
 N_TOKENS, D, E, TOPK, RATIO = 8192, 1152, 8, 2, 4
 
@@ -142,6 +143,9 @@ def main():
     ap.add_argument("--fc2-cfg", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-stages", action="store_true", help="skip the per-kernel timing pass")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy (a known-size kernel to scale "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the layer holds every expert on one MI355X and uses no "
@@ -156,6 +160,12 @@ def main():
     blk = make_block(args.variant, dev)
     x = torch.randn(N_TOKENS, D, generator=torch.Generator().manual_seed(0)).bfloat16().to(dev)
 
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     sec = time_layer(blk, x, args.steps, args.warmup)
     flops = layer_flops(args.variant)
     total_flops = sum(flops.values())

@@ -57,19 +57,23 @@ __device__ __forceinline__ float dot8<bf16_t, bf16_t>(const Vec8<bf16_t> &x, con
 // step halves the values a lane keeps (the partner takes the other half), so
 // the whole reduction costs 63 lane exchanges instead of 64 x 6, and the
 // summation order is fixed.
-__device__ __forceinline__ float reduce_transpose64(float (&v)[64], int lane) {
+template <int HALF>
+__device__ __forceinline__ void reduce_transpose_step(float (&v)[64], int lane) {
+  const bool upper = lane & HALF;  // partner distance == number of values kept
 #pragma unroll
-  for (int step = 0; step < 6; ++step) {
-    const int mask = 32 >> step;   // partner distance
-    const int half = 32 >> step;   // values kept after this step
-    const bool upper = lane & mask;
-#pragma unroll
-    for (int i = 0; i < half; ++i) {
-      const float keep = upper ? v[i + half] : v[i];
-      const float send = upper ? v[i] : v[i + half];
-      v[i] = keep + __shfl_xor(send, mask, kWave);
-    }
+  for (int i = 0; i < HALF; ++i) {
+    const float keep = upper ? v[i + HALF] : v[i];
+    const float send = upper ? v[i] : v[i + HALF];
+    v[i] = keep + __shfl_xor(send, HALF, kWave);
   }
+}
+__device__ __forceinline__ float reduce_transpose64(float (&v)[64], int lane) {
+  reduce_transpose_step<32>(v, lane);
+  reduce_transpose_step<16>(v, lane);
+  reduce_transpose_step<8>(v, lane);
+  reduce_transpose_step<4>(v, lane);
+  reduce_transpose_step<2>(v, lane);
+  reduce_transpose_step<1>(v, lane);
   return v[0];
 }
 
