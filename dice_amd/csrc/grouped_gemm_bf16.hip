@@ -806,7 +806,8 @@ int launch_grouped_gemm_bf16(const GemmParams &p, int mode, int w_dtype, int64_t
 
 namespace dice {
 constexpr int kCfgPersistent = 20;
-bool gemm_config_wants_persistent() { return g_cfg_fc1 == kCfgPersistent && g_cfg_fc2 == kCfgPersistent; }
+extern int g_persist_waves;
+bool gemm_config_wants_persistent() { return g_cfg_fc1 >= kCfgPersistent && g_cfg_fc2 >= kCfgPersistent; }
 }  // namespace dice
 
 // Tuning hook: selects the tile configuration (0: 128x128x64 / 4 waves,
@@ -815,5 +816,6 @@ bool gemm_config_wants_persistent() { return g_cfg_fc1 == kCfgPersistent && g_cf
 extern "C" int dice_set_gemm_config(int fc1_cfg, int fc2_cfg) {
   dice::g_cfg_fc1 = fc1_cfg;
   dice::g_cfg_fc2 = fc2_cfg;
+  if (fc1_cfg >= dice::kCfgPersistent) dice::g_persist_waves = fc1_cfg == dice::kCfgPersistent + 1 ? 4 : 8;
   return DICE_OK;
 }

@@ -26,21 +26,20 @@
 // Activations must be contiguous grouped rows (the dispatch kernel's gathered
 // copy); weights are [experts, rows, k] bf16 as in the reference's nn.Linear
 // layout (models.py:245-247).
+#include <type_traits>
+
 #include "gemm_common.h"
 
 namespace dice {
 namespace {
 
 constexpr int kPBM = 256, kPBN = 256, kPBK = 32;
-constexpr int kPWavesM = 2, kPWavesN = 4, kPWaves = 8;
+constexpr int kPWavesM = 2;
 constexpr int kPStages = 4, kPAhead = 3;
 constexpr int kPSlotBytes = (kPBM + kPBN) * 64;          // 32 KB
 constexpr int kPRingBytes = kPStages * kPSlotBytes;      // 128 KB
 constexpr int kPStageArea = 32 * 1024;                   // epilogue staging
 constexpr int kPLdsBytes = kPRingBytes + kPStageArea;    // 160 KB
-constexpr int kPCopiesA = kPBM / 16 / kPWaves;           // 1 KB copies per wave per step
-constexpr int kPCopiesB = kPBN / 16 / kPWaves;
-constexpr int kPCopies = kPCopiesA + kPCopiesB;
 constexpr uint32_t kRsrcFlags = 0x00020000u;             // raw buffer, 32-bit elements
 constexpr uint32_t kOutOfRange = 0x80000000u;            // voffset no descriptor covers
 
@@ -55,6 +54,8 @@ __device__ __forceinline__ void phase_barrier() {
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
 }
+
+template <int V> using template_int = std::integral_constant<int, V>;
 
 template <int N> __device__ __forceinline__ void pwait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
@@ -90,6 +91,19 @@ __device__ __forceinline__ void psched_half() {
   if constexpr (LEFT > 0) __builtin_amdgcn_sched_group_barrier(0x008, LEFT, 0);
 }
 
+// One MFMA stream of MF instructions with RD fragment reads behind the first
+// MFMAs (one each) and CP copies behind every other MFMA after that.
+template <int I, int MF, int RD, int CP>
+__device__ __forceinline__ void psched_stream() {
+  if constexpr (I < MF) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    if constexpr (I < RD) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    if constexpr (I >= RD && (I - RD) % 2 == 0 && (I - RD) / 2 < CP)
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    psched_stream<I + 1, MF, RD, CP>();
+  }
+}
+
 // Pins a wave-uniform value into SGPRs (the compiler cannot always prove uniformity
 // of values derived from lane reads; a buffer descriptor held in VGPRs would
 // cost a readfirstlane loop around every copy).
@@ -116,42 +130,60 @@ struct Tile {
   uint32_t c_pitch;          // ldc * 2
   const float *bias;         // + expert * n, or NULL
   int n0, n;                 // first output column, output columns of the problem
-  int steps;                 // k / 32
+  int steps;                 // pipeline steps (k / step extent)
   bool valid;
 };
 
-// HAS_BIAS is a compile-time switch so that the bias-free (reference SwiGLU)
-// instantiations carry no bias loads: a vector load in the epilogue makes the
-// compiler wait for every outstanding copy and store.
-template <int MODE, bool HAS_BIAS>
-__global__ __launch_bounds__(kPWaves *kWave, 1) void gemm_persist_kernel(PersistBatch batch) {
-  constexpr bool SWIGLU = MODE == kFc1Swiglu;
-  constexpr int BN_OUT = SWIGLU ? kPBN / 2 : kPBN;
-  constexpr int WTM = kPBM / kPWavesM, WTN = kPBN / kPWavesN;  // 128 x 64
-  constexpr int TM = WTM / 32, TN = WTN / 32;                  // 4 x 2
-  constexpr int OUT_BLOCKS = SWIGLU ? TN / 2 : TN;
-  constexpr int OUT_COLS = OUT_BLOCKS * 32;
-  constexpr int PITCH = OUT_COLS * 2 + 16;
-  constexpr int BAND = (kPWaves * 32 * PITCH <= kPStageArea) ? 32 : 16;  // rows staged at a time
-  static_assert(kPWaves * BAND * PITCH <= kPStageArea, "staging area too small");
-  constexpr int LANES_PER_ROW = OUT_COLS * 2 / 16;
-  constexpr int ROWS_PER_PASS = kWave / LANES_PER_ROW;
-  constexpr int PASSES = BAND / ROWS_PER_PASS;
-  static_assert(PASSES >= 1, "band smaller than one store pass");
-  constexpr int STORES = (WTM / BAND) * PASSES;  // buffer stores per wave per tile
-  constexpr int WAIT_STEADY = (kPAhead - 1) * kPCopies;  // copies of the two newest steps
-  constexpr int WAIT_AFTER_EPILOGUE = WAIT_STEADY + STORES;
-  static_assert(WAIT_AFTER_EPILOGUE < 64, "vmcnt is a 6-bit counter");
+// A tile description parked in ONE vector register (lane f holds 32-bit word f),
+// for descriptions that are not needed for a while: scalar registers are scarce
+// and a description spilled by the compiler would come back as per-lane values,
+// which buffer instructions cannot take without a loop over lanes.
+struct PackedTile {
+  uint32_t words;
+};
+__device__ __forceinline__ PackedTile pack_tile(const Tile &t, int lane) {
+  const uint64_t p[5] = {(uint64_t)t.a, (uint64_t)t.b0, (uint64_t)t.b1, (uint64_t)t.c, (uint64_t)t.bias};
+  const uint32_t w[10] = {t.a_bytes, t.a_pitch, t.b_bytes, t.b_pitch, t.c_bytes,
+                          t.c_pitch, (uint32_t)t.n0, (uint32_t)t.n, (uint32_t)t.steps, t.valid ? 1u : 0u};
+  uint32_t v = 0;
+#pragma unroll
+  for (int i = 0; i < 5; ++i) {
+    v = lane == 2 * i ? (uint32_t)p[i] : v;
+    v = lane == 2 * i + 1 ? (uint32_t)(p[i] >> 32) : v;
+  }
+#pragma unroll
+  for (int i = 0; i < 10; ++i) v = lane == 10 + i ? w[i] : v;
+  return PackedTile{v};
+}
+__device__ __forceinline__ Tile unpack_tile(const PackedTile &pk) {
+  auto word = [&](int i) { return (uint32_t)__builtin_amdgcn_readlane(pk.words, i); };
+  auto ptr = [&](int i) { return ((uint64_t)word(2 * i + 1) << 32) | word(2 * i); };
+  Tile t;
+  t.a = (const unsigned char *)ptr(0);
+  t.b0 = (const unsigned char *)ptr(1);
+  t.b1 = (const unsigned char *)ptr(2);
+  t.c = (unsigned char *)ptr(3);
+  t.bias = (const float *)ptr(4);
+  t.a_bytes = word(10); t.a_pitch = word(11); t.b_bytes = word(12); t.b_pitch = word(13);
+  t.c_bytes = word(14); t.c_pitch = word(15);
+  t.n0 = (int)word(16); t.n = (int)word(17); t.steps = (int)word(18);
+  t.valid = word(19) != 0;
+  return t;
+}
 
-  extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave / kPWavesN, wn = wave % kPWavesN;
+// The tile order of one launch and this workgroup's share of it.  Lane g of
+// every wave describes group g = (problem, expert): its rows, its tile grid and
+// the index of its first tile (at most 64 groups); a tile id is mapped back to
+// its group with one ballot.  Tiles are ordered problem-major, expert-major,
+// then n-tile with the m-tile fastest.  XCD x (= blockIdx.x % 8) owns the x-th
+// eighth of that order and its workgroups take tiles of the run round-robin.
+template <int BN_OUT>
+struct TileWalker {
+  int g_prob = 0, g_expert = 0, g_row0 = 0, g_cnt = 0, g_mt = 0, g_base = 0, g_end = 0;
+  int run_begin, run_end, wg_in_xcd, wgs_per_xcd;
 
-  // ---- group table: lane g describes group g = (problem, expert) ----
-  int g_prob = 0, g_expert = 0, g_row0 = 0, g_cnt = 0, g_mt = 0, g_nt = 0, g_base = 0;
-  {
-    int acc_groups = 0;
+  __device__ __forceinline__ TileWalker(const PersistBatch &batch, int lane) {
+    int g_nt = 0, acc_groups = 0;
     for (int pi = 0; pi < batch.n_problems; ++pi) {
       const PersistProblem &pr = batch.prob[pi];
       const int local = lane - acc_groups;
@@ -165,27 +197,27 @@ __global__ __launch_bounds__(kPWaves *kWave, 1) void gemm_persist_kernel(Persist
       }
       acc_groups += pr.n_experts;
     }
-    int tiles = g_mt * g_nt, inc = tiles;
+    const int tiles = g_mt * g_nt;
+    int inc = tiles;
 #pragma unroll
     for (int o = 1; o < kWave; o <<= 1) {
       const int up = __shfl_up(inc, o, kWave);
       if (lane >= o) inc += up;
     }
     g_base = inc - tiles;
+    g_end = inc;
+    const int total_tiles = __shfl(inc, kWave - 1, kWave);
+    const int per_xcd = (total_tiles + kNumXcd - 1) / kNumXcd;
+    const int xcd = blockIdx.x % kNumXcd;
+    wg_in_xcd = blockIdx.x / kNumXcd;
+    wgs_per_xcd = gridDim.x / kNumXcd;
+    run_begin = xcd * per_xcd;
+    run_end = run_begin + per_xcd < total_tiles ? run_begin + per_xcd : total_tiles;
   }
-  const int total_tiles = __shfl(g_base + g_mt * g_nt, kWave - 1, kWave);
-  const int g_end = g_base + g_mt * g_nt;
 
-  // This workgroup's share: XCD x (= blockIdx.x % 8) owns the x-th eighth of the
-  // tile order; its workgroups take tiles of that run round-robin.
-  const int per_xcd = (total_tiles + kNumXcd - 1) / kNumXcd;
-  const int xcd = blockIdx.x % kNumXcd;
-  const int wg_in_xcd = blockIdx.x / kNumXcd;
-  const int wgs_per_xcd = gridDim.x / kNumXcd;
-  const int run_begin = xcd * per_xcd;
-  const int run_end = run_begin + per_xcd < total_tiles ? run_begin + per_xcd : total_tiles;
-
-  auto decode = [&](int id) {
+  // Tile `id` of the order (ids past this XCD's run give an invalid tile whose
+  // descriptors cover no bytes); `bk` is the k extent of one pipeline step.
+  __device__ __forceinline__ Tile decode(const PersistBatch &batch, int id, int bk) const {
     Tile t;
     t.valid = id < run_end;
     const int idc = t.valid ? id : 0;
@@ -219,7 +251,7 @@ __global__ __launch_bounds__(kPWaves *kWave, 1) void gemm_persist_kernel(Persist
     t.c = (unsigned char *)pr.c + (size_t)(row0 + m_tile * kPBM) * t.c_pitch;
     t.c_bytes = (uint32_t)rows * t.c_pitch;
     t.bias = pr.bias ? pr.bias + (size_t)expert * pr.n : nullptr;
-    t.steps = pr.k / kPBK;
+    t.steps = pr.k / bk;
     t.a = uni(t.a); t.b0 = uni(t.b0); t.b1 = uni(t.b1); t.c = uni(t.c); t.bias = uni(t.bias);
     t.a_bytes = uni(t.a_bytes); t.a_pitch = uni(t.a_pitch);
     t.b_bytes = uni(t.b_bytes); t.b_pitch = uni(t.b_pitch);
@@ -227,7 +259,145 @@ __global__ __launch_bounds__(kPWaves *kWave, 1) void gemm_persist_kernel(Persist
     t.n0 = uni(t.n0); t.n = uni(t.n); t.steps = uni(t.steps);
     t.valid = uni((int)t.valid) != 0;
     return t;
-  };
+  }
+};
+
+// Geometry of one wave's epilogue: its TM x TN accumulator blocks become
+// OUT_COLS output columns (SwiGLU folds gate and up blocks), staged BAND rows at
+// a time through WAVE_BYTES of LDS and stored as whole 16-byte row chunks.
+template <int MODE, int WAVES, int TM, int TN>
+struct EpiGeom {
+  static constexpr bool SWIGLU = MODE == kFc1Swiglu;
+  static constexpr int OUT_BLOCKS = SWIGLU ? TN / 2 : TN;
+  static constexpr int OUT_COLS = OUT_BLOCKS * 32;
+  static constexpr int PITCH = OUT_COLS * 2 + 16;
+  static constexpr int BAND = (WAVES * 32 * PITCH <= kPStageArea) ? 32 : 16;  // rows staged at a time
+  static constexpr int LANES_PER_ROW = OUT_COLS * 2 / 16;
+  static constexpr int ROWS_PER_PASS = kWave / LANES_PER_ROW;
+  static constexpr int PASSES = BAND / ROWS_PER_PASS;
+  static constexpr int STORES = (TM * 32 / BAND) * PASSES;  // buffer stores per wave per tile
+  static constexpr int WAVE_BYTES = BAND * PITCH;
+  static_assert(WAVES * WAVE_BYTES <= kPStageArea, "staging area too small");
+  static_assert(PASSES >= 1, "band smaller than one store pass");
+};
+
+// One accumulator element for the epilogue's arithmetic.  With four waves the
+// accumulators live in the accumulation registers; left to itself the compiler
+// copies whole 16-register blocks out at the top of the epilogue and then spills
+// them, so the read is pinned to the place where the value is used.
+template <bool FROM_ACC_REGS>
+__device__ __forceinline__ float acc_value(const float &a) {
+  if constexpr (FROM_ACC_REGS) {
+    float v;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+    return v;
+  } else {
+    return a;
+  }
+}
+
+// Epilogue of tile `cp` for one wave: activation (and bias), transposition through
+// the wave's LDS staging rows, row-segment stores.  Rows past the group's end are
+// dropped by the descriptor's range check, columns past the problem's n by an
+// offset no descriptor covers.
+template <int MODE, bool HAS_BIAS, int WAVES, int TM, int TN>
+__device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM][TN], unsigned char *stage,
+                                              int wave_row0, int wave_col0, int lane) {
+  using G = EpiGeom<MODE, WAVES, TM, TN>;
+  constexpr bool SWIGLU = G::SWIGLU;
+  constexpr int OUT_BLOCKS = G::OUT_BLOCKS, PITCH = G::PITCH, BAND = G::BAND;
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  const int rd_row = lane / G::LANES_PER_ROW, rd_chunk = lane % G::LANES_PER_ROW;
+  const __amdgpu_buffer_rsrc_t crs =
+      __builtin_amdgcn_make_buffer_rsrc((void *)cp.c, 0, cp.c_bytes, kRsrcFlags);
+  const int col_base = cp.n0 + wave_col0;
+  // Bias of this lane's columns, fetched in one batch (one wait instead of one per element).
+  float bias_v[OUT_BLOCKS][16];
+  if (HAS_BIAS) {
+#pragma unroll
+    for (int j = 0; j < OUT_BLOCKS; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) bias_v[j][e] = 0.f;
+    if (cp.bias) {
+#pragma unroll
+      for (int j = 0; j < OUT_BLOCKS; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int cn = col_base + j * 32 + frag_half * 4 + (e >> 2) * 8 + (e & 3);
+          bias_v[j][e] = cp.bias[cn < cp.n ? cn : 0];
+        }
+    }
+  }
+#pragma unroll
+  for (int band = 0; band < TM * 32 / BAND; ++band) {
+    const int i = band * BAND / 32;             // 32-row block the band lies in
+    const int half = (band * BAND % 32) / 16;   // which 16 rows of it (BAND == 16 only)
+    if (BAND == 32 || (frag_row >> 4) == half) {
+      const int srow = BAND == 32 ? frag_row : (frag_row & 15);
+#pragma unroll
+      for (int j = 0; j < OUT_BLOCKS; ++j) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int col = j * 32 + frag_half * 4 + q * 8;
+          bf16x4_t o;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float v = acc_value<WAVES == 4>(acc[i][j][q * 4 + r]);
+            if (SWIGLU) {
+              v = silu_fast(v) * acc_value<WAVES == 4>(acc[i][j + OUT_BLOCKS][q * 4 + r]);
+            } else {
+              if (HAS_BIAS) v += bias_v[j][q * 4 + r];
+              if (MODE == kFc1Gelu) v = gelu_tanh_fast(v);
+            }
+            o[r] = (bf16_t)v;
+          }
+          *reinterpret_cast<u32x2_any_t *>(stage + srow * PITCH + col * 2) = __builtin_bit_cast(u32x2_t, o);
+        }
+      }
+    }
+    wave_lds_sync();
+#pragma unroll
+    for (int ps = 0; ps < G::PASSES; ++ps) {
+      const int r = ps * G::ROWS_PER_PASS + rd_row;
+      const u32x4_t v = *reinterpret_cast<const u32x4_any_t *>(stage + r * PITCH + rd_chunk * 16);
+      const int m = wave_row0 + band * BAND + r;
+      const int n = col_base + rd_chunk * 8;
+      const uint32_t voff = n < cp.n ? (uint32_t)m * cp.c_pitch + (uint32_t)n * 2 : kOutOfRange;
+      __builtin_amdgcn_raw_buffer_store_b128(v, crs, voff, 0, 0);
+    }
+    wave_lds_sync();  // the next band overwrites the staging rows
+    // Keeps the bands apart: hoisting the next band's accumulator reads over this
+    // one's stores only lengthens live ranges (register spills cost far more
+    // here than the lost overlap).
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// HAS_BIAS is a compile-time switch so that the bias-free (reference SwiGLU)
+// instantiations carry no bias loads: a vector load in the epilogue makes the
+// compiler wait for every outstanding copy and store.
+template <int MODE, bool HAS_BIAS, int kPWaves>
+__device__ __forceinline__ void gemm_persist_body(const PersistBatch &batch) {
+  static_assert(kPWaves == 4 || kPWaves == 8, "four or eight waves");
+  constexpr int kPWavesN = kPWaves / kPWavesM;
+  constexpr int kPCopiesA = kPBM / 16 / kPWaves;  // 1 KB copies per wave per step
+  constexpr int kPCopiesB = kPBN / 16 / kPWaves;
+  constexpr int kPCopies = kPCopiesA + kPCopiesB;
+  constexpr bool SWIGLU = MODE == kFc1Swiglu;
+  constexpr int BN_OUT = SWIGLU ? kPBN / 2 : kPBN;
+  constexpr int WTM = kPBM / kPWavesM, WTN = kPBN / kPWavesN;  // 128 x 64 (eight waves) or 128 x 128
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  using Epi = EpiGeom<MODE, kPWaves, TM, TN>;
+  constexpr int WAIT_STEADY = (kPAhead - 1) * kPCopies;  // copies of the two newest steps
+
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / kPWavesN, wn = wave % kPWavesN;
+
+  TileWalker<BN_OUT> walk(batch, lane);
+  const int run_begin = walk.run_begin, wg_in_xcd = walk.wg_in_xcd, wgs_per_xcd = walk.wgs_per_xcd;
+  auto decode = [&](int id) { return walk.decode(batch, id, kPBK); };
 
   // ---- per-lane copy offsets (row part depends on the tile's pitch) ----
   const int lrow = lane >> 2, lchunk = lane & 3;
@@ -246,26 +416,38 @@ __global__ __launch_bounds__(kPWaves *kWave, 1) void gemm_persist_kernel(Persist
     cp_chunk[kPCopiesA + i] = (lchunk ^ pswizzle(rt)) << 4;
   }
 
+  // Per-lane byte offsets of this wave's copies inside the tile being copied.
+  // They depend on the tile's row pitches only, so they are worked out once per
+  // tile; the asm statement keeps the compiler from re-deriving them (integer
+  // multiplies) inside every k step, where vector ALU work competes with the
+  // other group's MFMAs for the SIMD's issue slots.
+  uint32_t ld_voff[kPCopies];
+  auto set_copy_offsets = [&](const Tile &t) {
+#pragma unroll
+    for (int l = 0; l < kPCopies; ++l) {
+      ld_voff[l] = (uint32_t)cp_row[l] * (l < kPCopiesA ? t.a_pitch : t.b_pitch) + cp_chunk[l];
+      asm volatile("" : "+v"(ld_voff[l]));
+    }
+  };
+
   // Issues copy `l` of the step `kt` of tile `t` into ring slot `slot`.
   auto issue_copy = [&](const Tile &t, int kt, int slot, int l) {
     unsigned char *dst = lds_raw + slot * kPSlotBytes;
     if (l < kPCopiesA) {
       const __amdgpu_buffer_rsrc_t rs =
           __builtin_amdgcn_make_buffer_rsrc((void *)t.a, 0, t.a_bytes, kRsrcFlags);
-      const uint32_t voff = (uint32_t)cp_row[l] * t.a_pitch + cp_chunk[l];
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rs, (__attribute__((address_space(3))) void *)(dst + (wave + kPWaves * l) * 1024), 16, voff,
-          kt * 64, 0, 0);
+          rs, (__attribute__((address_space(3))) void *)(dst + (wave + kPWaves * l) * 1024), 16,
+          ld_voff[l], kt * 64, 0, 0);
     } else {
       const int i = l - kPCopiesA;
-      const bool up_half = SWIGLU && (wave + kPWaves * i) * 16 >= kPBN / 2;
+      const bool up_half = SWIGLU && kPWaves * i * 16 >= kPBN / 2;  // wave * 16 < 128 never crosses the halves
       const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
           (void *)(up_half ? t.b1 : t.b0), 0, t.b_bytes, kRsrcFlags);
-      const uint32_t voff = (uint32_t)cp_row[l] * t.b_pitch + cp_chunk[l];
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
           rs,
           (__attribute__((address_space(3))) void *)(dst + kPBM * 64 + (wave + kPWaves * i) * 1024), 16,
-          voff, kt * 64, 0, 0);
+          ld_voff[l], kt * 64, 0, 0);
     }
   };
 
@@ -278,16 +460,29 @@ __global__ __launch_bounds__(kPWaves *kWave, 1) void gemm_persist_kernel(Persist
   };
   const int frag_row = lane & 31, frag_half = lane >> 5;
   bf16x8_t wf[2][TN], af[2][TM];
-  auto read_frags = [&](int slot, int kk, int buf) {
-    const unsigned char *sa = lds_raw + slot * kPSlotBytes;
-    const unsigned char *sb = sa + kPBM * 64;
-    const int chunk = kk * 2 + frag_half;
+  // Lane part of the fragment addresses for the two 16-k halves of a step; the
+  // 32-row block and the ring slot only add compile-time constants (the swizzle
+  // uses row bits 1..3, which block offsets do not touch), so the reads of a
+  // step need no address arithmetic.
+  uint32_t rd_a[2], rd_b[2];
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
-      wf[buf][j] = *reinterpret_cast<const bf16x8_t *>(sb + pring_off(w_block_row(j) + frag_row, chunk));
+  for (int kk = 0; kk < 2; ++kk) {
+    rd_a[kk] = pring_off(wm * WTM + frag_row, kk * 2 + frag_half);
+    rd_b[kk] = kPBM * 64 + pring_off(w_block_row(0) + frag_row, kk * 2 + frag_half);
+    asm volatile("" : "+v"(rd_a[kk]), "+v"(rd_b[kk]));
+  }
+  auto read_frags = [&](auto slot_c, int kk, int buf) {
+    constexpr int SLOT = decltype(slot_c)::value;
+    const unsigned char *base = lds_raw + SLOT * kPSlotBytes;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      constexpr int HALF = TN / 2;
+      const int joff = (SWIGLU && j >= HALF) ? (kPBN / 2 + (j - HALF) * 32) * 64 : j * 32 * 64;
+      wf[buf][j] = *reinterpret_cast<const bf16x8_t *>(base + rd_b[kk] + joff);
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
-      af[buf][i] = *reinterpret_cast<const bf16x8_t *>(sa + pring_off(wm * WTM + i * 32 + frag_row, chunk));
+      af[buf][i] = *reinterpret_cast<const bf16x8_t *>(base + rd_a[kk] + i * 32 * 64);
   };
 
   f32x16_t acc[TM][TN];
@@ -307,16 +502,17 @@ __global__ __launch_bounds__(kPWaves *kWave, 1) void gemm_persist_kernel(Persist
   if (!ld.valid) return;                         // nothing to do for this workgroup
   Tile cp = ld;                                  // tile being multiplied
   int ld_kt = 0;
-  int cslot = 0;                                 // ring slot of the step being multiplied
 
   // Advances the copy side by one step (wave-uniform control flow only).
   auto advance_copy = [&]() {
     if (++ld_kt == ld.steps) {
       ld = decode(next_id);
+      set_copy_offsets(ld);
       next_id += wgs_per_xcd;
       ld_kt = 0;
     }
   };
+  set_copy_offsets(ld);
 
 #pragma unroll
   for (int s = 0; s < kPAhead; ++s) {
@@ -325,148 +521,379 @@ __global__ __launch_bounds__(kPWaves *kWave, 1) void gemm_persist_kernel(Persist
     advance_copy();
   }
   zero_acc();
-  pwait_vmcnt<WAIT_STEADY>();
-  phase_barrier();                      // everyone's copies of steps 0 and 1 have landed
   int since_epilogue = 2;
-
-  const int stage_base = kPRingBytes + wave * (BAND * PITCH);
-  const int rd_row = lane / LANES_PER_ROW, rd_chunk = lane % LANES_PER_ROW;
+  const int stage_base = kPRingBytes + wave * Epi::WAVE_BYTES;
   const int wave_col0 = SWIGLU ? wn * (WTN / 2) : wn * WTN;
 
-  // Two groups of four waves (one wave of each group per SIMD) alternate between
-  // a memory phase (fragment reads of one k step + this wave's share of the
-  // copies three steps ahead) and a compute phase (the step's 16 MFMAs), one
-  // phase apart: while one group multiplies the other one loads, so the matrix
-  // pipe only idles for the barrier hand-over between phases.
-  const int group = wm;
-  // Waits until at most the copies of the two newest steps (plus the stores of an
-  // epilogue that was issued in between) are still in flight.
-  auto copies_landed = [&]() {
-    if (since_epilogue < 2) pwait_vmcnt<WAIT_AFTER_EPILOGUE>();
-    else pwait_vmcnt<WAIT_STEADY>();
-    ++since_epilogue;
+  auto epilogue = [&]() {
+    // Loads and stores may retire out of order with respect to each other, so
+    // after the stores of the epilogue the counter no longer tells how many
+    // copies are pending.  Drain the copies first (the next tile's first three
+    // steps; the youngest were issued one step ago) and skip the waits of the
+    // next tile's first two steps, whose operands are then known to have landed.
+    pwait_vmcnt<0>();
+    tile_epilogue<MODE, HAS_BIAS, kPWaves, TM, TN>(cp, acc, lds_raw + stage_base, wm * WTM, wave_col0, lane);
   };
-  while (true) {  // one tile per iteration
-    if (group == 1) phase_barrier();
-    for (int s = 0; s < cp.steps; ++s) {
-      // ---- memory phase ----
-      const int lslot = (cslot + kPAhead) & (kPStages - 1);  // slot of the step before this one
-      read_frags(cslot, 0, 0);
-      read_frags(cslot, 1, 1);
-#pragma unroll
-      for (int l = 0; l < kPCopies; ++l) issue_copy(ld, ld_kt, lslot, l);
-      advance_copy();
-      // The first reader of step s+1 is the first group, right after the barrier
-      // that ends this phase pair.  Each wave therefore confirms that its own
-      // copies of step s+1 have landed at the last barrier before that point:
-      // the second group at the end of its memory phase, the first group at the
-      // end of its compute phase.  Copies get four to five phases to land.
-      if (group == 1) copies_landed();
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // slot fully read before anyone may refill it
-      phase_barrier();
-      // ---- compute phase ----
-#ifndef DICE_PRIO_COMPUTE
-#define DICE_PRIO_COMPUTE 0
-#endif
-#ifndef DICE_PRIO_MEMORY
-#define DICE_PRIO_MEMORY 0
-#endif
-      __builtin_amdgcn_s_setprio(DICE_PRIO_COMPUTE);
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[kk][j], af[kk][i], acc[i][j], 0, 0, 0);
-      __builtin_amdgcn_s_setprio(DICE_PRIO_MEMORY);
-      if (group == 0) copies_landed();
-      phase_barrier();
-      cslot = (cslot + 1) & (kPStages - 1);
-    }
-    if (group == 0) phase_barrier();  // let the other group finish the tile's last step
 
-    // ---- epilogue of tile `cp` ----
-    {
-      const __amdgpu_buffer_rsrc_t crs =
-          __builtin_amdgcn_make_buffer_rsrc((void *)cp.c, 0, cp.c_bytes, kRsrcFlags);
-      unsigned char *stage = lds_raw + stage_base;
-      const int col_base = cp.n0 + wave_col0;
-      // Bias of this lane's columns, fetched in one batch (one wait instead of one per element).
-      float bias_v[OUT_BLOCKS][16];
-      if (HAS_BIAS) {
-#pragma unroll
-        for (int j = 0; j < OUT_BLOCKS; ++j)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) bias_v[j][e] = 0.f;
-        if (cp.bias) {
-#pragma unroll
-          for (int j = 0; j < OUT_BLOCKS; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-              const int cn = col_base + j * 32 + frag_half * 4 + (e >> 2) * 8 + (e & 3);
-              bias_v[j][e] = cp.bias[cn < cp.n ? cn : 0];
-            }
-        }
+  if constexpr (kPWaves == 8) {
+    // Two groups of four waves (one wave of each group per SIMD) alternate between
+    // a memory phase (fragment reads of one k step + this wave's share of the
+    // copies three steps ahead) and a compute phase (the step's 16 MFMAs), one
+    // phase apart: while one group multiplies the other one loads, so the matrix
+    // pipe only idles for the barrier hand-over between phases.
+    const int group = wm;
+    // Waits until at most the copies of the two newest steps are still in flight.
+    auto copies_landed = [&]() {
+      if (since_epilogue >= 2) pwait_vmcnt<WAIT_STEADY>();
+      ++since_epilogue;
+    };
+    pwait_vmcnt<WAIT_STEADY>();
+    phase_barrier();                      // everyone's copies of step 0 have landed
+    while (true) {  // one tile per iteration
+      if (group == 1) phase_barrier();
+      // The ring position of a step is a compile-time constant: every tile has a
+      // multiple of kPStages steps, so a tile always starts in slot 0.
+      auto step = [&](auto slot_c) {
+        constexpr int cslot = decltype(slot_c)::value;
+        // ---- memory phase ----
+        constexpr int lslot = (cslot + kPAhead) & (kPStages - 1);  // slot of the step before this one
+        read_frags(slot_c, 0, 0);
+        read_frags(slot_c, 1, 1);
+  #pragma unroll
+        for (int l = 0; l < kPCopies; ++l) issue_copy(ld, ld_kt, lslot, l);
+        advance_copy();
+        // The first reader of step s+1 is the first group, right after the barrier
+        // that ends this phase pair.  Each wave therefore confirms that its own
+        // copies of step s+1 have landed at the last barrier before that point:
+        // the second group at the end of its memory phase, the first group at the
+        // end of its compute phase.  Copies get four to five phases to land.
+        if (group == 1) copies_landed();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // slot fully read before anyone may refill it
+        phase_barrier();
+        // ---- compute phase ----
+  #ifndef DICE_PRIO_COMPUTE
+  #define DICE_PRIO_COMPUTE 0
+  #endif
+  #ifndef DICE_PRIO_MEMORY
+  #define DICE_PRIO_MEMORY 0
+  #endif
+        __builtin_amdgcn_s_setprio(DICE_PRIO_COMPUTE);
+  #pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
+  #pragma unroll
+          for (int i = 0; i < TM; ++i)
+  #pragma unroll
+            for (int j = 0; j < TN; ++j)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[kk][j], af[kk][i], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_s_setprio(DICE_PRIO_MEMORY);
+        if (group == 0) copies_landed();
+        phase_barrier();
+      };
+      for (int s = 0; s < cp.steps; s += kPStages) {
+        step(std::integral_constant<int, 0>{});
+        step(std::integral_constant<int, 1>{});
+        step(std::integral_constant<int, 2>{});
+        step(std::integral_constant<int, 3>{});
       }
-#pragma unroll
-      for (int band = 0; band < WTM / BAND; ++band) {
-        const int i = band * BAND / 32;             // 32-row block the band lies in
-        const int half = (band * BAND % 32) / 16;   // which 16 rows of it (BAND == 16 only)
-        if (BAND == 32 || (frag_row >> 4) == half) {
-          const int srow = BAND == 32 ? frag_row : (frag_row & 15);
-#pragma unroll
-          for (int j = 0; j < OUT_BLOCKS; ++j) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const int col = j * 32 + frag_half * 4 + q * 8;
-              bf16x4_t o;
-#pragma unroll
-              for (int r = 0; r < 4; ++r) {
-                float v = acc[i][j][q * 4 + r];
-                if (SWIGLU) {
-                  v = silu_fast(v) * acc[i][j + OUT_BLOCKS][q * 4 + r];
-                } else {
-                  if (HAS_BIAS) v += bias_v[j][q * 4 + r];
-                  if (MODE == kFc1Gelu) v = gelu_tanh_fast(v);
-                }
-                o[r] = (bf16_t)v;
-              }
-              *reinterpret_cast<u32x2_any_t *>(stage + srow * PITCH + col * 2) = __builtin_bit_cast(u32x2_t, o);
-            }
-          }
-        }
-        wave_lds_sync();
-#pragma unroll
-        for (int ps = 0; ps < PASSES; ++ps) {
-          const int r = ps * ROWS_PER_PASS + rd_row;
-          const u32x4_t v = *reinterpret_cast<const u32x4_any_t *>(stage + r * PITCH + rd_chunk * 16);
-          const int m = wm * WTM + band * BAND + r;
-          const int n = col_base + rd_chunk * 8;
-          const uint32_t voff = n < cp.n ? (uint32_t)m * cp.c_pitch + (uint32_t)n * 2 : kOutOfRange;
-          __builtin_amdgcn_raw_buffer_store_b128(v, crs, voff, 0, 0);
-        }
-        wave_lds_sync();  // the next band overwrites the staging rows
-      }
+      if (group == 0) phase_barrier();  // let the other group finish the tile's last step
+
+      epilogue();
+      // Every tile has more than AHEAD steps, so the copy side is exactly one
+      // tile ahead here: the tile it is working on is the one to multiply next.
+      cp = ld;
+      if (!cp.valid) break;
+      since_epilogue = 0;
+      zero_acc();
     }
-    // Every tile has more than AHEAD steps, so the copy side is exactly one
-    // tile ahead here: the tile it is working on is the one to multiply next.
-    cp = ld;
-    if (!cp.valid) break;
-    since_epilogue = 0;
-    zero_acc();
   }
   pwait_vmcnt<0>();
 }
 
+// ---------------------------------------------------------------------------
+// 64-k pipeline, four waves, operands staged through registers.
+//
+// Two things bound the 32-k pipeline above.  The L2 serves whole 128-byte lines:
+// a 32-k step asks for half a line per row and reaches about half the copy rate
+// of a 64-k step.  And a copy takes 1 to 2 us from request to data while a 64-k
+// step multiplies for 1.3 us, so more than one step has to be in flight - but a
+// 64-k step of a 256x256 tile is 64 KB and only two fit the LDS next to the
+// epilogue's staging area.
+//
+// Here a step is 64 k (rows of 128 bytes, two 64 KB LDS slots) and the data in
+// flight lives in registers: four waves, one per SIMD with the whole register
+// file, own 128x128 of the tile each (accumulators in the accumulation
+// registers); every wave loads its share of a step (16 x 16 bytes per lane)
+// into one of two register stages FOUR steps ahead and writes it to the LDS
+// slot two steps later, as soon as that slot has been read for the last time.
+// Loads and LDS writes are cut into quarters, one per 16-MFMA block, so every
+// block carries the same small side load: 8 fragment reads, 4 LDS writes and 4
+// global loads threaded between its MFMAs.  The one barrier of a step sits
+// before its last block: by then every wave has read the last fragments of
+// the step's slot (so the slot may be rewritten) and has finished writing the
+// other slot (so the next step's first fragments may be read).
+constexpr int kQBK = 64;
+constexpr int kQWaves = 4;
+constexpr int kQSlotBytes = (kPBM + kPBN) * 128;   // 64 KB
+constexpr int kQRingBytes = 2 * kQSlotBytes;       // staging area follows
+constexpr int kQCopies = (kPBM + kPBN) / 8 / kQWaves;  // 16-byte-per-lane loads (8 rows each) per wave per step
+constexpr int kQMinSteps = 6;                      // loads run four steps ahead, within the next tile
+static_assert(kQRingBytes == kPRingBytes, "both pipelines share the LDS budget");
+static_assert(kQCopies == 16, "a step is four quarters of four loads");
+
+__device__ __forceinline__ int qswizzle(int row) { return (row >> 1) & 7; }
+// Byte offset of 16-byte chunk `chunk` (0..7) of `row` inside a slot half: any
+// 16 consecutive rows put one chunk index into 16 different bank groups.
+__device__ __forceinline__ int qring_off(int row, int chunk) {
+  return row * 128 + ((chunk ^ qswizzle(row)) << 4);
+}
+
+// Instruction order of one block of MF MFMAs: RD fragment reads behind the
+// first MFMAs (one each), then WR LDS writes and LD global loads, one behind
+// each of the following MFMAs.
+template <int I, int MF, int RD, int WR, int LD>
+__device__ __forceinline__ void qsched_block() {
+  if constexpr (I < MF) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    if constexpr (I < RD) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    else if constexpr (I < RD + WR) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+    else if constexpr (I < RD + WR + LD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    qsched_block<I + 1, MF, RD, WR, LD>();
+  }
+}
+
+template <int MODE, bool HAS_BIAS>
+__device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
+  constexpr bool SWIGLU = MODE == kFc1Swiglu;
+  constexpr int BN_OUT = SWIGLU ? kPBN / 2 : kPBN;
+  constexpr int WTM = 128, WTN = 128, TM = 4, TN = 4;
+  using Epi = EpiGeom<MODE, kQWaves, TM, TN>;
+  const template_int<0> c0; const template_int<1> c1; const template_int<2> c2; const template_int<3> c3;
+
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+
+  TileWalker<BN_OUT> walk(batch, lane);
+  auto decode = [&](int id) { return walk.decode(batch, id, kQBK); };
+
+  // ---- global loads: one instruction fetches 8 rows x 128 bytes (8 lanes per
+  // row, i.e. whole lines); load l of a wave covers rows (wave + 4 (l % 8)) * 8
+  // .. + 8 of the activation tile (l < 8) or of the weight tile. ----
+  const int cp_row0 = wave * 8 + (lane >> 3);
+  const int cp_chunk = lane & 7;
+  // LDS address of this lane's chunk in slot 0 (row bits 1..3, which the swizzle
+  // reads, are the same for every l)
+  uint32_t wr_off = qring_off(cp_row0, cp_chunk);
+  asm volatile("" : "+v"(wr_off));
+  uint32_t ld_voff_a = 0, ld_voff_b = 0;  // per-lane byte offsets inside the tile being loaded
+  auto set_copy_offsets = [&](const Tile &t) {
+    ld_voff_a = (uint32_t)cp_row0 * t.a_pitch + cp_chunk * 16;
+    ld_voff_b = (uint32_t)cp_row0 * t.b_pitch + cp_chunk * 16;
+    asm volatile("" : "+v"(ld_voff_a), "+v"(ld_voff_b));
+  };
+  u32x4_t stage_regs[2][kQCopies];
+
+  // ---- fragment reads: lane part per 16-k block; 32-row blocks and the slot
+  // add compile-time constants ----
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  const int b_row0 = SWIGLU ? wn * (WTN / 2) : wn * WTN;
+  uint32_t rd_a[4], rd_b[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) {
+    rd_a[kk] = qring_off(wm * WTM + frag_row, kk * 2 + frag_half);
+    rd_b[kk] = kPBM * 128 + qring_off(b_row0 + frag_row, kk * 2 + frag_half);
+    asm volatile("" : "+v"(rd_a[kk]), "+v"(rd_b[kk]));
+  }
+  bf16x8_t wf[2][TN], af[2][TM];
+  auto read_frags = [&](auto slot_c, auto kk_c, int buf) {
+    constexpr int SLOT = decltype(slot_c)::value, KK = decltype(kk_c)::value;
+    const unsigned char *base = lds_raw + SLOT * kQSlotBytes;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      constexpr int HALF = TN / 2;
+      const int jrow = (SWIGLU && j >= HALF) ? kPBN / 2 + (j - HALF) * 32 : j * 32;
+      wf[buf][j] = *reinterpret_cast<const bf16x8_t *>(base + rd_b[KK] + jrow * 128);
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      af[buf][i] = *reinterpret_cast<const bf16x8_t *>(base + rd_a[KK] + i * 32 * 128);
+  };
+
+  f32x16_t acc[TM][TN];
+  auto zero_acc = [&]() {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+  };
+  auto mfma_block = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[buf][j], af[buf][i], acc[i][j], 0, 0, 0);
+  };
+
+  // ---- pipeline state ----
+  // The load side runs four steps ahead of the MFMAs, so it crosses into the
+  // next tile once while a tile is multiplied.  That tile's description (`nxt`)
+  // is worked out between tiles, where registers are free, not inside the k loop.
+  int next_id = walk.run_begin + walk.wg_in_xcd;
+  Tile ld = decode(next_id);                      // tile being loaded
+  next_id += walk.wgs_per_xcd;
+  if (!ld.valid) return;                          // nothing to do for this workgroup
+  PackedTile nxt = pack_tile(decode(next_id), lane);    // the one the load side opens next
+  next_id += walk.wgs_per_xcd;
+  Tile cp = ld;                                   // tile being multiplied
+  int ld_kt = 0;
+  set_copy_offsets(ld);
+  auto advance_copy = [&]() {
+    if (++ld_kt == ld.steps) {
+      ld = unpack_tile(nxt);
+      set_copy_offsets(ld);
+      ld_kt = 0;
+    }
+  };
+  // Quarter q (loads 4 q .. 4 q + 3) of the step the load side stands at, into
+  // register stage P.
+  auto load_quarter = [&](auto stage_c, auto q_c) {
+    constexpr int P = decltype(stage_c)::value, Q = decltype(q_c)::value;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      constexpr int HALF_COPIES = kQCopies / 2;
+      const int l = Q * 4 + c, i = l % HALF_COPIES;
+      if (l < HALF_COPIES) {
+        const __amdgpu_buffer_rsrc_t rs =
+            __builtin_amdgcn_make_buffer_rsrc((void *)ld.a, 0, ld.a_bytes, kRsrcFlags);
+        stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(rs, ld_voff_a + (uint32_t)(32 * i) * ld.a_pitch,
+                                                                 ld_kt * 128, 0);
+      } else {
+        const bool up_half = SWIGLU && 32 * i >= kPBN / 2;  // wave * 8 + 7 < 32 never crosses the halves
+        const int row = up_half ? 32 * i - kPBN / 2 : 32 * i;
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(up_half ? ld.b1 : ld.b0), 0, ld.b_bytes, kRsrcFlags);
+        stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(rs, ld_voff_b + (uint32_t)row * ld.b_pitch,
+                                                                 ld_kt * 128, 0);
+      }
+    }
+  };
+  // Quarter q of register stage P into LDS slot P.
+  auto write_quarter = [&](auto stage_c, auto q_c) {
+    constexpr int P = decltype(stage_c)::value, Q = decltype(q_c)::value;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      constexpr int HALF_COPIES = kQCopies / 2;
+      const int l = Q * 4 + c, i = l % HALF_COPIES;
+      unsigned char *dst = lds_raw + P * kQSlotBytes + (l < HALF_COPIES ? 0 : kPBM * 128) + i * 32 * 128 + wr_off;
+      *reinterpret_cast<u32x4_any_t *>(dst) = stage_regs[P][l];
+    }
+  };
+  auto load_step = [&](auto stage_c) {
+    load_quarter(stage_c, c0); load_quarter(stage_c, c1); load_quarter(stage_c, c2); load_quarter(stage_c, c3);
+    advance_copy();
+  };
+  auto write_step = [&](auto stage_c) {
+    write_quarter(stage_c, c0); write_quarter(stage_c, c1); write_quarter(stage_c, c2); write_quarter(stage_c, c3);
+  };
+
+  // Prologue: steps 0 and 1 through the stages into the slots (of step 1 only
+  // the first quarter: the rest follows during step 0, as in the steady state),
+  // steps 2 and 3 into the stages behind them.
+  load_step(c0);           // step 0
+  load_step(c1);           // step 1
+  write_step(c0);
+  load_step(c0);           // step 2
+  write_quarter(c1, c0);
+  load_quarter(c1, c0);    // first quarter of step 3; the stage keeps quarters 1..3 of step 1
+  zero_acc();
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  phase_barrier();
+  read_frags(c0, c0, 0);
+  __builtin_amdgcn_sched_barrier(0);
+
+  const int stage_base = kQRingBytes + wave * Epi::WAVE_BYTES;
+  const int wave_col0 = SWIGLU ? wn * (WTN / 2) : wn * WTN;
+
+  while (true) {  // one tile per iteration
+    // Every tile has an even number of steps, so a tile always starts in slot 0.
+    auto step = [&](auto slot_c) {
+      constexpr int S = decltype(slot_c)::value;
+      const template_int<S ^ 1> other_c;
+      read_frags(slot_c, c1, 1);
+      write_quarter(other_c, c1);
+      load_quarter(other_c, c1);
+      mfma_block(0);
+      qsched_block<0, TM * TN, TM + TN, 4, 4>();
+      __builtin_amdgcn_sched_barrier(0);
+      read_frags(slot_c, c2, 0);
+      write_quarter(other_c, c2);
+      load_quarter(other_c, c2);
+      mfma_block(1);
+      qsched_block<0, TM * TN, TM + TN, 4, 4>();
+      __builtin_amdgcn_sched_barrier(0);
+      read_frags(slot_c, c3, 1);
+      write_quarter(other_c, c3);
+      load_quarter(other_c, c3);
+      mfma_block(0);
+      qsched_block<0, TM * TN, TM + TN, 4, 4>();
+      __builtin_amdgcn_sched_barrier(0);
+      advance_copy();
+      // This wave has read slot S for the last time and has finished writing the
+      // other slot; after the barrier both hold for every wave.
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      phase_barrier();
+      read_frags(other_c, c0, 0);
+      write_quarter(slot_c, c0);
+      load_quarter(slot_c, c0);
+      mfma_block(1);
+      qsched_block<0, TM * TN, TM + TN, 4, 4>();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    for (int s = 0; s < cp.steps; s += 2) {
+      step(c0);
+      step(c1);
+    }
+    tile_epilogue<MODE, HAS_BIAS, kQWaves, TM, TN>(cp, acc, lds_raw + stage_base, wm * WTM, wave_col0, lane);
+    // The load side is within the next tile here (every tile has at least
+    // kQMinSteps steps).
+    cp = ld;
+    if (!cp.valid) break;
+    nxt = pack_tile(decode(next_id), lane);
+    next_id += walk.wgs_per_xcd;
+    zero_acc();
+    // The last block above already fetched these fragments; reading them again
+    // here keeps 32 registers free during the epilogue.
+    read_frags(c0, c0, 0);
+  }
+}
+
+// The kernels are thin wrappers: builtins and inline assembly that only exist
+// for the device must not appear in a __global__ template's own body, or the
+// host pass silently drops its definition.
+template <int MODE, bool HAS_BIAS>
+__global__ __launch_bounds__(8 * kWave, 1) void gemm_persist_kernel8(PersistBatch batch) {
+  gemm_persist_body<MODE, HAS_BIAS, 8>(batch);
+}
+// Four waves, one per SIMD, each with the whole 512-entry register file.
+template <int MODE, bool HAS_BIAS>
+__global__ __launch_bounds__(4 * kWave, 1) void gemm_persist_kernel4(PersistBatch batch) {
+  gemm_persist64_body<MODE, HAS_BIAS>(batch);
+}
+
 }  // namespace
+
+int g_persist_waves = 4;  // tuning hook: 4 = 64-k register-staged pipeline, 8 = 32-k ping-pong pipeline
 
 bool persist_supported(const PersistBatch &b, int mode) {
   int groups = 0;
   for (int i = 0; i < b.n_problems; ++i) {
     const PersistProblem &p = b.prob[i];
     groups += p.n_experts;
-    if (p.k % kPBK != 0 || p.k < kPBK * (kPAhead + 1)) return false;
+    if (p.k % (kPBK * kPStages) != 0) return false;  // whole trips round the ring per tile
+    if (g_persist_waves == 4 && p.k < kQBK * kQMinSteps) return false;
     if (p.n % 8 != 0 || p.lda % 8 != 0 || p.ldc % 8 != 0) return false;
     if (mode == kFc1Swiglu && p.n % (kPBN / 2) != 0) return false;  // gate/up halves share one range check
     if ((size_t)kPBM * p.lda * 2 >= (1ull << 31) || (size_t)kPBN * p.k * 2 >= (1ull << 31)) return false;
@@ -488,14 +915,23 @@ int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s) 
   bool has_bias = false;
   for (int i = 0; i < b.n_problems; ++i) has_bias = has_bias || b.prob[i].bias != nullptr;
   if (mode == kFc1Swiglu) has_bias = false;
+  const int waves = g_persist_waves == 4 ? 4 : 8;
   void (*kern)(PersistBatch) = nullptr;
-  switch (mode) {
-    case kFc1Swiglu: kern = gemm_persist_kernel<kFc1Swiglu, false>; break;
-    case kFc1Gelu: kern = has_bias ? gemm_persist_kernel<kFc1Gelu, true> : gemm_persist_kernel<kFc1Gelu, false>; break;
-    default: kern = has_bias ? gemm_persist_kernel<kFc2, true> : gemm_persist_kernel<kFc2, false>; break;
+  if (waves == 4) {
+    switch (mode) {
+      case kFc1Swiglu: kern = gemm_persist_kernel4<kFc1Swiglu, false>; break;
+      case kFc1Gelu: kern = has_bias ? gemm_persist_kernel4<kFc1Gelu, true> : gemm_persist_kernel4<kFc1Gelu, false>; break;
+      default: kern = has_bias ? gemm_persist_kernel4<kFc2, true> : gemm_persist_kernel4<kFc2, false>; break;
+    }
+  } else {
+    switch (mode) {
+      case kFc1Swiglu: kern = gemm_persist_kernel8<kFc1Swiglu, false>; break;
+      case kFc1Gelu: kern = has_bias ? gemm_persist_kernel8<kFc1Gelu, true> : gemm_persist_kernel8<kFc1Gelu, false>; break;
+      default: kern = has_bias ? gemm_persist_kernel8<kFc2, true> : gemm_persist_kernel8<kFc2, false>; break;
+    }
   }
-  const int slot = mode * 2 + (has_bias ? 1 : 0);
-  static thread_local bool configured[6] = {false, false, false, false, false, false};
+  const int slot = (mode * 2 + (has_bias ? 1 : 0)) * 2 + (waves == 4 ? 1 : 0);
+  static thread_local bool configured[12] = {};
   if (!configured[slot]) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kPLdsBytes);
@@ -503,7 +939,7 @@ int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s) 
       return fail(DICE_ERR_LAUNCH, "persistent expert GEMM: LDS attribute: %s", hipGetErrorString(e));
     configured[slot] = true;
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kPWaves * kWave), kPLdsBytes, s, b);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(waves * kWave), kPLdsBytes, s, b);
   return launch_status("grouped_gemm_persist");
 }
 
