@@ -309,7 +309,7 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
   const int frag_row = lane & 31, frag_half = lane >> 5;
   const int rd_row = lane / G::LANES_PER_ROW, rd_chunk = lane % G::LANES_PER_ROW;
   const __amdgpu_buffer_rsrc_t crs =
-      __builtin_amdgcn_make_buffer_rsrc((void *)cp.c, 0, cp.c_bytes, kRsrcFlags);
+      __builtin_amdgcn_make_buffer_rsrc((void *)uni(cp.c), 0, uni(cp.c_bytes), kRsrcFlags);
   const int col_base = cp.n0 + wave_col0;
   // Bias of this lane's columns, fetched in one batch (one wait instead of one per element).
   float bias_v[OUT_BLOCKS][16];
@@ -647,17 +647,18 @@ __device__ __forceinline__ int qring_off(int row, int chunk) {
   return row * 128 + ((chunk ^ qswizzle(row)) << 4);
 }
 
-// Instruction order of one block of MF MFMAs: RD fragment reads behind the
-// first MFMAs (one each), then WR LDS writes and LD global loads, one behind
-// each of the following MFMAs.
-template <int I, int MF, int RD, int WR, int LD>
+// Instruction order of one block of 16 MFMAs: a fragment read behind every even
+// MFMA, LDS writes and global loads alternating behind the odd ones.  The LDS
+// takes 16 cycles per 16-byte-per-lane write against 4 per read, so the writes
+// of the four waves are spread over the whole block rather than bunched.
+template <int I>
 __device__ __forceinline__ void qsched_block() {
-  if constexpr (I < MF) {
+  if constexpr (I < 16) {
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    if constexpr (I < RD) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    else if constexpr (I < RD + WR) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-    else if constexpr (I < RD + WR + LD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-    qsched_block<I + 1, MF, RD, WR, LD>();
+    if constexpr (I % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    else if constexpr (I % 4 == 1) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+    else __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    qsched_block<I + 1>();
   }
 }
 
@@ -669,7 +670,12 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   using Epi = EpiGeom<MODE, kQWaves, TM, TN>;
   const template_int<0> c0; const template_int<1> c1; const template_int<2> c2; const template_int<3> c3;
 
-  extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
+  // Three separate LDS objects, so that the compiler knows that fragment reads of
+  // one slot and writes to the other never touch the same bytes and may pass
+  // each other when the instructions of a block are interleaved.
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_slot0[kQSlotBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_slot1[kQSlotBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_stage[kPStageArea];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
@@ -708,7 +714,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   bf16x8_t wf[2][TN], af[2][TM];
   auto read_frags = [&](auto slot_c, auto kk_c, int buf) {
     constexpr int SLOT = decltype(slot_c)::value, KK = decltype(kk_c)::value;
-    const unsigned char *base = lds_raw + SLOT * kQSlotBytes;
+    const unsigned char *base = SLOT == 0 ? lds_slot0 : lds_slot1;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       constexpr int HALF = TN / 2;
@@ -766,17 +772,19 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
       constexpr int HALF_COPIES = kQCopies / 2;
       const int l = Q * 4 + c, i = l % HALF_COPIES;
       if (l < HALF_COPIES) {
+        // (uni() costs nothing while the description sits in scalar registers and
+        // avoids a loop over lanes around the load if the compiler moved it out)
         const __amdgpu_buffer_rsrc_t rs =
-            __builtin_amdgcn_make_buffer_rsrc((void *)ld.a, 0, ld.a_bytes, kRsrcFlags);
-        stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(rs, ld_voff_a + (uint32_t)(32 * i) * ld.a_pitch,
-                                                                 ld_kt * 128, 0);
+            __builtin_amdgcn_make_buffer_rsrc((void *)uni(ld.a), 0, uni(ld.a_bytes), kRsrcFlags);
+        stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(
+            rs, ld_voff_a + (uint32_t)(32 * i) * uni(ld.a_pitch), uni(ld_kt * 128), 0);
       } else {
         const bool up_half = SWIGLU && 32 * i >= kPBN / 2;  // wave * 8 + 7 < 32 never crosses the halves
         const int row = up_half ? 32 * i - kPBN / 2 : 32 * i;
         const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)(up_half ? ld.b1 : ld.b0), 0, ld.b_bytes, kRsrcFlags);
-        stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(rs, ld_voff_b + (uint32_t)row * ld.b_pitch,
-                                                                 ld_kt * 128, 0);
+            (void *)uni(up_half ? ld.b1 : ld.b0), 0, uni(ld.b_bytes), kRsrcFlags);
+        stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(
+            rs, ld_voff_b + (uint32_t)row * uni(ld.b_pitch), uni(ld_kt * 128), 0);
       }
     }
   };
@@ -787,7 +795,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
     for (int c = 0; c < 4; ++c) {
       constexpr int HALF_COPIES = kQCopies / 2;
       const int l = Q * 4 + c, i = l % HALF_COPIES;
-      unsigned char *dst = lds_raw + P * kQSlotBytes + (l < HALF_COPIES ? 0 : kPBM * 128) + i * 32 * 128 + wr_off;
+      unsigned char *dst = (P == 0 ? lds_slot0 : lds_slot1) + (l < HALF_COPIES ? 0 : kPBM * 128) + i * 32 * 128 + wr_off;
       *reinterpret_cast<u32x4_any_t *>(dst) = stage_regs[P][l];
     }
   };
@@ -814,7 +822,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   read_frags(c0, c0, 0);
   __builtin_amdgcn_sched_barrier(0);
 
-  const int stage_base = kQRingBytes + wave * Epi::WAVE_BYTES;
+  unsigned char *const stage_rows = lds_stage + wave * Epi::WAVE_BYTES;
   const int wave_col0 = SWIGLU ? wn * (WTN / 2) : wn * WTN;
 
   while (true) {  // one tile per iteration
@@ -826,19 +834,19 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
       write_quarter(other_c, c1);
       load_quarter(other_c, c1);
       mfma_block(0);
-      qsched_block<0, TM * TN, TM + TN, 4, 4>();
+      qsched_block<0>();
       __builtin_amdgcn_sched_barrier(0);
       read_frags(slot_c, c2, 0);
       write_quarter(other_c, c2);
       load_quarter(other_c, c2);
       mfma_block(1);
-      qsched_block<0, TM * TN, TM + TN, 4, 4>();
+      qsched_block<0>();
       __builtin_amdgcn_sched_barrier(0);
       read_frags(slot_c, c3, 1);
       write_quarter(other_c, c3);
       load_quarter(other_c, c3);
       mfma_block(0);
-      qsched_block<0, TM * TN, TM + TN, 4, 4>();
+      qsched_block<0>();
       __builtin_amdgcn_sched_barrier(0);
       advance_copy();
       // This wave has read slot S for the last time and has finished writing the
@@ -849,14 +857,14 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
       write_quarter(slot_c, c0);
       load_quarter(slot_c, c0);
       mfma_block(1);
-      qsched_block<0, TM * TN, TM + TN, 4, 4>();
+      qsched_block<0>();
       __builtin_amdgcn_sched_barrier(0);
     };
     for (int s = 0; s < cp.steps; s += 2) {
       step(c0);
       step(c1);
     }
-    tile_epilogue<MODE, HAS_BIAS, kQWaves, TM, TN>(cp, acc, lds_raw + stage_base, wm * WTM, wave_col0, lane);
+    tile_epilogue<MODE, HAS_BIAS, kQWaves, TM, TN>(cp, acc, stage_rows, wm * WTM, wave_col0, lane);
     // The load side is within the next tile here (every tile has at least
     // kQMinSteps steps).
     cp = ld;
@@ -931,15 +939,18 @@ int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s) 
     }
   }
   const int slot = (mode * 2 + (has_bias ? 1 : 0)) * 2 + (waves == 4 ? 1 : 0);
+  // The 32-k kernel takes its 160 KB of LDS as dynamic memory (which needs the
+  // attribute once per kernel); the 64-k kernel declares its LDS statically.
+  const size_t dyn_lds = waves == 4 ? 0 : kPLdsBytes;
   static thread_local bool configured[12] = {};
-  if (!configured[slot]) {
+  if (dyn_lds != 0 && !configured[slot]) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kPLdsBytes);
     if (e != hipSuccess)
       return fail(DICE_ERR_LAUNCH, "persistent expert GEMM: LDS attribute: %s", hipGetErrorString(e));
     configured[slot] = true;
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(waves * kWave), kPLdsBytes, s, b);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(waves * kWave), dyn_lds, s, b);
   return launch_status("grouped_gemm_persist");
 }
 
