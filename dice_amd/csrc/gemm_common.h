@@ -132,6 +132,7 @@ struct PersistProblem {
   void *c;
   int ldc;
   int n, k;
+  int max_rows;            // host-side upper bound on the grouped rows (offsets live on the device)
 };
 constexpr int kMaxPersistProblems = 3;
 struct PersistBatch {

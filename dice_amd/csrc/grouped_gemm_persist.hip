@@ -141,6 +141,8 @@ struct Tile {
 struct PackedTile {
   uint32_t words;
 };
+constexpr int kTileWords = 20;   // pointers a, b0, b1, c, bias, then ten 32-bit fields
+constexpr int kTableTurns = 64;  // turns of one workgroup that the LDS tile table holds
 __device__ __forceinline__ PackedTile pack_tile(const Tile &t, int lane) {
   const uint64_t p[5] = {(uint64_t)t.a, (uint64_t)t.b0, (uint64_t)t.b1, (uint64_t)t.c, (uint64_t)t.bias};
   const uint32_t w[10] = {t.a_bytes, t.a_pitch, t.b_bytes, t.b_pitch, t.c_bytes,
@@ -175,15 +177,16 @@ __device__ __forceinline__ Tile unpack_tile(const PackedTile &pk) {
 // every wave describes group g = (problem, expert): its rows, its tile grid and
 // the index of its first tile (at most 64 groups); a tile id is mapped back to
 // its group with one ballot.  Tiles are ordered problem-major, expert-major,
-// then n-tile with the m-tile fastest.  XCD x (= blockIdx.x % 8) owns the x-th
-// eighth of that order and its workgroups take tiles of the run round-robin.
+// then n-tile with the m-tile fastest; callers list the problem with the longest
+// k first.  XCD x (= blockIdx.x % 8) owns the x-th eighth of that order and its
+// workgroups take tiles of the run in turns.
 template <int BN_OUT>
 struct TileWalker {
   int g_prob = 0, g_expert = 0, g_row0 = 0, g_cnt = 0, g_mt = 0, g_base = 0, g_end = 0;
   int run_begin, run_end, wg_in_xcd, wgs_per_xcd;
 
   __device__ __forceinline__ TileWalker(const PersistBatch &batch, int lane) {
-    int g_nt = 0, acc_groups = 0;
+    int g_nt = 0, g_k32 = 1, acc_groups = 0;
     for (int pi = 0; pi < batch.n_problems; ++pi) {
       const PersistProblem &pr = batch.prob[pi];
       const int local = lane - acc_groups;
@@ -194,31 +197,118 @@ struct TileWalker {
         g_cnt = pr.offsets[local + 1] - g_row0;
         g_mt = (g_cnt + kPBM - 1) / kPBM;
         g_nt = (pr.n + BN_OUT - 1) / BN_OUT;
+        g_k32 = pr.k / 32;
       }
       acc_groups += pr.n_experts;
     }
     const int tiles = g_mt * g_nt;
-    int inc = tiles;
+    // Inclusive scans over the groups: tile counts, and cost in units of 32 k
+    // (tiles of different problems differ in length).
+    const int cost = tiles * g_k32;
+    int inc = tiles, cinc = cost;
 #pragma unroll
     for (int o = 1; o < kWave; o <<= 1) {
-      const int up = __shfl_up(inc, o, kWave);
-      if (lane >= o) inc += up;
+      const int up = __shfl_up(inc, o, kWave), cup = __shfl_up(cinc, o, kWave);
+      if (lane >= o) {
+        inc += up;
+        cinc += cup;
+      }
     }
     g_base = inc - tiles;
     g_end = inc;
     const int total_tiles = __shfl(inc, kWave - 1, kWave);
-    const int per_xcd = (total_tiles + kNumXcd - 1) / kNumXcd;
+    const int total_cost = __shfl(cinc, kWave - 1, kWave);
+    // XCD x takes the tiles between the x-th and the (x+1)-th eighth of the total
+    // COST, so that every XCD gets the same amount of work whatever the mix.
     const int xcd = blockIdx.x % kNumXcd;
-    wg_in_xcd = blockIdx.x / kNumXcd;
-    wgs_per_xcd = gridDim.x / kNumXcd;
-    run_begin = xcd * per_xcd;
-    run_end = run_begin + per_xcd < total_tiles ? run_begin + per_xcd : total_tiles;
+    wg_in_xcd = uni((int)(blockIdx.x / kNumXcd));
+    wgs_per_xcd = uni((int)(gridDim.x / kNumXcd));
+    auto boundary = [&](int x) {
+      if (x >= kNumXcd) return total_tiles;
+      const int target = (int)((long long)total_cost * x / kNumXcd);
+      const uint64_t hit = __ballot(cost > 0 && target >= cinc - cost && target < cinc);
+      if (!hit) return total_tiles;
+      const int g = __builtin_ctzll(hit);
+      const int base = __builtin_amdgcn_readlane(g_base, g);
+      const int cbase = __builtin_amdgcn_readlane(cinc - cost, g);
+      const int k32 = __builtin_amdgcn_readlane(g_k32, g);
+      return base + (target - cbase + k32 / 2) / k32;
+    };
+    run_begin = uni(boundary(xcd));
+    run_end = uni(boundary(xcd + 1));
+  }
+
+  // Describes this workgroup's first 64 turns at once - lane r works out turn r -
+  // and leaves them in LDS, kTileWords dwords per turn in PackedTile order, so
+  // that a tile switch inside the kernel is a single LDS read.  Turns past the
+  // XCD's run give descriptions that cover no bytes.  Called by one wave.
+  __device__ __forceinline__ void build_table(const PersistBatch &batch, int lane, int bk,
+                                              uint32_t *table) const {
+    const int w = (lane & 1) ? wgs_per_xcd - 1 - wg_in_xcd : wg_in_xcd;
+    const int id = run_begin + lane * wgs_per_xcd + w;
+    const bool valid = id < run_end;
+    const int idc = valid ? id : 0;
+    int n_groups = 0;
+    for (int pi = 0; pi < batch.n_problems; ++pi) n_groups += batch.prob[pi].n_experts;
+    int grp = 0;
+    for (int g = 0; g < n_groups; ++g) {
+      const int b = __builtin_amdgcn_readlane(g_base, g), e = __builtin_amdgcn_readlane(g_end, g);
+      grp = (idc >= b && idc < e) ? g : grp;
+    }
+    const int pi = __shfl(g_prob, grp, kWave), expert = __shfl(g_expert, grp, kWave);
+    const int row0 = __shfl(g_row0, grp, kWave), cnt = __shfl(g_cnt, grp, kWave);
+    const int mt = __shfl(g_mt, grp, kWave), base = __shfl(g_base, grp, kWave);
+    // this lane's problem (a handful of selects instead of a divergent struct index)
+    uint64_t pa = 0, pw = 0, pc = 0, pbias = 0;
+    int lda = 0, ldc = 0, w_rows = 0, up_offset = 0, n = 0, k = 0;
+    for (int q = 0; q < batch.n_problems; ++q) {
+      const PersistProblem &pr = batch.prob[q];
+      if (pi == q) {
+        pa = (uint64_t)pr.a; pw = (uint64_t)pr.w; pc = (uint64_t)pr.c; pbias = (uint64_t)pr.bias;
+        lda = pr.lda; ldc = pr.ldc; w_rows = pr.w_rows; up_offset = pr.up_offset; n = pr.n; k = pr.k;
+      }
+    }
+    const int r = idc - base;
+    const int n_tile = mt > 0 ? r / mt : 0;
+    const int m_tile = r - n_tile * mt;
+    const int left = cnt - m_tile * kPBM;
+    const int rows = left < kPBM ? left : kPBM;
+    const int n0 = n_tile * BN_OUT;
+    const int cols_left = n - n0;
+    const int wrows = cols_left < BN_OUT ? cols_left : BN_OUT;
+    const uint32_t a_pitch = (uint32_t)lda * 2, b_pitch = (uint32_t)k * 2, c_pitch = (uint32_t)ldc * 2;
+    const uint64_t wexp = pw + (uint64_t)expert * w_rows * b_pitch;
+    const uint64_t ptrs[5] = {pa + (uint64_t)(row0 + m_tile * kPBM) * a_pitch, wexp + (uint64_t)n0 * b_pitch,
+                              wexp + (uint64_t)(up_offset + n0) * b_pitch,
+                              pc + (uint64_t)(row0 + m_tile * kPBM) * c_pitch,
+                              pbias ? pbias + ((uint64_t)expert * n) * sizeof(float) : 0};
+    const uint32_t words[10] = {valid ? (uint32_t)rows * a_pitch : 0u, a_pitch, valid ? (uint32_t)wrows * b_pitch : 0u,
+                                b_pitch, (uint32_t)rows * c_pitch, c_pitch, (uint32_t)n0, (uint32_t)n,
+                                (uint32_t)(k / bk), valid ? 1u : 0u};
+    uint32_t *entry = table + lane * kTileWords;
+#pragma unroll
+    for (int i = 0; i < 5; ++i) {
+      entry[2 * i] = (uint32_t)ptrs[i];
+      entry[2 * i + 1] = (uint32_t)(ptrs[i] >> 32);
+    }
+#pragma unroll
+    for (int i = 0; i < 10; ++i) entry[10 + i] = words[i];
+  }
+
+  // The id of the tile this workgroup takes in its `round`-th turn.  Turns
+  // alternate direction over the XCD's workgroups (0..W-1, W-1..0, ...): the
+  // order runs from the longest tiles to the shortest, so the workgroups that got
+  // the last long tiles get the fewest short ones.
+  __device__ __forceinline__ int tile_id(int round) const {
+    const int w = (round & 1) ? wgs_per_xcd - 1 - wg_in_xcd : wg_in_xcd;
+    return uni(run_begin + round * wgs_per_xcd + w);
   }
 
   // Tile `id` of the order (ids past this XCD's run give an invalid tile whose
   // descriptors cover no bytes); `bk` is the k extent of one pipeline step.
   __device__ __forceinline__ Tile decode(const PersistBatch &batch, int id, int bk) const {
     Tile t;
+    id = uni(id);  // wave-uniform by construction; says so to the compiler (scalar arithmetic below)
     t.valid = id < run_end;
     const int idc = t.valid ? id : 0;
     const uint64_t hit = __ballot(idc >= g_base && idc < g_end);
@@ -273,27 +363,25 @@ struct EpiGeom {
   static constexpr int PITCH = OUT_COLS * 2 + 16;
   static constexpr int BAND = (WAVES * 32 * PITCH <= kPStageArea) ? 32 : 16;  // rows staged at a time
   static constexpr int LANES_PER_ROW = OUT_COLS * 2 / 16;
-  static constexpr int ROWS_PER_PASS = kWave / LANES_PER_ROW;
-  static constexpr int PASSES = BAND / ROWS_PER_PASS;
+  static constexpr int ROWS_PER_PASS = kWave / LANES_PER_ROW;   // lanes past ROWS_PER_PASS rows idle
+  static constexpr int PASSES = (BAND + ROWS_PER_PASS - 1) / ROWS_PER_PASS;
+  static constexpr bool EXACT = kWave % LANES_PER_ROW == 0 && BAND % ROWS_PER_PASS == 0;
   static constexpr int STORES = (TM * 32 / BAND) * PASSES;  // buffer stores per wave per tile
   static constexpr int WAVE_BYTES = BAND * PITCH;
   static_assert(WAVES * WAVE_BYTES <= kPStageArea, "staging area too small");
   static_assert(PASSES >= 1, "band smaller than one store pass");
 };
 
-// One accumulator element for the epilogue's arithmetic.  With four waves the
+// One 32x32 accumulator block for the epilogue's arithmetic.  With four waves the
 // accumulators live in the accumulation registers; left to itself the compiler
-// copies whole 16-register blocks out at the top of the epilogue and then spills
-// them, so the read is pinned to the place where the value is used.
+// copies all of them out at the top of the epilogue and then spills, so the block
+// is pulled into vector registers at the place where it is used (the empty asm
+// statement demands a vector-register operand and cannot be moved).
 template <bool FROM_ACC_REGS>
-__device__ __forceinline__ float acc_value(const float &a) {
-  if constexpr (FROM_ACC_REGS) {
-    float v;
-    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
-    return v;
-  } else {
-    return a;
-  }
+__device__ __forceinline__ f32x16_t acc_block(const f32x16_t &a) {
+  f32x16_t t = a;
+  if constexpr (FROM_ACC_REGS) asm volatile("" : "+v"(t));
+  return t;
 }
 
 // Epilogue of tile `cp` for one wave: activation (and bias), transposition through
@@ -336,15 +424,18 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
       const int srow = BAND == 32 ? frag_row : (frag_row & 15);
 #pragma unroll
       for (int j = 0; j < OUT_BLOCKS; ++j) {
+        const f32x16_t blk = acc_block<WAVES == 4>(acc[i][j]);
+        f32x16_t up;
+        if (SWIGLU) up = acc_block<WAVES == 4>(acc[i][j + OUT_BLOCKS]);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int col = j * 32 + frag_half * 4 + q * 8;
           bf16x4_t o;
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            float v = acc_value<WAVES == 4>(acc[i][j][q * 4 + r]);
+            float v = blk[q * 4 + r];
             if (SWIGLU) {
-              v = silu_fast(v) * acc_value<WAVES == 4>(acc[i][j + OUT_BLOCKS][q * 4 + r]);
+              v = silu_fast(v) * up[q * 4 + r];
             } else {
               if (HAS_BIAS) v += bias_v[j][q * 4 + r];
               if (MODE == kFc1Gelu) v = gelu_tanh_fast(v);
@@ -358,11 +449,16 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
     wave_lds_sync();
 #pragma unroll
     for (int ps = 0; ps < G::PASSES; ++ps) {
-      const int r = ps * G::ROWS_PER_PASS + rd_row;
+      int r = ps * G::ROWS_PER_PASS + rd_row;
+      bool live = true;
+      if (!G::EXACT) {
+        live = rd_row < G::ROWS_PER_PASS && r < BAND;
+        r = live ? r : 0;
+      }
       const u32x4_t v = *reinterpret_cast<const u32x4_any_t *>(stage + r * PITCH + rd_chunk * 16);
       const int m = wave_row0 + band * BAND + r;
       const int n = col_base + rd_chunk * 8;
-      const uint32_t voff = n < cp.n ? (uint32_t)m * cp.c_pitch + (uint32_t)n * 2 : kOutOfRange;
+      const uint32_t voff = (live && n < cp.n) ? (uint32_t)m * cp.c_pitch + (uint32_t)n * 2 : kOutOfRange;
       __builtin_amdgcn_raw_buffer_store_b128(v, crs, voff, 0, 0);
     }
     wave_lds_sync();  // the next band overwrites the staging rows
@@ -396,7 +492,6 @@ __device__ __forceinline__ void gemm_persist_body(const PersistBatch &batch) {
   const int wm = wave / kPWavesN, wn = wave % kPWavesN;
 
   TileWalker<BN_OUT> walk(batch, lane);
-  const int run_begin = walk.run_begin, wg_in_xcd = walk.wg_in_xcd, wgs_per_xcd = walk.wgs_per_xcd;
   auto decode = [&](int id) { return walk.decode(batch, id, kPBK); };
 
   // ---- per-lane copy offsets (row part depends on the tile's pitch) ----
@@ -496,9 +591,8 @@ __device__ __forceinline__ void gemm_persist_body(const PersistBatch &batch) {
   };
 
   // ---- pipeline state ----
-  int next_id = run_begin + wg_in_xcd;           // next tile the copy side will open
-  Tile ld = decode(next_id);                     // tile being copied
-  next_id += wgs_per_xcd;
+  int next_round = 0;                            // this workgroup's next turn
+  Tile ld = decode(walk.tile_id(next_round++));  // tile being copied
   if (!ld.valid) return;                         // nothing to do for this workgroup
   Tile cp = ld;                                  // tile being multiplied
   int ld_kt = 0;
@@ -506,9 +600,8 @@ __device__ __forceinline__ void gemm_persist_body(const PersistBatch &batch) {
   // Advances the copy side by one step (wave-uniform control flow only).
   auto advance_copy = [&]() {
     if (++ld_kt == ld.steps) {
-      ld = decode(next_id);
+      ld = decode(walk.tile_id(next_round++));
       set_copy_offsets(ld);
-      next_id += wgs_per_xcd;
       ld_kt = 0;
     }
   };
@@ -635,10 +728,8 @@ constexpr int kQBK = 64;
 constexpr int kQWaves = 4;
 constexpr int kQSlotBytes = (kPBM + kPBN) * 128;   // 64 KB
 constexpr int kQRingBytes = 2 * kQSlotBytes;       // staging area follows
-constexpr int kQCopies = (kPBM + kPBN) / 8 / kQWaves;  // 16-byte-per-lane loads (8 rows each) per wave per step
 constexpr int kQMinSteps = 6;                      // loads run four steps ahead, within the next tile
 static_assert(kQRingBytes == kPRingBytes, "both pipelines share the LDS budget");
-static_assert(kQCopies == 16, "a step is four quarters of four loads");
 
 __device__ __forceinline__ int qswizzle(int row) { return (row >> 1) & 7; }
 // Byte offset of 16-byte chunk `chunk` (0..7) of `row` inside a slot half: any
@@ -647,26 +738,35 @@ __device__ __forceinline__ int qring_off(int row, int chunk) {
   return row * 128 + ((chunk ^ qswizzle(row)) << 4);
 }
 
-// Instruction order of one block of 16 MFMAs: a fragment read behind every even
-// MFMA, LDS writes and global loads alternating behind the odd ones.  The LDS
-// takes 16 cycles per 16-byte-per-lane write against 4 per read, so the writes
-// of the four waves are spread over the whole block rather than bunched.
-template <int I>
+// Instruction order of one block of MF MFMAs: RD fragment reads, 4 LDS writes
+// and 4 global loads spread evenly behind the MFMAs (reads from the first MFMA
+// on, writes and loads offset against each other).  The LDS takes 16 cycles per
+// 16-byte-per-lane write against 4 per read, so the writes of the four waves are
+// spread over the whole block rather than bunched.
+template <int I, int MF, int RD>
 __device__ __forceinline__ void qsched_block() {
-  if constexpr (I < 16) {
+  if constexpr (I < MF) {
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    if constexpr (I % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    else if constexpr (I % 4 == 1) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-    else __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-    qsched_block<I + 1>();
+    constexpr int reads = (I + 1) * RD / MF - I * RD / MF;
+    if constexpr (reads > 0) __builtin_amdgcn_sched_group_barrier(0x100, reads, 0);
+    constexpr int Q = MF / 4;  // one write and one load per quarter of the block
+    if constexpr (I % Q == Q / 4) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+    if constexpr (I % Q == Q / 4 + Q / 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    qsched_block<I + 1, MF, RD>();
   }
 }
 
-template <int MODE, bool HAS_BIAS>
+// BN is the number of weight rows of a tile: 256, or 192 for output widths that
+// 192 divides and 256 does not (1152 = 6 x 192: no padded columns to multiply).
+template <int MODE, bool HAS_BIAS, int BN>
 __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   constexpr bool SWIGLU = MODE == kFc1Swiglu;
-  constexpr int BN_OUT = SWIGLU ? kPBN / 2 : kPBN;
-  constexpr int WTM = 128, WTN = 128, TM = 4, TN = 4;
+  static_assert(BN == 256 || (BN == 192 && !SWIGLU), "tile widths");
+  constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
+  constexpr int WTM = 128, WTN = BN / 2, TM = 4, TN = WTN / 32;
+  constexpr int kCopiesA = kPBM / 8 / kQWaves, kCopiesB = BN / 8 / kQWaves;  // 16-byte-per-lane loads, 8 rows each
+  constexpr int kQCopies = kCopiesA + kCopiesB;
+  static_assert(kCopiesA % 2 == 0 && kCopiesB % 2 == 0, "a step is four quarters: two of A, two of B");
   using Epi = EpiGeom<MODE, kQWaves, TM, TN>;
   const template_int<0> c0; const template_int<1> c1; const template_int<2> c2; const template_int<3> c3;
 
@@ -680,8 +780,19 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
 
-  TileWalker<BN_OUT> walk(batch, lane);
-  auto decode = [&](int id) { return walk.decode(batch, id, kQBK); };
+  // This workgroup's tiles, described once and parked in LDS behind the epilogue's
+  // staging rows; lane f of a table read gets word f of the description.
+  static_assert(kQWaves * Epi::WAVE_BYTES + kTableTurns * kTileWords * 4 <= kPStageArea, "no room for the tile table");
+  uint32_t *const tile_table = reinterpret_cast<uint32_t *>(lds_stage + kPStageArea - kTableTurns * kTileWords * 4);
+  if (wave == 0) {
+    TileWalker<BN_OUT> walk(batch, lane);
+    walk.build_table(batch, lane, kQBK, tile_table);
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  phase_barrier();
+  auto fetch_tile = [&](int turn) {
+    return PackedTile{tile_table[turn * kTileWords + (lane < kTileWords ? lane : 0)]};
+  };
 
   // ---- global loads: one instruction fetches 8 rows x 128 bytes (8 lanes per
   // row, i.e. whole lines); load l of a wave covers rows (wave + 4 (l % 8)) * 8
@@ -718,7 +829,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       constexpr int HALF = TN / 2;
-      const int jrow = (SWIGLU && j >= HALF) ? kPBN / 2 + (j - HALF) * 32 : j * 32;
+      const int jrow = (SWIGLU && j >= HALF) ? BN / 2 + (j - HALF) * 32 : j * 32;
       wf[buf][j] = *reinterpret_cast<const bf16x8_t *>(base + rd_b[KK] + jrow * 128);
     }
 #pragma unroll
@@ -747,12 +858,10 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   // The load side runs four steps ahead of the MFMAs, so it crosses into the
   // next tile once while a tile is multiplied.  That tile's description (`nxt`)
   // is worked out between tiles, where registers are free, not inside the k loop.
-  int next_id = walk.run_begin + walk.wg_in_xcd;
-  Tile ld = decode(next_id);                      // tile being loaded
-  next_id += walk.wgs_per_xcd;
+  int next_turn = 0;                              // this workgroup's next turn
+  Tile ld = unpack_tile(fetch_tile(next_turn++));  // tile being loaded
   if (!ld.valid) return;                          // nothing to do for this workgroup
-  PackedTile nxt = pack_tile(decode(next_id), lane);    // the one the load side opens next
-  next_id += walk.wgs_per_xcd;
+  PackedTile nxt = fetch_tile(next_turn++);       // the one the load side opens next
   Tile cp = ld;                                   // tile being multiplied
   int ld_kt = 0;
   set_copy_offsets(ld);
@@ -763,15 +872,17 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
       ld_kt = 0;
     }
   };
-  // Quarter q (loads 4 q .. 4 q + 3) of the step the load side stands at, into
-  // register stage P.
+  // A step's loads in four quarters: the two halves of the activation rows, then
+  // the two halves of the weight rows.  first(q) .. first(q + 1) are quarter q's
+  // indices into the register stage.
+  auto quarter_first = [](int q) { return q <= 2 ? q * (kCopiesA / 2) : kCopiesA + kCopiesB / 2; };
+  // Quarter q of the step the load side stands at, into register stage P.
   auto load_quarter = [&](auto stage_c, auto q_c) {
     constexpr int P = decltype(stage_c)::value, Q = decltype(q_c)::value;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      constexpr int HALF_COPIES = kQCopies / 2;
-      const int l = Q * 4 + c, i = l % HALF_COPIES;
-      if (l < HALF_COPIES) {
+    for (int l = quarter_first(Q); l < (Q == 3 ? kQCopies : quarter_first(Q + 1)); ++l) {
+      if (l < kCopiesA) {
+        const int i = l;
         // (uni() costs nothing while the description sits in scalar registers and
         // avoids a loop over lanes around the load if the compiler moved it out)
         const __amdgpu_buffer_rsrc_t rs =
@@ -779,8 +890,9 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
         stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(
             rs, ld_voff_a + (uint32_t)(32 * i) * uni(ld.a_pitch), uni(ld_kt * 128), 0);
       } else {
-        const bool up_half = SWIGLU && 32 * i >= kPBN / 2;  // wave * 8 + 7 < 32 never crosses the halves
-        const int row = up_half ? 32 * i - kPBN / 2 : 32 * i;
+        const int i = l - kCopiesA;
+        const bool up_half = SWIGLU && 32 * i >= BN / 2;  // wave * 8 + 7 < 32 never crosses the halves
+        const int row = up_half ? 32 * i - BN / 2 : 32 * i;
         const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
             (void *)uni(up_half ? ld.b1 : ld.b0), 0, uni(ld.b_bytes), kRsrcFlags);
         stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(
@@ -792,10 +904,9 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   auto write_quarter = [&](auto stage_c, auto q_c) {
     constexpr int P = decltype(stage_c)::value, Q = decltype(q_c)::value;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      constexpr int HALF_COPIES = kQCopies / 2;
-      const int l = Q * 4 + c, i = l % HALF_COPIES;
-      unsigned char *dst = (P == 0 ? lds_slot0 : lds_slot1) + (l < HALF_COPIES ? 0 : kPBM * 128) + i * 32 * 128 + wr_off;
+    for (int l = quarter_first(Q); l < (Q == 3 ? kQCopies : quarter_first(Q + 1)); ++l) {
+      const int i = l < kCopiesA ? l : l - kCopiesA;
+      unsigned char *dst = (P == 0 ? lds_slot0 : lds_slot1) + (l < kCopiesA ? 0 : kPBM * 128) + i * 32 * 128 + wr_off;
       *reinterpret_cast<u32x4_any_t *>(dst) = stage_regs[P][l];
     }
   };
@@ -834,19 +945,19 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
       write_quarter(other_c, c1);
       load_quarter(other_c, c1);
       mfma_block(0);
-      qsched_block<0>();
+      qsched_block<0, TM * TN, TM + TN>();
       __builtin_amdgcn_sched_barrier(0);
       read_frags(slot_c, c2, 0);
       write_quarter(other_c, c2);
       load_quarter(other_c, c2);
       mfma_block(1);
-      qsched_block<0>();
+      qsched_block<0, TM * TN, TM + TN>();
       __builtin_amdgcn_sched_barrier(0);
       read_frags(slot_c, c3, 1);
       write_quarter(other_c, c3);
       load_quarter(other_c, c3);
       mfma_block(0);
-      qsched_block<0>();
+      qsched_block<0, TM * TN, TM + TN>();
       __builtin_amdgcn_sched_barrier(0);
       advance_copy();
       // This wave has read slot S for the last time and has finished writing the
@@ -857,7 +968,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
       write_quarter(slot_c, c0);
       load_quarter(slot_c, c0);
       mfma_block(1);
-      qsched_block<0>();
+      qsched_block<0, TM * TN, TM + TN>();
       __builtin_amdgcn_sched_barrier(0);
     };
     for (int s = 0; s < cp.steps; s += 2) {
@@ -869,8 +980,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
     // kQMinSteps steps).
     cp = ld;
     if (!cp.valid) break;
-    nxt = pack_tile(decode(next_id), lane);
-    next_id += walk.wgs_per_xcd;
+    nxt = fetch_tile(next_turn++);
     zero_acc();
     // The last block above already fetched these fragments; reading them again
     // here keeps 32 registers free during the epilogue.
@@ -886,9 +996,9 @@ __global__ __launch_bounds__(8 * kWave, 1) void gemm_persist_kernel8(PersistBatc
   gemm_persist_body<MODE, HAS_BIAS, 8>(batch);
 }
 // Four waves, one per SIMD, each with the whole 512-entry register file.
-template <int MODE, bool HAS_BIAS>
+template <int MODE, bool HAS_BIAS, int BN>
 __global__ __launch_bounds__(4 * kWave, 1) void gemm_persist_kernel4(PersistBatch batch) {
-  gemm_persist64_body<MODE, HAS_BIAS>(batch);
+  gemm_persist64_body<MODE, HAS_BIAS, BN>(batch);
 }
 
 }  // namespace
@@ -925,11 +1035,20 @@ int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s) 
   if (mode == kFc1Swiglu) has_bias = false;
   const int waves = g_persist_waves == 4 ? 4 : 8;
   void (*kern)(PersistBatch) = nullptr;
-  if (waves == 4) {
+  // 192-row weight tiles where they avoid padded columns (n = 1152 = 6 x 192).
+  bool narrow = mode != kFc1Swiglu;
+  for (int i = 0; i < b.n_problems; ++i)
+    narrow = narrow && b.prob[i].n % 192 == 0 && b.prob[i].n % 256 != 0;
+  if (waves == 4 && narrow) {
     switch (mode) {
-      case kFc1Swiglu: kern = gemm_persist_kernel4<kFc1Swiglu, false>; break;
-      case kFc1Gelu: kern = has_bias ? gemm_persist_kernel4<kFc1Gelu, true> : gemm_persist_kernel4<kFc1Gelu, false>; break;
-      default: kern = has_bias ? gemm_persist_kernel4<kFc2, true> : gemm_persist_kernel4<kFc2, false>; break;
+      case kFc1Gelu: kern = has_bias ? gemm_persist_kernel4<kFc1Gelu, true, 192> : gemm_persist_kernel4<kFc1Gelu, false, 192>; break;
+      default: kern = has_bias ? gemm_persist_kernel4<kFc2, true, 192> : gemm_persist_kernel4<kFc2, false, 192>; break;
+    }
+  } else if (waves == 4) {
+    switch (mode) {
+      case kFc1Swiglu: kern = gemm_persist_kernel4<kFc1Swiglu, false, 256>; break;
+      case kFc1Gelu: kern = has_bias ? gemm_persist_kernel4<kFc1Gelu, true, 256> : gemm_persist_kernel4<kFc1Gelu, false, 256>; break;
+      default: kern = has_bias ? gemm_persist_kernel4<kFc2, true, 256> : gemm_persist_kernel4<kFc2, false, 256>; break;
     }
   } else {
     switch (mode) {

@@ -135,11 +135,11 @@ int grouped_mlp_impl(int stages, const void *x, int act_dtype, const int32_t *pe
     PersistBatch pb1{};
     pb1.n_problems = 1;
     pb1.prob[0] = PersistProblem{x, hidden, offsets, n_experts, w1, swiglu ? 2 * inter : inter, inter,
-                                 swiglu ? nullptr : b1, h, inter, inter, hidden};
+                                 swiglu ? nullptr : b1, h, inter, inter, hidden, (int)max_rows};
     PersistBatch pb2{};
     pb2.n_problems = 1;
     pb2.prob[0] = PersistProblem{h, inter, offsets, n_experts, w2, hidden, 0, swiglu ? nullptr : b2,
-                                 out, hidden, hidden, inter};
+                                 out, hidden, hidden, inter, (int)max_rows};
     const int m1 = swiglu ? kFc1Swiglu : kFc1Gelu;
     if (persist_supported(pb1, m1) && persist_supported(pb2, kFc2)) {
       if (stages & 1) {
@@ -289,16 +289,16 @@ extern "C" int dice_moe_forward(const dice_moe_layer_t *L, const void *x, int64_
     void *xg = w.slot_out;  // the gathered rows die before fc2 writes its outputs there
     f1.prob[0] = PersistProblem{xg, L->hidden, w.offsets, L->n_experts, L->w1,
                                 swiglu ? 2 * L->inter : L->inter, L->inter, swiglu ? nullptr : L->b1,
-                                w.h, L->inter, L->inter, L->hidden};
+                                w.h, L->inter, L->inter, L->hidden, (int)max_rows};
     f2.prob[0] = PersistProblem{w.h, L->inter, w.offsets, L->n_experts, L->w2, L->hidden, 0,
-                                swiglu ? nullptr : L->b2, w.slot_out, L->hidden, L->hidden, L->inter};
+                                swiglu ? nullptr : L->b2, w.slot_out, L->hidden, L->hidden, L->inter, (int)max_rows};
     f1.n_problems = f2.n_problems = 1;
     if (L->shared_inter > 0) {
       const int si = L->shared_inter;
       f1.prob[1] = PersistProblem{x, L->hidden, w.shared_offsets, 1, L->shared_w1, swiglu ? 2 * si : si, si,
-                                  swiglu ? nullptr : L->shared_b1, w.shared_h, si, si, L->hidden};
+                                  swiglu ? nullptr : L->shared_b1, w.shared_h, si, si, L->hidden, (int)n_tokens};
       f2.prob[1] = PersistProblem{w.shared_h, si, w.shared_offsets, 1, L->shared_w2, L->hidden, 0,
-                                  swiglu ? nullptr : L->shared_b2, w.shared_out, L->hidden, L->hidden, si};
+                                  swiglu ? nullptr : L->shared_b2, w.shared_out, L->hidden, L->hidden, si, (int)n_tokens};
       f1.n_problems = f2.n_problems = 2;
     }
     if (persist_supported(f1, m1) && persist_supported(f2, kFc2)) {
