@@ -210,9 +210,10 @@ def main():
         out["stage_ms"] = st
         bf = 2
         slots = N_TOKENS * TOPK
+        # (the row gather is part of the fc1 kernel's loads on this path: "moe.gather" only
+        # shows the timer's own overhead)
         hbm = {"moe.gate": N_TOKENS * D * bf + slots * 8,
                "moe.dispatch": slots * 12,
-               "moe.gather": (N_TOKENS + slots) * D * bf,
                "moe.combine": (slots * D + 2 * N_TOKENS * D) * bf + slots * 8}
         out["hbm_stage_gbs"] = {s: hbm[s] / (st[s] * 1e-3) / 1e9 for s in hbm}
         out["hbm_stage_frac_of_peak"] = {s: v / PEAK_HBM_GBS for s, v in out["hbm_stage_gbs"].items()}

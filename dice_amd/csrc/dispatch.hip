@@ -100,8 +100,13 @@ template <int MAXR>
 __global__ __launch_bounds__(kFusedWaves *kWave) void dispatch_fused_kernel(
     const int32_t *__restrict__ idx, const uint8_t *__restrict__ skip, int64_t n_slots,
     int n_experts, int nbits, int rounds, int32_t *__restrict__ counts,
-    int32_t *__restrict__ offsets, int32_t *__restrict__ perm, int32_t *__restrict__ inv_perm) {
+    int32_t *__restrict__ offsets, int32_t *__restrict__ perm, int32_t *__restrict__ inv_perm,
+    int32_t *__restrict__ range_out, int32_t range_n) {
   __shared__ volatile int32_t wrow[kFusedWaves][kMaxExperts];
+  if (range_out && threadIdx.x == 0) {
+    range_out[0] = 0;
+    range_out[1] = range_n;
+  }
   __shared__ int32_t eoff[kMaxExperts + 1];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
@@ -216,8 +221,14 @@ __global__ __launch_bounds__(kTileWaves *kWave) void dispatch_count_kernel(
 __global__ __launch_bounds__(1024) void dispatch_scan_kernel(int32_t *__restrict__ unit_cnt,
                                                              int n_experts, int units,
                                                              int32_t *__restrict__ counts,
-                                                             int32_t *__restrict__ offsets) {
+                                                             int32_t *__restrict__ offsets,
+                                                             int32_t *__restrict__ range_out,
+                                                             int32_t range_n) {
   __shared__ int32_t wave_tot[16];
+  if (range_out && threadIdx.x == 0) {
+    range_out[0] = 0;
+    range_out[1] = range_n;
+  }
   __shared__ int32_t eoff[kMaxExperts + 1];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
@@ -311,11 +322,12 @@ extern "C" size_t dice_dispatch_workspace_bytes(int64_t n_slots, int n_experts) 
   return align_up((size_t)units * n_experts * sizeof(int32_t), 256);
 }
 
-extern "C" int dice_dispatch(const int32_t *flat_idx, const uint8_t *skip_mask, int64_t n_slots,
-                             int n_experts, int32_t *counts, int32_t *offsets, int32_t *perm,
-                             int32_t *inv_perm, void *workspace, size_t workspace_bytes,
-                             void *stream) {
-  using namespace dice;
+namespace dice {
+// `range_out` (optional) receives {0, range_n}: the one-group offset table of
+// the shared expert, written here so that the layer needs no extra launch for it.
+int dispatch_impl(const int32_t *flat_idx, const uint8_t *skip_mask, int64_t n_slots, int n_experts,
+                  int32_t *counts, int32_t *offsets, int32_t *perm, int32_t *inv_perm, void *workspace,
+                  size_t workspace_bytes, int32_t *range_out, int32_t range_n, void *stream) {
   DICE_REQUIRE(counts && offsets && (n_slots == 0 || (flat_idx && perm && inv_perm)),
                DICE_ERR_BAD_ARG, "dice_dispatch: null pointer");
   DICE_REQUIRE(n_experts >= 1 && n_experts <= kMaxExperts, DICE_ERR_UNSUPPORTED,
@@ -328,13 +340,13 @@ extern "C" int dice_dispatch(const int32_t *flat_idx, const uint8_t *skip_mask, 
     int rounds = (int)((n_slots + kFusedWaves * kWave - 1) / (kFusedWaves * kWave));
     if (rounds <= 16)
       hipLaunchKernelGGL(dispatch_fused_kernel<16>, dim3(1), dim3(kFusedWaves * kWave), 0, s, flat_idx,
-                         skip_mask, n_slots, n_experts, nbits, rounds, counts, offsets, perm, inv_perm);
+                         skip_mask, n_slots, n_experts, nbits, rounds, counts, offsets, perm, inv_perm, range_out, range_n);
     else if (rounds <= 32)
       hipLaunchKernelGGL(dispatch_fused_kernel<32>, dim3(1), dim3(kFusedWaves * kWave), 0, s, flat_idx,
-                         skip_mask, n_slots, n_experts, nbits, rounds, counts, offsets, perm, inv_perm);
+                         skip_mask, n_slots, n_experts, nbits, rounds, counts, offsets, perm, inv_perm, range_out, range_n);
     else
       hipLaunchKernelGGL(dispatch_fused_kernel<64>, dim3(1), dim3(kFusedWaves * kWave), 0, s, flat_idx,
-                         skip_mask, n_slots, n_experts, nbits, rounds, counts, offsets, perm, inv_perm);
+                         skip_mask, n_slots, n_experts, nbits, rounds, counts, offsets, perm, inv_perm, range_out, range_n);
     return launch_status("dice_dispatch");
   }
   const int64_t units64 = (n_slots + kTileRounds * kWave - 1) / (kTileRounds * kWave);
@@ -347,10 +359,19 @@ extern "C" int dice_dispatch(const int32_t *flat_idx, const uint8_t *skip_mask, 
   hipLaunchKernelGGL(dispatch_count_kernel, dim3(blocks), dim3(kTileWaves * kWave), 0, s, flat_idx,
                      skip_mask, n_slots, n_experts, nbits, units, unit_cnt);
   hipLaunchKernelGGL(dispatch_scan_kernel, dim3(1), dim3(1024), 0, s, unit_cnt, n_experts, units,
-                     counts, offsets);
+                     counts, offsets, range_out, range_n);
   hipLaunchKernelGGL(dispatch_rank_kernel, dim3(blocks), dim3(kTileWaves * kWave), 0, s, flat_idx,
                      skip_mask, n_slots, n_experts, nbits, units, unit_cnt, offsets, perm, inv_perm);
   return launch_status("dice_dispatch");
+}
+}  // namespace dice
+
+extern "C" int dice_dispatch(const int32_t *flat_idx, const uint8_t *skip_mask, int64_t n_slots,
+                             int n_experts, int32_t *counts, int32_t *offsets, int32_t *perm,
+                             int32_t *inv_perm, void *workspace, size_t workspace_bytes,
+                             void *stream) {
+  return dice::dispatch_impl(flat_idx, skip_mask, n_slots, n_experts, counts, offsets, perm, inv_perm,
+                             workspace, workspace_bytes, nullptr, 0, stream);
 }
 
 namespace dice {

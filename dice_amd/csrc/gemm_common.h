@@ -117,9 +117,10 @@ __device__ __forceinline__ float gelu_tanh_fast(float x) {
   return x * sigmoid_fast(2.0f * k0 * (x + k1 * x * x * x));
 }
 
-// One grouped GEMM of a persistent launch: contiguous grouped activation rows
-// (row r of expert e = a + (offsets[e] + r) * lda), bf16 weights
-// [n_experts, w_rows, k], output rows in the same grouped order.
+// One grouped GEMM of a persistent launch: grouped activation rows (row r of
+// expert e = a + (offsets[e] + r) * lda, or, with a_rows, the source row
+// a_rows[offsets[e] + r] / a_div of a), bf16 weights [n_experts, w_rows, k],
+// output rows in grouped order.
 struct PersistProblem {
   const void *a;
   int lda;
@@ -133,6 +134,9 @@ struct PersistProblem {
   int ldc;
   int n, k;
   int max_rows;            // host-side upper bound on the grouped rows (offsets live on the device)
+  const int32_t *a_rows;   // grouped row -> slot (the dispatch permutation), or NULL: rows are contiguous
+  int a_div;               // slots per source row (top-k)
+  int a_src_rows;          // rows of the source matrix (range check of the gather)
 };
 constexpr int kMaxPersistProblems = 3;
 struct PersistBatch {
@@ -143,6 +147,9 @@ bool persist_supported(const PersistBatch &b, int mode);
 bool gemm_config_wants_persistent();  // tuning hook state: both stages set to the persistent kernel
 int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s);
 
+int dispatch_impl(const int32_t *flat_idx, const uint8_t *skip_mask, int64_t n_slots, int n_experts,
+                  int32_t *counts, int32_t *offsets, int32_t *perm, int32_t *inv_perm, void *workspace,
+                  size_t workspace_bytes, int32_t *range_out, int32_t range_n, void *stream);
 int gather_rows_impl(const void *x, int dtype, const int32_t *perm, int slots_per_token,
                      int64_t n_rows, int hidden, void *out, int32_t *range_out, int32_t range_n,
                      void *stream);

@@ -132,6 +132,9 @@ struct Tile {
   int n0, n;                 // first output column, output columns of the problem
   int steps;                 // pipeline steps (k / step extent)
   bool valid;
+  const int32_t *a_rows;     // gathered tiles: slot of the tile's first row (else NULL)
+  uint32_t a_magic;          // gathered tiles: source row = mulhi(slot, a_magic) (= slot / a_div)
+  int rows;                  // rows of the tile that belong to its group
 };
 
 // A tile description parked in ONE vector register (lane f holds 32-bit word f),
@@ -141,7 +144,7 @@ struct Tile {
 struct PackedTile {
   uint32_t words;
 };
-constexpr int kTileWords = 20;   // pointers a, b0, b1, c, bias, then ten 32-bit fields
+constexpr int kTileWords = 24;   // pointers a, b0, b1, c, bias, ten 32-bit fields, then a_rows, a_magic, rows
 constexpr int kTableTurns = 64;  // turns of one workgroup that the LDS tile table holds
 __device__ __forceinline__ PackedTile pack_tile(const Tile &t, int lane) {
   const uint64_t p[5] = {(uint64_t)t.a, (uint64_t)t.b0, (uint64_t)t.b1, (uint64_t)t.c, (uint64_t)t.bias};
@@ -155,6 +158,10 @@ __device__ __forceinline__ PackedTile pack_tile(const Tile &t, int lane) {
   }
 #pragma unroll
   for (int i = 0; i < 10; ++i) v = lane == 10 + i ? w[i] : v;
+  v = lane == 20 ? (uint32_t)(uint64_t)t.a_rows : v;
+  v = lane == 21 ? (uint32_t)((uint64_t)t.a_rows >> 32) : v;
+  v = lane == 22 ? t.a_magic : v;
+  v = lane == 23 ? (uint32_t)t.rows : v;
   return PackedTile{v};
 }
 __device__ __forceinline__ Tile unpack_tile(const PackedTile &pk) {
@@ -170,6 +177,9 @@ __device__ __forceinline__ Tile unpack_tile(const PackedTile &pk) {
   t.c_bytes = word(14); t.c_pitch = word(15);
   t.n0 = (int)word(16); t.n = (int)word(17); t.steps = (int)word(18);
   t.valid = word(19) != 0;
+  t.a_rows = (const int32_t *)(((uint64_t)word(21) << 32) | word(20));
+  t.a_magic = word(22);
+  t.rows = (int)word(23);
   return t;
 }
 
@@ -259,13 +269,14 @@ struct TileWalker {
     const int row0 = __shfl(g_row0, grp, kWave), cnt = __shfl(g_cnt, grp, kWave);
     const int mt = __shfl(g_mt, grp, kWave), base = __shfl(g_base, grp, kWave);
     // this lane's problem (a handful of selects instead of a divergent struct index)
-    uint64_t pa = 0, pw = 0, pc = 0, pbias = 0;
-    int lda = 0, ldc = 0, w_rows = 0, up_offset = 0, n = 0, k = 0;
+    uint64_t pa = 0, pw = 0, pc = 0, pbias = 0, prows = 0;
+    int lda = 0, ldc = 0, w_rows = 0, up_offset = 0, n = 0, k = 0, a_div = 1, a_src_rows = 0;
     for (int q = 0; q < batch.n_problems; ++q) {
       const PersistProblem &pr = batch.prob[q];
       if (pi == q) {
         pa = (uint64_t)pr.a; pw = (uint64_t)pr.w; pc = (uint64_t)pr.c; pbias = (uint64_t)pr.bias;
         lda = pr.lda; ldc = pr.ldc; w_rows = pr.w_rows; up_offset = pr.up_offset; n = pr.n; k = pr.k;
+        prows = (uint64_t)pr.a_rows; a_div = pr.a_div; a_src_rows = pr.a_src_rows;
       }
     }
     const int r = idc - base;
@@ -278,11 +289,13 @@ struct TileWalker {
     const int wrows = cols_left < BN_OUT ? cols_left : BN_OUT;
     const uint32_t a_pitch = (uint32_t)lda * 2, b_pitch = (uint32_t)k * 2, c_pitch = (uint32_t)ldc * 2;
     const uint64_t wexp = pw + (uint64_t)expert * w_rows * b_pitch;
-    const uint64_t ptrs[5] = {pa + (uint64_t)(row0 + m_tile * kPBM) * a_pitch, wexp + (uint64_t)n0 * b_pitch,
+    // Gathered rows are addressed from the start of the source matrix.
+    const uint64_t ptrs[5] = {prows ? pa : pa + (uint64_t)(row0 + m_tile * kPBM) * a_pitch, wexp + (uint64_t)n0 * b_pitch,
                               wexp + (uint64_t)(up_offset + n0) * b_pitch,
                               pc + (uint64_t)(row0 + m_tile * kPBM) * c_pitch,
                               pbias ? pbias + ((uint64_t)expert * n) * sizeof(float) : 0};
-    const uint32_t words[10] = {valid ? (uint32_t)rows * a_pitch : 0u, a_pitch, valid ? (uint32_t)wrows * b_pitch : 0u,
+    const uint32_t a_extent = prows ? (uint32_t)a_src_rows * a_pitch : (uint32_t)rows * a_pitch;
+    const uint32_t words[10] = {valid ? a_extent : 0u, a_pitch, valid ? (uint32_t)wrows * b_pitch : 0u,
                                 b_pitch, (uint32_t)rows * c_pitch, c_pitch, (uint32_t)n0, (uint32_t)n,
                                 (uint32_t)(k / bk), valid ? 1u : 0u};
     uint32_t *entry = table + lane * kTileWords;
@@ -293,6 +306,11 @@ struct TileWalker {
     }
 #pragma unroll
     for (int i = 0; i < 10; ++i) entry[10 + i] = words[i];
+    const uint64_t tile_rows = prows ? prows + (uint64_t)(row0 + m_tile * kPBM) * sizeof(int32_t) : 0;
+    entry[20] = (uint32_t)tile_rows;
+    entry[21] = (uint32_t)(tile_rows >> 32);
+    entry[22] = (uint32_t)(0xffffffffull / (uint32_t)a_div + 1);  // mulhi(slot, .) = slot / a_div for slot < 2^28, a_div <= 16
+    entry[23] = (uint32_t)(valid ? rows : 0);
   }
 
   // The id of the tile this workgroup takes in its `round`-th turn.  Turns
@@ -342,6 +360,9 @@ struct TileWalker {
     t.c_bytes = (uint32_t)rows * t.c_pitch;
     t.bias = pr.bias ? pr.bias + (size_t)expert * pr.n : nullptr;
     t.steps = pr.k / bk;
+    t.a_rows = nullptr;
+    t.a_magic = 0;
+    t.rows = rows;
     t.a = uni(t.a); t.b0 = uni(t.b0); t.b1 = uni(t.b1); t.c = uni(t.c); t.bias = uni(t.bias);
     t.a_bytes = uni(t.a_bytes); t.a_pitch = uni(t.a_pitch);
     t.b_bytes = uni(t.b_bytes); t.b_pitch = uni(t.b_pitch);
@@ -758,7 +779,9 @@ __device__ __forceinline__ void qsched_block() {
 
 // BN is the number of weight rows of a tile: 256, or 192 for output widths that
 // 192 divides and 256 does not (1152 = 6 x 192: no padded columns to multiply).
-template <int MODE, bool HAS_BIAS, int BN>
+// GATHER: activation rows may be addressed through a row table (the dispatch
+// permutation), which saves the separate gathered copy of the activations.
+template <int MODE, bool HAS_BIAS, int BN, bool GATHER>
 __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   constexpr bool SWIGLU = MODE == kFc1Swiglu;
   static_assert(BN == 256 || (BN == 192 && !SWIGLU), "tile widths");
@@ -782,8 +805,11 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
 
   // This workgroup's tiles, described once and parked in LDS behind the epilogue's
   // staging rows; lane f of a table read gets word f of the description.
-  static_assert(kQWaves * Epi::WAVE_BYTES + kTableTurns * kTileWords * 4 <= kPStageArea, "no room for the tile table");
-  uint32_t *const tile_table = reinterpret_cast<uint32_t *>(lds_stage + kPStageArea - kTableTurns * kTileWords * 4);
+  constexpr int kTableBytes = kTableTurns * kTileWords * 4, kRowSlotBytes = GATHER ? kPBM * 4 : 0;
+  static_assert(kQWaves * Epi::WAVE_BYTES + kTableBytes + kRowSlotBytes <= kPStageArea, "no room for the tile table");
+  uint32_t *const tile_table = reinterpret_cast<uint32_t *>(lds_stage + kPStageArea - kTableBytes);
+  // (gathered activations) the slots of the 256 rows of the tile the load side opens next
+  int32_t *const lds_row_slots = reinterpret_cast<int32_t *>(lds_stage + kPStageArea - kTableBytes - kPBM * 4);
   if (wave == 0) {
     TileWalker<BN_OUT> walk(batch, lane);
     walk.build_table(batch, lane, kQBK, tile_table);
@@ -803,11 +829,44 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   // reads, are the same for every l)
   uint32_t wr_off = qring_off(cp_row0, cp_chunk);
   asm volatile("" : "+v"(wr_off));
-  uint32_t ld_voff_a = 0, ld_voff_b = 0;  // per-lane byte offsets inside the tile being loaded
+  // Per-lane byte offsets inside the tile being loaded.  Without a row table
+  // load i of the activations is row cp_row0 + 32 i: one offset plus a scalar
+  // stride.  With one, each of a lane's kCopiesA rows has its own offset, worked
+  // out at the tile switch from the tile's 256 row numbers, which the first wave
+  // copied into LDS (one global->LDS instruction) a tile earlier.
+  uint32_t ld_voff_a = 0, ld_voff_b = 0;
+  uint32_t ld_voff_rows[GATHER ? kCopiesA : 1];
+  auto copy_row_slots = [&](const PackedTile &pk) {
+    if constexpr (GATHER) {
+      const uint64_t ptr = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane(pk.words, 21) << 32) |
+                           (uint32_t)__builtin_amdgcn_readlane(pk.words, 20);
+      const int rows = __builtin_amdgcn_readlane(pk.words, 23);
+      if (wave == 0 && ptr != 0) {
+        // rows past the group's end read as slot 0 (a legal row; their products are never stored)
+        const __amdgpu_buffer_rsrc_t rs =
+            __builtin_amdgcn_make_buffer_rsrc((void *)ptr, 0, (uint32_t)rows * 4, kRsrcFlags);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void *)lds_row_slots, 16,
+                                                 lane * 16, 0, 0, 0);
+      }
+    }
+  };
   auto set_copy_offsets = [&](const Tile &t) {
     ld_voff_a = (uint32_t)cp_row0 * t.a_pitch + cp_chunk * 16;
     ld_voff_b = (uint32_t)cp_row0 * t.b_pitch + cp_chunk * 16;
     asm volatile("" : "+v"(ld_voff_a), "+v"(ld_voff_b));
+    if constexpr (GATHER) {
+#pragma unroll
+      for (int i = 0; i < kCopiesA; ++i) {
+        const int r = cp_row0 + 32 * i;
+        uint32_t off = ld_voff_a + (uint32_t)(32 * i) * t.a_pitch;
+        if (t.a_rows) {
+          const uint32_t slot = (uint32_t)lds_row_slots[r];
+          off = r < t.rows ? __umulhi(slot, t.a_magic) * t.a_pitch + cp_chunk * 16 : kOutOfRange;
+        }
+        ld_voff_rows[i] = off;
+        asm volatile("" : "+v"(ld_voff_rows[i]));
+      }
+    }
   };
   u32x4_t stage_regs[2][kQCopies];
 
@@ -859,12 +918,23 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   // next tile once while a tile is multiplied.  That tile's description (`nxt`)
   // is worked out between tiles, where registers are free, not inside the k loop.
   int next_turn = 0;                              // this workgroup's next turn
-  Tile ld = unpack_tile(fetch_tile(next_turn++));  // tile being loaded
+  PackedTile nxt = fetch_tile(next_turn++);
+  Tile ld = unpack_tile(nxt);                     // tile being loaded
   if (!ld.valid) return;                          // nothing to do for this workgroup
-  PackedTile nxt = fetch_tile(next_turn++);       // the one the load side opens next
+  if constexpr (GATHER) {
+    copy_row_slots(nxt);
+    pwait_vmcnt<0>();
+    phase_barrier();
+  }
   Tile cp = ld;                                   // tile being multiplied
   int ld_kt = 0;
   set_copy_offsets(ld);
+  nxt = fetch_tile(next_turn++);                  // the one the load side opens next
+  if constexpr (GATHER) {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // everyone has read the first tile's row slots
+    phase_barrier();
+    copy_row_slots(nxt);
+  }
   auto advance_copy = [&]() {
     if (++ld_kt == ld.steps) {
       ld = unpack_tile(nxt);
@@ -887,8 +957,8 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
         // avoids a loop over lanes around the load if the compiler moved it out)
         const __amdgpu_buffer_rsrc_t rs =
             __builtin_amdgcn_make_buffer_rsrc((void *)uni(ld.a), 0, uni(ld.a_bytes), kRsrcFlags);
-        stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(
-            rs, ld_voff_a + (uint32_t)(32 * i) * uni(ld.a_pitch), uni(ld_kt * 128), 0);
+        const uint32_t voff = GATHER ? ld_voff_rows[i] : ld_voff_a + (uint32_t)(32 * i) * uni(ld.a_pitch);
+        stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, uni(ld_kt * 128), 0);
       } else {
         const int i = l - kCopiesA;
         const bool up_half = SWIGLU && 32 * i >= BN / 2;  // wave * 8 + 7 < 32 never crosses the halves
@@ -981,6 +1051,12 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
     cp = ld;
     if (!cp.valid) break;
     nxt = fetch_tile(next_turn++);
+    // The load side opened this tile's predecessor at least kQMinSteps - 4 steps
+    // (each with a barrier) ago and read its row slots then: the buffer is free.
+    // The copy below is older than every load of the coming steps, so the waits
+    // for those (at most 32 newer loads are ever in flight) cover it long before
+    // the load side opens `nxt`, at least two steps from here.
+    copy_row_slots(nxt);
     zero_acc();
     // The last block above already fetched these fragments; reading them again
     // here keeps 32 registers free during the epilogue.
@@ -996,9 +1072,9 @@ __global__ __launch_bounds__(8 * kWave, 1) void gemm_persist_kernel8(PersistBatc
   gemm_persist_body<MODE, HAS_BIAS, 8>(batch);
 }
 // Four waves, one per SIMD, each with the whole 512-entry register file.
-template <int MODE, bool HAS_BIAS, int BN>
+template <int MODE, bool HAS_BIAS, int BN, bool GATHER>
 __global__ __launch_bounds__(4 * kWave, 1) void gemm_persist_kernel4(PersistBatch batch) {
-  gemm_persist64_body<MODE, HAS_BIAS, BN>(batch);
+  gemm_persist64_body<MODE, HAS_BIAS, BN, GATHER>(batch);
 }
 
 }  // namespace
@@ -1012,6 +1088,11 @@ bool persist_supported(const PersistBatch &b, int mode) {
     groups += p.n_experts;
     if (p.k % (kPBK * kPStages) != 0) return false;  // whole trips round the ring per tile
     if (g_persist_waves == 4 && p.k < kQBK * kQMinSteps) return false;
+    if (p.a_rows) {  // gathered activation rows: 64-k SwiGLU kernel only
+      if (g_persist_waves != 4 || mode != kFc1Swiglu) return false;
+      if (p.a_div < 1 || p.a_div > 16 || (int64_t)p.a_src_rows * p.a_div >= (1ll << 28)) return false;
+      if ((size_t)p.a_src_rows * p.lda * 2 >= (1ull << 31)) return false;
+    }
     if (p.n % 8 != 0 || p.lda % 8 != 0 || p.ldc % 8 != 0) return false;
     if (mode == kFc1Swiglu && p.n % (kPBN / 2) != 0) return false;  // gate/up halves share one range check
     if ((size_t)kPBM * p.lda * 2 >= (1ull << 31) || (size_t)kPBN * p.k * 2 >= (1ull << 31)) return false;
@@ -1035,20 +1116,24 @@ int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s) 
   if (mode == kFc1Swiglu) has_bias = false;
   const int waves = g_persist_waves == 4 ? 4 : 8;
   void (*kern)(PersistBatch) = nullptr;
+  bool gathered = false;
+  for (int i = 0; i < b.n_problems; ++i) gathered = gathered || b.prob[i].a_rows != nullptr;
   // 192-row weight tiles where they avoid padded columns (n = 1152 = 6 x 192).
   bool narrow = mode != kFc1Swiglu;
   for (int i = 0; i < b.n_problems; ++i)
     narrow = narrow && b.prob[i].n % 192 == 0 && b.prob[i].n % 256 != 0;
   if (waves == 4 && narrow) {
     switch (mode) {
-      case kFc1Gelu: kern = has_bias ? gemm_persist_kernel4<kFc1Gelu, true, 192> : gemm_persist_kernel4<kFc1Gelu, false, 192>; break;
-      default: kern = has_bias ? gemm_persist_kernel4<kFc2, true, 192> : gemm_persist_kernel4<kFc2, false, 192>; break;
+      case kFc1Gelu: kern = has_bias ? gemm_persist_kernel4<kFc1Gelu, true, 192, false> : gemm_persist_kernel4<kFc1Gelu, false, 192, false>; break;
+      default: kern = has_bias ? gemm_persist_kernel4<kFc2, true, 192, false> : gemm_persist_kernel4<kFc2, false, 192, false>; break;
     }
   } else if (waves == 4) {
     switch (mode) {
-      case kFc1Swiglu: kern = gemm_persist_kernel4<kFc1Swiglu, false, 256>; break;
-      case kFc1Gelu: kern = has_bias ? gemm_persist_kernel4<kFc1Gelu, true, 256> : gemm_persist_kernel4<kFc1Gelu, false, 256>; break;
-      default: kern = has_bias ? gemm_persist_kernel4<kFc2, true, 256> : gemm_persist_kernel4<kFc2, false, 256>; break;
+      case kFc1Swiglu:
+        kern = gathered ? gemm_persist_kernel4<kFc1Swiglu, false, 256, true> : gemm_persist_kernel4<kFc1Swiglu, false, 256, false>;
+        break;
+      case kFc1Gelu: kern = has_bias ? gemm_persist_kernel4<kFc1Gelu, true, 256, false> : gemm_persist_kernel4<kFc1Gelu, false, 256, false>; break;
+      default: kern = has_bias ? gemm_persist_kernel4<kFc2, true, 256, false> : gemm_persist_kernel4<kFc2, false, 256, false>; break;
     }
   } else {
     switch (mode) {

@@ -58,13 +58,6 @@ LayerWorkspace carve_layer(const dice_moe_layer_t *L, int64_t n_tokens, void *ws
   return w;
 }
 
-__global__ void set_range_kernel(int32_t *offsets, int32_t n) {
-  if (threadIdx.x == 0) {
-    offsets[0] = 0;
-    offsets[1] = n;
-  }
-}
-
 // Stage timers of dice_moe_forward: HIP events recorded on the caller's stream
 // between the launches, the counterpart of the reference's CudaProfiler scopes
 // "moe.gate" / "moe.mlp" / "moe.mlp_shared" (models.py:305,356,375;
@@ -272,8 +265,9 @@ extern "C" int dice_moe_forward(const dice_moe_layer_t *L, const void *x, int64_
                       L->n_experts, L->top_k, L->norm_topk_prob, idx, nullptr, wt, nullptr, stream);
   if (rc) return rc;
   stamp(1, s);
-  rc = dice_dispatch(idx, mode == 2 ? skip_mask : nullptr, slots, L->n_experts, w.counts, w.offsets,
-                     w.perm, w.inv_perm, w.dispatch_ws, w.dispatch_ws_bytes, stream);
+  rc = dispatch_impl(idx, mode == 2 ? skip_mask : nullptr, slots, L->n_experts, w.counts, w.offsets, w.perm,
+                     w.inv_perm, w.dispatch_ws, w.dispatch_ws_bytes,
+                     L->shared_inter > 0 ? w.shared_offsets : nullptr, (int32_t)n_tokens, stream);
   if (rc) return rc;
   stamp(2, s);
   // A skip step recomputes one slot per token.
@@ -301,10 +295,21 @@ extern "C" int dice_moe_forward(const dice_moe_layer_t *L, const void *x, int64_
                                   swiglu ? nullptr : L->shared_b2, w.shared_out, L->hidden, L->hidden, si, (int)n_tokens};
       f1.n_problems = f2.n_problems = 2;
     }
-    if (persist_supported(f1, m1) && persist_supported(f2, kFc2)) {
-      rc = gather_rows_impl(x, L->act_dtype, w.perm, L->top_k, max_rows, L->hidden, xg,
-                            L->shared_inter > 0 ? w.shared_offsets : nullptr, (int32_t)n_tokens, stream);
-      if (rc) return rc;
+    // Where the kernel can address the activation rows through the permutation
+    // itself, the gathered copy is skipped.
+    PersistBatch f1g = f1;
+    f1g.prob[0].a = x;
+    f1g.prob[0].a_rows = w.perm;
+    f1g.prob[0].a_div = L->top_k;
+    f1g.prob[0].a_src_rows = (int)n_tokens;
+    const bool fused_gather = persist_supported(f1g, m1) && persist_supported(f2, kFc2);
+    if (fused_gather || (persist_supported(f1, m1) && persist_supported(f2, kFc2))) {
+      if (fused_gather) {
+        f1 = f1g;
+      } else {
+        rc = gather_rows_impl(x, L->act_dtype, w.perm, L->top_k, max_rows, L->hidden, xg, nullptr, 0, stream);
+        if (rc) return rc;
+      }
       stamp(3, s);
       rc = launch_grouped_gemm_persist(f1, m1, s);
       if (rc) return rc;
@@ -325,7 +330,6 @@ extern "C" int dice_moe_forward(const dice_moe_layer_t *L, const void *x, int64_
                         L->w_dtype, L->act_variant, w.h, w.slot_out, 1, stream);
   if (rc) return rc;
   if (L->shared_inter > 0) {
-    hipLaunchKernelGGL(set_range_kernel, dim3(1), dim3(64), 0, s, w.shared_offsets, (int32_t)n_tokens);
     rc = dice_grouped_mlp(x, L->act_dtype, nullptr, 1, w.shared_offsets, 1, n_tokens, L->hidden,
                           L->shared_inter, L->shared_w1, L->shared_b1, L->shared_w2, L->shared_b2,
                           nullptr, nullptr, L->act_dtype, L->act_variant, w.shared_h, w.shared_out, 0,
