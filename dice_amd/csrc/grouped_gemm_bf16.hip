@@ -816,6 +816,7 @@ bool gemm_config_wants_persistent() { return g_cfg_fc1 >= kCfgPersistent && g_cf
 extern "C" int dice_set_gemm_config(int fc1_cfg, int fc2_cfg) {
   dice::g_cfg_fc1 = fc1_cfg;
   dice::g_cfg_fc2 = fc2_cfg;
-  if (fc1_cfg >= dice::kCfgPersistent) dice::g_persist_waves = fc1_cfg == dice::kCfgPersistent + 1 ? 4 : 8;
+  // 20: the 32-k eight-wave pipeline only; anything else: the 64-k pipeline where it applies (default)
+  dice::g_persist_waves = fc1_cfg == dice::kCfgPersistent ? 8 : 4;
   return DICE_OK;
 }

@@ -1079,42 +1079,81 @@ __global__ __launch_bounds__(4 * kWave, 1) void gemm_persist_kernel4(PersistBatc
 
 }  // namespace
 
-int g_persist_waves = 4;  // tuning hook: 4 = 64-k register-staged pipeline, 8 = 32-k ping-pong pipeline
+int g_persist_waves = 4;  // tuning hook: 4 = 64-k register-staged pipeline first, 8 = 32-k ping-pong pipeline only
 
-bool persist_supported(const PersistBatch &b, int mode) {
+namespace {
+
+int cu_count() {
+  static thread_local int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess)
+      cus = n;
+  }
+  return cus;
+}
+
+// Conditions both pipelines share.
+bool persist_common_ok(const PersistBatch &b, int mode) {
   int groups = 0;
   for (int i = 0; i < b.n_problems; ++i) {
     const PersistProblem &p = b.prob[i];
     groups += p.n_experts;
     if (p.k % (kPBK * kPStages) != 0) return false;  // whole trips round the ring per tile
-    if (g_persist_waves == 4 && p.k < kQBK * kQMinSteps) return false;
-    if (p.a_rows) {  // gathered activation rows: 64-k SwiGLU kernel only
-      if (g_persist_waves != 4 || mode != kFc1Swiglu) return false;
-      if (p.a_div < 1 || p.a_div > 16 || (int64_t)p.a_src_rows * p.a_div >= (1ll << 28)) return false;
-      if ((size_t)p.a_src_rows * p.lda * 2 >= (1ull << 31)) return false;
-    }
     if (p.n % 8 != 0 || p.lda % 8 != 0 || p.ldc % 8 != 0) return false;
     if (mode == kFc1Swiglu && p.n % (kPBN / 2) != 0) return false;  // gate/up halves share one range check
     if ((size_t)kPBM * p.lda * 2 >= (1ull << 31) || (size_t)kPBN * p.k * 2 >= (1ull << 31)) return false;
   }
-  return groups >= 1 && groups <= kWave;
+  return groups >= 1 && groups <= kWave && cu_count() >= kNumXcd;
 }
 
-int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s) {
-  if (!persist_supported(b, mode))
-    return fail(DICE_ERR_UNSUPPORTED, "persistent expert GEMM: unsupported shape");
-  static thread_local int grid = 0;
-  if (grid == 0) {
-    int dev = 0, cus = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < kNumXcd)
-      return fail(DICE_ERR_LAUNCH, "persistent expert GEMM: cannot query the CU count");
-    grid = cus / kNumXcd * kNumXcd;
+// 64-k kernel: long enough tiles, and a workgroup's tile descriptions must fit
+// the LDS table of kTableTurns entries (the last one stays an invalid tile).
+// The turns of one workgroup are bounded from the host-side row bounds: an XCD
+// gets 1/8 of the total cost, in the worst case all of it in its shortest tiles.
+bool persist64_ok(const PersistBatch &b, int mode) {
+  int64_t cost = 0;
+  int min_k32 = 1 << 30;
+  for (int i = 0; i < b.n_problems; ++i) {
+    const PersistProblem &p = b.prob[i];
+    if (p.k < kQBK * kQMinSteps) return false;
+    if (p.a_rows) {  // gathered activation rows: SwiGLU instantiation only
+      if (mode != kFc1Swiglu) return false;
+      if (p.a_div < 1 || p.a_div > 16 || (int64_t)p.a_src_rows * p.a_div >= (1ll << 28)) return false;
+      if ((size_t)p.a_src_rows * p.lda * 2 >= (1ull << 31)) return false;
+    }
+    const int bn_out = mode == kFc1Swiglu ? kPBN / 2 : (p.n % 192 == 0 && p.n % 256 != 0 ? 192 : kPBN);
+    const int64_t m_tiles = ((int64_t)p.max_rows + kPBM - 1) / kPBM + p.n_experts;
+    const int64_t n_tiles = (p.n + bn_out - 1) / bn_out;
+    cost += m_tiles * n_tiles * (p.k / 32);
+    min_k32 = p.k / 32 < min_k32 ? p.k / 32 : min_k32;
   }
+  const int wgs_per_xcd = cu_count() / kNumXcd;
+  const int64_t tiles_per_xcd = cost / kNumXcd / min_k32 + 2;
+  return (tiles_per_xcd + wgs_per_xcd - 1) / wgs_per_xcd + 2 <= kTableTurns;
+}
+
+// 0: neither pipeline applies; 4: the 64-k four-wave kernel; 8: the 32-k eight-wave kernel.
+int persist_variant(const PersistBatch &b, int mode) {
+  if (!persist_common_ok(b, mode)) return 0;
+  if (g_persist_waves == 4 && persist64_ok(b, mode)) return 4;
+  for (int i = 0; i < b.n_problems; ++i)
+    if (b.prob[i].a_rows) return 0;  // the 32-k kernel wants contiguous rows
+  return 8;
+}
+
+}  // namespace
+
+bool persist_supported(const PersistBatch &b, int mode) { return persist_variant(b, mode) != 0; }
+
+int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s) {
+  const int waves = persist_variant(b, mode);
+  if (waves == 0) return fail(DICE_ERR_UNSUPPORTED, "persistent expert GEMM: unsupported shape");
+  const int grid = cu_count() / kNumXcd * kNumXcd;
   bool has_bias = false;
   for (int i = 0; i < b.n_problems; ++i) has_bias = has_bias || b.prob[i].bias != nullptr;
   if (mode == kFc1Swiglu) has_bias = false;
-  const int waves = g_persist_waves == 4 ? 4 : 8;
   void (*kern)(PersistBatch) = nullptr;
   bool gathered = false;
   for (int i = 0; i < b.n_problems; ++i) gathered = gathered || b.prob[i].a_rows != nullptr;

@@ -253,6 +253,55 @@ def test_mlp_bf16_tilings(dev, variant, cfg):
     _check_mlp(dev, 600, 1152, 4, 4, torch.bfloat16, variant, cfg=(cfg, cfg))  # XL width, 4.5 n-tiles
 
 
+def _check_mlp_persistent(dev, N, D, E, ratio, variant, cfg, counts=None, seed=0):
+    """The persistent kernels take contiguous grouped rows (perm = None)."""
+    from dice_amd import lib, ops
+    dtype = torch.bfloat16
+    g = _gen(seed + N + D)
+    p = O.make_block_params(D, E, 2, ratio, n_shared=0, seed=seed, dtype=dtype, variant=variant)
+    if variant == "gelu_tanh":
+        for e in p.experts:
+            e.fc1_b = (torch.randn(e.fc1_b.shape, generator=g) * 0.1).to(dtype)
+            e.fc2_b = (torch.randn(e.fc2_b.shape, generator=g) * 0.1).to(dtype)
+    x = torch.randn(N, D, generator=g).to(dtype)
+    if counts is None:
+        idx = torch.randint(0, E, (N * 2,), generator=g)
+    else:
+        idx = torch.cat([torch.full((c,), e) for e, c in enumerate(counts)])
+        idx = idx[torch.randperm(idx.numel(), generator=g)]
+        assert idx.numel() == N * 2
+    _, offsets, perm, _ = O.dispatch_tables(idx, E)
+    xg = x[perm // 2]
+    w1, w2, b1, b2 = _packed(p, variant, dtype, dev)
+    lib.load().dice_set_gemm_config(cfg, cfg)
+    try:
+        out = ops.grouped_mlp(xg.to(dev), None, 1, offsets.int().to(dev), N * 2, w1, w2, variant, b1, b2).cpu()
+    finally:
+        lib.load().dice_set_gemm_config(0, 0)
+    want = torch.empty(N * 2, D, dtype=dtype)
+    for e in range(E):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        if hi > lo:
+            want[lo:hi] = p.experts[e](xg[lo:hi])
+    assert rel_l2(out, want) < BF16_TOL, f"grouped output off: {rel_l2(out, want)}"
+    err = (out.double() - want.double()).norm(dim=1) / want.double().norm(dim=1).clamp_min(1e-6)
+    assert err.max() < 5 * BF16_TOL, f"worst row {int(err.argmax())} rel err {float(err.max())}"
+
+
+@pytest.mark.parametrize("cfg", [20, 21])   # 20: 32-k eight-wave pipeline only; 21: 64-k pipeline where it applies
+@pytest.mark.parametrize("variant", ["swiglu", "gelu_tanh"])
+def test_mlp_bf16_persistent_kernels(dev, variant, cfg):
+    _check_mlp_persistent(dev, 1024, 256, 8, 4, variant, cfg)            # k = 256: too short for 64-k steps
+    _check_mlp_persistent(dev, 600, 1152, 4, 4, variant, cfg)            # XL width: 192-row fc2 tiles
+    _check_mlp_persistent(dev, 700, 384, 8, 4, variant, cfg)             # k = 384: six 64-k steps, fc2 n = 384 (padded tile)
+    _check_mlp_persistent(dev, 512, 640, 8, 2, variant, cfg)             # k = 640 is no multiple of 128: no persistent kernel
+    # empty experts, single-row groups, a group of exactly one tile, one hot expert
+    _check_mlp_persistent(dev, 512, 512, 8, 2, variant, cfg, counts=[0, 1, 256, 0, 257, 3, 507, 0])
+    _check_mlp_persistent(dev, 512, 512, 8, 2, variant, cfg, counts=[1024, 0, 0, 0, 0, 0, 0, 0])
+
+
+
+
 @pytest.mark.parametrize("cfg", [0, 1, 2])
 def test_mlp_bf16_ragged_groups(dev, cfg):
     # empty experts, single-row groups, a group of exactly one tile, one hot expert
@@ -371,6 +420,19 @@ def test_block_c2_bf16_full_size(dev, variant):
     assert rel_l2(y.view(-1, D)[sub][ok], want[ok]) < BF16_TOL
     # determinism: a second call is bit-identical
     assert torch.equal(blk(x.to(dev)).cpu(), y)
+
+
+def test_block_many_tokens_per_workgroup(dev):
+    """More tiles per workgroup than the 64-k kernel's tile table holds: the layer
+    has to pick another kernel and still agree with the oracle."""
+    D, E, N = 384, 8, 172032
+    p = O.make_block_params(D, E, 2, 4, 2, seed=5, dtype=torch.bfloat16, variant="swiglu")
+    x = torch.randn(1, N, D, generator=_gen(5)).bfloat16()
+    blk, y = _run_block(dev, p, x, "swiglu", torch.bfloat16)
+    sub = torch.randperm(N, generator=_gen(6))[:256]
+    want, _, logits = _subset_oracle(p, x.view(-1, D), sub, torch.bfloat16)
+    ties = O.gate_tie_rows(logits, 2).view(-1)
+    assert rel_l2(y.view(-1, D)[sub][~ties], want[~ties]) < BF16_TOL
 
 
 def test_block_c3_zipf_load(dev):
