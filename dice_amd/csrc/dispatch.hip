@@ -19,7 +19,9 @@ namespace {
 
 constexpr int kMaxExperts = 256;
 constexpr int kFusedWaves = 16;       // single-workgroup path: 1024 threads
-constexpr int64_t kFusedMaxSlots = 65536;
+constexpr int64_t kFusedMaxSlots = 2048;    // one workgroup, one launch: launch-latency bound sizes
+constexpr int kMidRounds = 4;               // two-launch path: 256 slots per wave
+constexpr int64_t kMidMaxTable = 1 << 16;   // ... while units x experts stays this small
 constexpr int kTileWaves = 4;         // multi-workgroup path: 256 threads
 constexpr int kTileRounds = 8;        // 512 slots per wave
 
@@ -202,7 +204,7 @@ __global__ __launch_bounds__(kFusedWaves *kWave) void dispatch_fused_kernel(
 
 __global__ __launch_bounds__(kTileWaves *kWave) void dispatch_count_kernel(
     const int32_t *__restrict__ idx, const uint8_t *__restrict__ skip, int64_t n_slots,
-    int n_experts, int nbits, int units, int32_t *__restrict__ unit_cnt) {
+    int n_experts, int nbits, int units, int rounds, int32_t *__restrict__ unit_cnt) {
   __shared__ volatile int32_t wrow[kTileWaves][kMaxExperts];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
@@ -210,8 +212,8 @@ __global__ __launch_bounds__(kTileWaves *kWave) void dispatch_count_kernel(
   for (int e = lane; e < n_experts; e += kWave) wrow[wave][e] = 0;
   __syncthreads();
   if (unit < units) {
-    count_span(idx, skip, n_slots, n_experts, nbits, (int64_t)unit * kTileRounds * kWave,
-               kTileRounds, wrow[wave], lane);
+    count_span(idx, skip, n_slots, n_experts, nbits, (int64_t)unit * rounds * kWave, rounds, wrow[wave],
+               lane);
     for (int e = lane; e < n_experts; e += kWave) unit_cnt[(size_t)e * units + unit] = wrow[wave][e];
   }
 }
@@ -284,6 +286,66 @@ __global__ __launch_bounds__(kTileWaves *kWave) void dispatch_rank_kernel(
   }
 }
 
+// Second kernel of the two-launch path (mid-size inputs): every wave sums the
+// unit table itself - totals per expert for the offsets, and the counts of the
+// units before its own for its start positions - then ranks its unit.  The
+// table is units x experts integers, a few KB, and comes out of the L2.
+__global__ __launch_bounds__(kTileWaves *kWave) void dispatch_scan_rank_kernel(
+    const int32_t *__restrict__ idx, const uint8_t *__restrict__ skip, int64_t n_slots,
+    int n_experts, int nbits, int units, int rounds, const int32_t *__restrict__ unit_cnt,
+    int32_t *__restrict__ counts, int32_t *__restrict__ offsets, int32_t *__restrict__ perm,
+    int32_t *__restrict__ inv_perm, int32_t *__restrict__ range_out, int32_t range_n) {
+  __shared__ volatile int32_t wrow[kTileWaves][kMaxExperts];
+  __shared__ int32_t wtot[kTileWaves][kMaxExperts];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int unit = blockIdx.x * kTileWaves + wave;
+  if (range_out && blockIdx.x == 0 && threadIdx.x == 0) {
+    range_out[0] = 0;
+    range_out[1] = range_n;
+  }
+  if (unit >= units) return;
+  // per expert: total over all units and total over the units before this one
+  int carry = 0;  // running exclusive offset over experts
+  for (int c = 0; c < n_experts; c += kWave) {
+    const int e = c + lane;
+    int tot = 0, before = 0;
+    if (e < n_experts) {
+      const int32_t *rowp = unit_cnt + (size_t)e * units;
+      for (int u = 0; u < units; ++u) {
+        const int v = rowp[u];
+        tot += v;
+        before += u < unit ? v : 0;
+      }
+    }
+    int inc = tot;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+      const int up = __shfl_up(inc, o, kWave);
+      if (lane >= o) inc += up;
+    }
+    if (e < n_experts) {
+      const int off = carry + inc - tot;
+      wrow[wave][e] = off + before;
+      wtot[wave][e] = tot;
+      if (unit == 0) {
+        counts[e] = tot;
+        offsets[e] = off;
+      }
+    }
+    carry += __shfl(inc, kWave - 1, kWave);
+  }
+  if (unit == 0 && lane == 0) offsets[n_experts] = carry;
+  __builtin_amdgcn_wave_barrier();
+  const int64_t begin = (int64_t)unit * rounds * kWave;
+  rank_span(idx, skip, n_slots, n_experts, nbits, begin, rounds, wrow[wave], lane, perm, inv_perm);
+  const int total = carry;
+  for (int r = 0; r < rounds; ++r) {
+    const int64_t i = begin + (int64_t)r * kWave + lane;
+    if (i >= total && i < n_slots) perm[i] = -1;
+  }
+}
+
 // `range_out` (optional) receives {0, range_n}: the one-group offset table of
 // the shared expert, written here so the layer needs no extra launch for it.
 template <typename V>
@@ -318,7 +380,10 @@ int bits_for(int n_experts) {
 extern "C" size_t dice_dispatch_workspace_bytes(int64_t n_slots, int n_experts) {
   using namespace dice;
   if (n_slots <= kFusedMaxSlots || n_experts <= 0) return 256;
-  const int64_t units = (n_slots + kTileRounds * kWave - 1) / (kTileRounds * kWave);
+  const int64_t mid_units = (n_slots + kMidRounds * kWave - 1) / (kMidRounds * kWave);
+  const int64_t units = mid_units * n_experts <= kMidMaxTable
+                            ? mid_units
+                            : (n_slots + kTileRounds * kWave - 1) / (kTileRounds * kWave);
   return align_up((size_t)units * n_experts * sizeof(int32_t), 256);
 }
 
@@ -337,27 +402,35 @@ int dispatch_impl(const int32_t *flat_idx, const uint8_t *skip_mask, int64_t n_s
   hipStream_t s = (hipStream_t)stream;
   const int nbits = bits_for(n_experts);
   if (n_slots <= kFusedMaxSlots) {
-    int rounds = (int)((n_slots + kFusedWaves * kWave - 1) / (kFusedWaves * kWave));
-    if (rounds <= 16)
-      hipLaunchKernelGGL(dispatch_fused_kernel<16>, dim3(1), dim3(kFusedWaves * kWave), 0, s, flat_idx,
-                         skip_mask, n_slots, n_experts, nbits, rounds, counts, offsets, perm, inv_perm, range_out, range_n);
-    else if (rounds <= 32)
-      hipLaunchKernelGGL(dispatch_fused_kernel<32>, dim3(1), dim3(kFusedWaves * kWave), 0, s, flat_idx,
-                         skip_mask, n_slots, n_experts, nbits, rounds, counts, offsets, perm, inv_perm, range_out, range_n);
-    else
-      hipLaunchKernelGGL(dispatch_fused_kernel<64>, dim3(1), dim3(kFusedWaves * kWave), 0, s, flat_idx,
-                         skip_mask, n_slots, n_experts, nbits, rounds, counts, offsets, perm, inv_perm, range_out, range_n);
+    constexpr int kMaxRounds = (int)(kFusedMaxSlots / (kFusedWaves * kWave));
+    const int rounds = (int)((n_slots + kFusedWaves * kWave - 1) / (kFusedWaves * kWave));
+    hipLaunchKernelGGL(dispatch_fused_kernel<kMaxRounds>, dim3(1), dim3(kFusedWaves * kWave), 0, s, flat_idx,
+                       skip_mask, n_slots, n_experts, nbits, rounds, counts, offsets, perm, inv_perm, range_out,
+                       range_n);
     return launch_status("dice_dispatch");
   }
-  const int64_t units64 = (n_slots + kTileRounds * kWave - 1) / (kTileRounds * kWave);
-  const int units = (int)units64;
   const size_t need = dice_dispatch_workspace_bytes(n_slots, n_experts);
   DICE_REQUIRE(workspace && workspace_bytes >= need, DICE_ERR_WORKSPACE,
                "dice_dispatch: workspace %zu < %zu bytes", workspace_bytes, need);
   int32_t *unit_cnt = (int32_t *)workspace;
+  const int64_t mid_units = (n_slots + kMidRounds * kWave - 1) / (kMidRounds * kWave);
+  if (mid_units * n_experts <= kMidMaxTable) {
+    // Mid sizes: per-wave histograms, then one kernel that scans the (small)
+    // table in every wave and ranks.
+    const int units = (int)mid_units;
+    const int blocks = (units + kTileWaves - 1) / kTileWaves;
+    hipLaunchKernelGGL(dispatch_count_kernel, dim3(blocks), dim3(kTileWaves * kWave), 0, s, flat_idx,
+                       skip_mask, n_slots, n_experts, nbits, units, kMidRounds, unit_cnt);
+    hipLaunchKernelGGL(dispatch_scan_rank_kernel, dim3(blocks), dim3(kTileWaves * kWave), 0, s, flat_idx,
+                       skip_mask, n_slots, n_experts, nbits, units, kMidRounds, unit_cnt, counts, offsets,
+                       perm, inv_perm, range_out, range_n);
+    return launch_status("dice_dispatch");
+  }
+  const int64_t units64 = (n_slots + kTileRounds * kWave - 1) / (kTileRounds * kWave);
+  const int units = (int)units64;
   const int blocks = (units + kTileWaves - 1) / kTileWaves;
   hipLaunchKernelGGL(dispatch_count_kernel, dim3(blocks), dim3(kTileWaves * kWave), 0, s, flat_idx,
-                     skip_mask, n_slots, n_experts, nbits, units, unit_cnt);
+                     skip_mask, n_slots, n_experts, nbits, units, kTileRounds, unit_cnt);
   hipLaunchKernelGGL(dispatch_scan_kernel, dim3(1), dim3(1024), 0, s, unit_cnt, n_experts, units,
                      counts, offsets, range_out, range_n);
   hipLaunchKernelGGL(dispatch_rank_kernel, dim3(blocks), dim3(kTileWaves * kWave), 0, s, flat_idx,
