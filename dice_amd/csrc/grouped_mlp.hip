@@ -66,18 +66,27 @@ LayerWorkspace carve_layer(const dice_moe_layer_t *L, int64_t n_tokens, void *ws
 constexpr int kStages = 6;
 const char *const kStageNames[kStages] = {"moe.gate", "moe.dispatch", "moe.gather", "moe.mlp.fc1",
                                           "moe.mlp.fc2", "moe.combine"};
+// A ring of event sets, one per timed call, so that a run of back-to-back calls
+// can be timed without a host synchronisation between them.
+constexpr int kTimerRing = 64;
+constexpr int kFc1Stage = 3;  // index of "moe.mlp.fc1"
 struct StageTimers {
-  bool enabled = false;
+  int mode = 0;       // 0 off, 1 every stage, 2 only the brackets of moe.mlp.fc1
   bool have_events = false;
-  bool recorded = false;
-  hipEvent_t ev[kStages + 1];
+  int recorded = 0;   // calls recorded since the last read (saturates at kTimerRing)
+  int next = 0;       // ring position of the call being recorded
+  hipEvent_t ev[kTimerRing][kStages + 1];
 };
 StageTimers g_timers;
 
 void stamp(int i, hipStream_t s) {
-  if (g_timers.enabled && g_timers.have_events) {
-    (void)hipEventRecord(g_timers.ev[i], s);
-    if (i == kStages) g_timers.recorded = true;
+  if (g_timers.mode != 0 && g_timers.have_events) {
+    if (g_timers.mode == 1 || i == kFc1Stage || i == kFc1Stage + 1)
+      (void)hipEventRecord(g_timers.ev[g_timers.next][i], s);
+    if (i == kStages) {
+      g_timers.next = (g_timers.next + 1) % kTimerRing;
+      if (g_timers.recorded < kTimerRing) ++g_timers.recorded;
+    }
   }
 }
 
@@ -344,14 +353,15 @@ extern "C" int dice_moe_forward(const dice_moe_layer_t *L, const void *x, int64_
 extern "C" int dice_profile_enable(int on) {
   using namespace dice;
   if (on && !g_timers.have_events) {
-    for (int i = 0; i <= kStages; ++i) {
-      hipError_t e = hipEventCreate(&g_timers.ev[i]);
-      if (e != hipSuccess) return fail(DICE_ERR_LAUNCH, "dice_profile_enable: %s", hipGetErrorString(e));
-    }
+    for (int r = 0; r < kTimerRing; ++r)
+      for (int i = 0; i <= kStages; ++i) {
+        hipError_t e = hipEventCreate(&g_timers.ev[r][i]);
+        if (e != hipSuccess) return fail(DICE_ERR_LAUNCH, "dice_profile_enable: %s", hipGetErrorString(e));
+      }
     g_timers.have_events = true;
   }
-  g_timers.enabled = on != 0;
-  g_timers.recorded = false;
+  g_timers.mode = on == 2 ? 2 : (on != 0 ? 1 : 0);
+  g_timers.recorded = 0;
   return DICE_OK;
 }
 
@@ -364,13 +374,23 @@ extern "C" const char *dice_profile_stage_name(int i) {
 extern "C" int dice_profile_read(float *ms_out, int n) {
   using namespace dice;
   DICE_REQUIRE(ms_out && n >= kStages, DICE_ERR_BAD_ARG, "dice_profile_read: need room for %d stages", kStages);
-  DICE_REQUIRE(g_timers.enabled && g_timers.recorded, DICE_ERR_BAD_ARG,
+  DICE_REQUIRE(g_timers.mode != 0 && g_timers.recorded > 0, DICE_ERR_BAD_ARG,
                "dice_profile_read: no timed dice_moe_forward call (bf16 path) since dice_profile_enable");
-  hipError_t e = hipEventSynchronize(g_timers.ev[kStages]);
+  const int calls = g_timers.recorded;
+  const int last = (g_timers.next + kTimerRing - 1) % kTimerRing;
+  hipError_t e = hipEventSynchronize(g_timers.ev[last][g_timers.mode == 1 ? kStages : kFc1Stage + 1]);
   if (e != hipSuccess) return fail(DICE_ERR_LAUNCH, "dice_profile_read: %s", hipGetErrorString(e));
-  for (int i = 0; i < kStages; ++i) {
-    e = hipEventElapsedTime(&ms_out[i], g_timers.ev[i], g_timers.ev[i + 1]);
-    if (e != hipSuccess) return fail(DICE_ERR_LAUNCH, "dice_profile_read: %s", hipGetErrorString(e));
+  for (int i = 0; i < kStages; ++i) ms_out[i] = 0.f;
+  for (int c = 0; c < calls; ++c) {
+    const int r = (last + kTimerRing - c) % kTimerRing;
+    for (int i = 0; i < kStages; ++i) {
+      if (g_timers.mode == 2 && i != kFc1Stage) continue;
+      float ms = 0.f;
+      e = hipEventElapsedTime(&ms, g_timers.ev[r][i], g_timers.ev[r][i + 1]);
+      if (e != hipSuccess) return fail(DICE_ERR_LAUNCH, "dice_profile_read: %s", hipGetErrorString(e));
+      ms_out[i] += ms / calls;
+    }
   }
+  g_timers.recorded = 0;
   return DICE_OK;
 }

@@ -217,8 +217,13 @@ int dice_moe_forward(const dice_moe_layer_t *layer, const void *x,
  * layer ("moe.gate", "moe.mlp", "moe.mlp_shared": models.py:305,356,375;
  * cudaprof/prof.py:19-60, expertpara/prof_analyse.py:3-17).  When enabled,
  * dice_moe_forward (bf16 path) records HIP events on the caller's stream
- * between its launches; dice_profile_read waits for the last one and returns
- * the elapsed milliseconds of every stage of the most recent call.
+ * between its launches (a ring of 64 event sets, so that back-to-back calls
+ * need no host synchronisation in between); dice_profile_read waits for the
+ * last one and returns, per stage, the mean elapsed milliseconds over the calls
+ * made since the previous read (the most recent 64 at most).  on = 1 times
+ * every stage; on = 2 only brackets "moe.mlp.fc1" (two events per call, for
+ * timing the dominant launch inside a throughput measurement; the other
+ * stages read as 0).
  */
 int dice_profile_enable(int on);
 int dice_profile_stage_count(void);
