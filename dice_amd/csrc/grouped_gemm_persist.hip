@@ -1,31 +1,36 @@
-// Persistent bf16 grouped GEMM for the expert MLPs (routed experts and the
+// Persistent bf16 grouped GEMMs for the expert MLPs (routed experts and the
 // shared expert in ONE launch per GEMM stage).
 //
-// One workgroup per CU stays resident and walks a list of 256x256 output tiles;
-// the k loop of consecutive tiles forms one continuous software pipeline:
+// One workgroup per CU stays resident and walks a list of 256-row output tiles;
+// the k loop of consecutive tiles forms one continuous software pipeline, so
+// there is no per-tile prologue and no workgroup re-launch between tiles.
+// Operands are addressed through buffer descriptors: the range check zero-fills
+// rows past a group's end and past the last output column, so ragged groups
+// need no special code.  The epilogue applies SwiGLU / GELU / bias, transposes
+// through a small LDS staging area and writes whole row segments with buffer
+// stores (rows past the group's end are dropped by the range check).
 //
-//   * global -> LDS copies (buffer_load_dwordx4 ... lds) run AHEAD = 3 steps of
-//     32 k ahead of the MFMAs in a ring of four 32 KB LDS slots and simply
-//     carry on into the next tile while the current one finishes, so there is
-//     no per-tile prologue and no workgroup re-launch between tiles;
-//   * operands are addressed through buffer descriptors: the descriptor's
-//     range check zero-fills rows past a group's end and past the last output
-//     column, so ragged groups need no special code, and a tile switch only
-//     rewrites a few SGPRs;
-//   * eight waves (two per SIMD) each own a 128x64 block of the tile
-//     (v_mfma_f32_32x32x16_bf16, fp32 accumulate); fragment reads of the next
-//     half step and the copies are threaded between the MFMAs;
-//   * the epilogue applies SwiGLU / GELU / bias, transposes through a small
-//     LDS staging area and writes whole row segments with buffer stores (rows
-//     past the group's end are dropped by the range check).
+// Two pipelines share the tile order and the epilogue; the launcher picks one
+// per launch (persist_variant):
 //
-// Tiles are ordered problem-major, expert-major, then n-tile with the m-tile
-// fastest; each XCD takes one contiguous run of that order so the 32 CUs that
-// share an L2 work on the same expert's weights at the same time.
+//   * 64 k per step, four waves (one per SIMD, 128x128 or 128x96 of the tile
+//     each, accumulators in the accumulation registers), operands staged
+//     through registers four steps ahead and written to one of two 64 KB LDS
+//     slots; optional row table for the activations (the dispatch permutation).
+//     The product path: see the comment above gemm_persist64_body.
+//   * 32 k per step, eight waves (two per SIMD, 128x64 each), global -> LDS
+//     copies (buffer_load_dwordx4 ... lds) three steps ahead in a ring of four
+//     32 KB slots, the two wave groups alternating memory and MFMA phases.
+//     Takes shorter k and any number of tiles per workgroup.
 //
-// Activations must be contiguous grouped rows (the dispatch kernel's gathered
-// copy); weights are [experts, rows, k] bf16 as in the reference's nn.Linear
-// layout (models.py:245-247).
+// Tiles are ordered problem-major (longest k first), expert-major, then n-tile
+// with the m-tile fastest; each XCD takes one contiguous, equally expensive run
+// of that order, so the 32 CUs that share an L2 work on the same expert's
+// weights at the same time.
+//
+// Weights are [experts, rows, k] bf16 as in the reference's nn.Linear layout
+// (models.py:245-247); activations are grouped rows (contiguous, or rows of
+// the token matrix named by a row table).
 #include <type_traits>
 
 #include "gemm_common.h"
@@ -59,49 +64,6 @@ template <int V> using template_int = std::integral_constant<int, V>;
 
 template <int N> __device__ __forceinline__ void pwait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
-template <int I, int N, int RD>
-__device__ __forceinline__ void psched_reads() {
-  if constexpr (I < N) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    __builtin_amdgcn_sched_group_barrier(0x100, (I == N - 1 && (RD & 1)) ? 1 : 2, 0);
-    psched_reads<I + 1, N, RD>();
-  }
-}
-template <int I, int N, int GAP>
-__device__ __forceinline__ void psched_copies() {
-  if constexpr (I < N) {
-    __builtin_amdgcn_sched_group_barrier(0x008, GAP, 0);
-    __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-    psched_copies<I + 1, N, GAP>();
-  }
-}
-// Half a k step: two fragment reads behind each of the first MFMAs, then
-// COPIES copies spread over the remaining MFMAs.
-template <int MF, int RD, int COPIES>
-__device__ __forceinline__ void psched_half() {
-  constexpr int RDG = (RD + 1) / 2;
-  static_assert(MF > RDG, "too few MFMAs to thread the fragment reads through");
-  constexpr int REST = MF - RDG;
-  constexpr int GAP = COPIES > 0 ? (REST / COPIES > 0 ? REST / COPIES : 1) : REST;
-  psched_reads<0, RDG, RD>();
-  psched_copies<0, COPIES, GAP>();
-  constexpr int LEFT = REST - COPIES * GAP;
-  if constexpr (LEFT > 0) __builtin_amdgcn_sched_group_barrier(0x008, LEFT, 0);
-}
-
-// One MFMA stream of MF instructions with RD fragment reads behind the first
-// MFMAs (one each) and CP copies behind every other MFMA after that.
-template <int I, int MF, int RD, int CP>
-__device__ __forceinline__ void psched_stream() {
-  if constexpr (I < MF) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    if constexpr (I < RD) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    if constexpr (I >= RD && (I - RD) % 2 == 0 && (I - RD) / 2 < CP)
-      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-    psched_stream<I + 1, MF, RD, CP>();
-  }
 }
 
 // Pins a wave-uniform value into SGPRs (the compiler cannot always prove uniformity
@@ -146,24 +108,6 @@ struct PackedTile {
 };
 constexpr int kTileWords = 24;   // pointers a, b0, b1, c, bias, ten 32-bit fields, then a_rows, a_magic, rows
 constexpr int kTableTurns = 64;  // turns of one workgroup that the LDS tile table holds
-__device__ __forceinline__ PackedTile pack_tile(const Tile &t, int lane) {
-  const uint64_t p[5] = {(uint64_t)t.a, (uint64_t)t.b0, (uint64_t)t.b1, (uint64_t)t.c, (uint64_t)t.bias};
-  const uint32_t w[10] = {t.a_bytes, t.a_pitch, t.b_bytes, t.b_pitch, t.c_bytes,
-                          t.c_pitch, (uint32_t)t.n0, (uint32_t)t.n, (uint32_t)t.steps, t.valid ? 1u : 0u};
-  uint32_t v = 0;
-#pragma unroll
-  for (int i = 0; i < 5; ++i) {
-    v = lane == 2 * i ? (uint32_t)p[i] : v;
-    v = lane == 2 * i + 1 ? (uint32_t)(p[i] >> 32) : v;
-  }
-#pragma unroll
-  for (int i = 0; i < 10; ++i) v = lane == 10 + i ? w[i] : v;
-  v = lane == 20 ? (uint32_t)(uint64_t)t.a_rows : v;
-  v = lane == 21 ? (uint32_t)((uint64_t)t.a_rows >> 32) : v;
-  v = lane == 22 ? t.a_magic : v;
-  v = lane == 23 ? (uint32_t)t.rows : v;
-  return PackedTile{v};
-}
 __device__ __forceinline__ Tile unpack_tile(const PackedTile &pk) {
   auto word = [&](int i) { return (uint32_t)__builtin_amdgcn_readlane(pk.words, i); };
   auto ptr = [&](int i) { return ((uint64_t)word(2 * i + 1) << 32) | word(2 * i); };

@@ -531,3 +531,38 @@ def test_skip_full_size_identities(dev):
         full2 = blk.run(x2, MODE_PLAIN).clone()
         stale = blk.run(x2, MODE_SKIP, mask, cache, None).clone()
         assert 0 < rel_l2(stale, full2) < 0.2
+
+
+def test_stage_timers_ring_and_fc1_mode(dev):
+    """The CudaProfiler-scope replacement: every stage timed over a run of calls, and the
+    mode that brackets the fc1 launch only."""
+    import ctypes
+    from dice_amd.lib import check, load
+    lib = load()
+    p = O.make_block_params(384, 8, 2, 4, 2, seed=3, dtype=torch.bfloat16, variant="swiglu")
+    x = torch.randn(2, 512, 384, generator=_gen(3)).bfloat16()
+    blk, _ = _run_block(dev, p, x, "swiglu", torch.bfloat16)
+    n = lib.dice_profile_stage_count()
+    names = [lib.dice_profile_stage_name(i).decode() for i in range(n)]
+    assert names == ["moe.gate", "moe.dispatch", "moe.gather", "moe.mlp.fc1", "moe.mlp.fc2", "moe.combine"]
+    buf = (ctypes.c_float * n)()
+    xd = x.view(-1, 384).to(dev)
+    assert lib.dice_profile_read(buf, n) != 0           # not enabled: an error, not garbage
+    check(lib.dice_profile_enable(1))
+    try:
+        assert lib.dice_profile_read(buf, n) != 0       # nothing recorded yet
+        for _ in range(70):                             # more calls than the ring holds
+            blk.run(xd)
+        check(lib.dice_profile_read(buf, n))
+        all_ms = list(buf)
+        assert all(0.0 < v < 50.0 for i, v in enumerate(all_ms) if names[i] != "moe.gather"), all_ms
+        assert lib.dice_profile_read(buf, n) != 0       # the read consumed the record
+        check(lib.dice_profile_enable(2))
+        for _ in range(3):
+            blk.run(xd)
+        check(lib.dice_profile_read(buf, n))
+        fc1 = names.index("moe.mlp.fc1")
+        assert 0.0 < buf[fc1] < 50.0
+        assert all(buf[i] == 0.0 for i in range(n) if i != fc1)
+    finally:
+        check(lib.dice_profile_enable(0))
