@@ -118,10 +118,21 @@ __global__ __launch_bounds__(kGateWaves *kWave) void gate_topk_kernel(
       const int64_t tt = t0 + t < n_tokens ? t0 + t : n_tokens - 1;
       xrow[t] = x + tt * hidden;
     }
-    for (int c = lane; c < chunks; c += kWave) {
-      Vec8<XT> xv[TOK];
+    // The token rows of the next 64-chunk stride are requested before this one is
+    // multiplied, so two rounds of loads are in flight (the kernel is a handful of
+    // dependent memory round trips long; the arithmetic is negligible).
+    Vec8<XT> xv[TOK], xnext[TOK];
+    if (lane < chunks) {
 #pragma unroll
-      for (int t = 0; t < TOK; ++t) xv[t] = load8(xrow[t] + c * 8);
+      for (int t = 0; t < TOK; ++t) xnext[t] = load8(xrow[t] + lane * 8);
+    }
+    for (int c = lane; c < chunks; c += kWave) {
+#pragma unroll
+      for (int t = 0; t < TOK; ++t) xv[t] = xnext[t];
+      if (c + kWave < chunks) {
+#pragma unroll
+        for (int t = 0; t < TOK; ++t) xnext[t] = load8(xrow[t] + (c + kWave) * 8);
+      }
 #pragma unroll
       for (int e = 0; e < EP; ++e) {
         if (e < n_experts) {
