@@ -45,6 +45,13 @@ int fail(int code, const char *fmt, ...);
     if (!(cond)) return ::dice::fail((code), __VA_ARGS__); \
   } while (0)
 
+// Returns DICE_ERR_LAUNCH with the runtime's message when a HIP call fails.
+#define DICE_HIP(call)                                                              \
+  do {                                                                              \
+    hipError_t e_ = (call);                                                         \
+    if (e_ != hipSuccess) return ::dice::fail(DICE_ERR_LAUNCH, "%s: %s", #call, hipGetErrorString(e_)); \
+  } while (0)
+
 // Checks the launch that was just enqueued.
 inline int launch_status(const char *what) {
   hipError_t e = hipGetLastError();

@@ -229,72 +229,119 @@ extern "C" size_t dice_moe_workspace_bytes(const dice_moe_layer_t *layer, int64_
   return dice::carve_layer(layer, n_tokens, nullptr).total;
 }
 
-extern "C" int dice_moe_forward(const dice_moe_layer_t *L, const void *x, int64_t n_tokens,
-                                int mode, const uint8_t *skip_mask, const void *cache_in,
-                                void *cache_out, void *y, int32_t *topk_idx_out,
-                                float *topk_weight_out, void *workspace, size_t workspace_bytes,
-                                void *stream) {
-  using namespace dice;
-  DICE_REQUIRE(L && x && y, DICE_ERR_BAD_ARG, "dice_moe_forward: null pointer");
-  DICE_REQUIRE(mode >= 0 && mode <= 2, DICE_ERR_BAD_ARG, "dice_moe_forward: mode %d", mode);
-  DICE_REQUIRE(L->gate_w && L->w1 && L->w2, DICE_ERR_BAD_ARG, "dice_moe_forward: null weights");
+namespace dice {
+namespace {
+// Shared body of dice_moe_forward and dice_moe_forward_lagged.  `put` receives
+// this call's routing (NULL: it lives in the workspace), `work` names the entry
+// whose routed experts run now and `emit` the entry that is combined into y
+// (NULL: the entry one stage earlier in put -> work -> emit).
+int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_layer_t *LE, const void *x,
+                 int64_t n_tokens, bool drop_skipped, const uint8_t *skip_mask,
+                 dice_moe_lag_entry_t *put, const dice_moe_lag_entry_t *work_in,
+                 const dice_moe_lag_entry_t *emit_in, int combine_mode, const void *cache_in,
+                 void *cache_out, bool use_latest_weights, void *y, int32_t *topk_idx_out,
+                 float *topk_weight_out, void *workspace, size_t workspace_bytes, void *stream) {
+  DICE_REQUIRE(L && x && y, DICE_ERR_BAD_ARG, "%s: null pointer", who);
+  DICE_REQUIRE(combine_mode >= 0 && combine_mode <= 2, DICE_ERR_BAD_ARG, "%s: mode %d", who, combine_mode);
+  DICE_REQUIRE(L->gate_w && LE->w1 && LE->w2, DICE_ERR_BAD_ARG, "%s: null weights", who);
   DICE_REQUIRE(L->top_k >= 1 && L->top_k <= 8 && L->top_k <= L->n_experts, DICE_ERR_BAD_ARG,
-               "dice_moe_forward: top_k %d", L->top_k);
-  int rc = check_mlp_shape("dice_moe_forward", L->act_dtype, L->w_dtype, L->act_variant, L->hidden,
-                           L->inter, L->n_experts);
+               "%s: top_k %d", who, L->top_k);
+  int rc = check_mlp_shape(who, L->act_dtype, LE->w_dtype, LE->act_variant, L->hidden, LE->inter,
+                           L->n_experts);
   if (rc) return rc;
-  DICE_REQUIRE(L->n_experts <= 64, DICE_ERR_UNSUPPORTED, "dice_moe_forward: n_experts %d > 64",
-               L->n_experts);
+  DICE_REQUIRE(L->n_experts <= 64, DICE_ERR_UNSUPPORTED, "%s: n_experts %d > 64", who, L->n_experts);
+  DICE_REQUIRE(LE->hidden == L->hidden && LE->inter == L->inter && LE->n_experts == L->n_experts &&
+                   LE->top_k == L->top_k && LE->act_dtype == L->act_dtype &&
+                   LE->act_variant == L->act_variant,
+               DICE_ERR_BAD_ARG, "%s: the layer whose experts run must have this layer's shape", who);
   if (L->shared_inter > 0) {
     DICE_REQUIRE(L->shared_w1 && L->shared_w2 && L->shared_inter % 64 == 0, DICE_ERR_BAD_ARG,
-                 "dice_moe_forward: shared expert weights / shared_inter %d", L->shared_inter);
+                 "%s: shared expert weights / shared_inter %d", who, L->shared_inter);
   }
-  if (mode == 1) DICE_REQUIRE(skip_mask && cache_out, DICE_ERR_BAD_ARG,
-                              "dice_moe_forward: a put step needs skip_mask and cache_out");
-  if (mode == 2) {
-    DICE_REQUIRE(skip_mask && cache_in, DICE_ERR_BAD_ARG,
-                 "dice_moe_forward: a skip step needs skip_mask and cache_in");
-    DICE_REQUIRE(L->top_k == 2, DICE_ERR_UNSUPPORTED,
-                 "dice_moe_forward: skipping supports top_k == 2 only (got %d)", L->top_k);
-  }
-  DICE_REQUIRE(n_tokens >= 0 && n_tokens * L->top_k < (1ll << 31), DICE_ERR_BAD_ARG,
-               "dice_moe_forward: n_tokens %lld", (long long)n_tokens);
+  if (combine_mode == 1)
+    DICE_REQUIRE(skip_mask && cache_out, DICE_ERR_BAD_ARG, "%s: a put step needs skip_mask and cache_out", who);
+  if (combine_mode == 2)
+    DICE_REQUIRE(skip_mask && cache_in, DICE_ERR_BAD_ARG, "%s: a skip step needs skip_mask and cache_in", who);
+  if (drop_skipped) DICE_REQUIRE(skip_mask, DICE_ERR_BAD_ARG, "%s: dropping slots needs skip_mask", who);
+  if (drop_skipped || combine_mode == 2)
+    DICE_REQUIRE(L->top_k == 2, DICE_ERR_UNSUPPORTED, "%s: skipping supports top_k == 2 only (got %d)",
+                 who, L->top_k);
+  DICE_REQUIRE(n_tokens >= 0 && n_tokens * L->top_k < (1ll << 31), DICE_ERR_BAD_ARG, "%s: n_tokens %lld",
+               who, (long long)n_tokens);
   if (n_tokens == 0) return DICE_OK;
   LayerWorkspace w = carve_layer(L, n_tokens, workspace);
-  DICE_REQUIRE(workspace && workspace_bytes >= w.total, DICE_ERR_WORKSPACE,
-               "dice_moe_forward: workspace %zu < %zu bytes", workspace_bytes, w.total);
+  DICE_REQUIRE(workspace && workspace_bytes >= w.total, DICE_ERR_WORKSPACE, "%s: workspace %zu < %zu bytes",
+               who, workspace_bytes, w.total);
   hipStream_t s = (hipStream_t)stream;
   const int64_t slots = n_tokens * L->top_k;
+  const size_t es = dtype_size(L->act_dtype);
+
+  // This call's own routing entry: in the caller's buffers when it outlives
+  // the call, else in the workspace.
+  dice_moe_lag_entry_t own;
+  if (put) {
+    DICE_REQUIRE(put->x && put->offsets && put->perm && put->inv_perm && put->topk_weight,
+                 DICE_ERR_BAD_ARG, "%s: the entry to fill lacks a buffer", who);
+    own = *put;
+  } else {
+    own.x = nullptr;
+    own.offsets = w.offsets;
+    own.perm = w.perm;
+    own.inv_perm = w.inv_perm;
+    own.topk_weight = topk_weight_out ? topk_weight_out : w.topk_weight;
+    own.rows = w.slot_out;
+  }
+  // A skip step recomputes one slot per token.
+  own.max_rows = drop_skipped ? n_tokens * (L->top_k - 1) : slots;
+  if (put) put->max_rows = own.max_rows;
   int32_t *idx = topk_idx_out ? topk_idx_out : w.topk_idx;
-  float *wt = topk_weight_out ? topk_weight_out : w.topk_weight;
+  float *wt = own.topk_weight;
 
   g_timers.recorded = false;
   stamp(0, s);
   rc = dice_gate_topk(x, L->act_dtype, L->gate_w, L->gate_w_dtype, L->gate_bias, n_tokens, L->hidden,
                       L->n_experts, L->top_k, L->norm_topk_prob, idx, nullptr, wt, nullptr, stream);
   if (rc) return rc;
+  if (put && topk_weight_out)
+    DICE_HIP(hipMemcpyAsync(topk_weight_out, wt, slots * sizeof(float), hipMemcpyDeviceToDevice, s));
   stamp(1, s);
-  rc = dispatch_impl(idx, mode == 2 ? skip_mask : nullptr, slots, L->n_experts, w.counts, w.offsets, w.perm,
-                     w.inv_perm, w.dispatch_ws, w.dispatch_ws_bytes,
+  rc = dispatch_impl(idx, drop_skipped ? skip_mask : nullptr, slots, L->n_experts, w.counts, own.offsets,
+                     own.perm, own.inv_perm, w.dispatch_ws, w.dispatch_ws_bytes,
                      L->shared_inter > 0 ? w.shared_offsets : nullptr, (int32_t)n_tokens, stream);
   if (rc) return rc;
+  if (put && put->x != x)
+    DICE_HIP(hipMemcpyAsync(put->x, x, (size_t)n_tokens * L->hidden * es, hipMemcpyDeviceToDevice, s));
   stamp(2, s);
-  // A skip step recomputes one slot per token.
-  const int64_t max_rows = mode == 2 ? n_tokens * (L->top_k - 1) : slots;
-  const uint8_t *mask = mode == 0 ? nullptr : skip_mask;
 
-  // bf16 path: gather the grouped rows once, then two persistent launches,
-  // each covering the routed experts and the shared expert together.
-  if (L->act_dtype == DICE_BF16 && L->w_dtype == DICE_BF16) {
+  // The entry whose routed experts run in this call.
+  dice_moe_lag_entry_t work = work_in ? *work_in : own;
+  if (!work_in) work.x = const_cast<void *>(x);
+  DICE_REQUIRE(work.x && work.offsets && work.perm && work.rows, DICE_ERR_BAD_ARG,
+               "%s: the entry to run the experts on lacks a buffer", who);
+  DICE_REQUIRE(work.max_rows >= 0 && work.max_rows <= slots, DICE_ERR_BAD_ARG,
+               "%s: entry holds %lld rows, this call at most %lld", who, (long long)work.max_rows,
+               (long long)slots);
+  const dice_moe_lag_entry_t emit = emit_in ? *emit_in : work;
+  DICE_REQUIRE(emit.rows && emit.inv_perm && emit.topk_weight, DICE_ERR_BAD_ARG,
+               "%s: the entry to combine lacks a buffer", who);
+  const int64_t max_rows = work.max_rows;
+  const uint8_t *mask = combine_mode == 0 ? nullptr : skip_mask;
+  const float *combine_wt = use_latest_weights ? wt : emit.topk_weight;
+
+  // bf16 path: two persistent launches, each covering the routed experts and
+  // the shared expert together.
+  bool done = false;
+  if (L->act_dtype == DICE_BF16 && LE->w_dtype == DICE_BF16) {
     const bool swiglu = L->act_variant == DICE_ACT_SWIGLU;
     const int m1 = swiglu ? kFc1Swiglu : kFc1Gelu;
     PersistBatch f1{}, f2{};
-    void *xg = w.slot_out;  // the gathered rows die before fc2 writes its outputs there
-    f1.prob[0] = PersistProblem{xg, L->hidden, w.offsets, L->n_experts, L->w1,
-                                swiglu ? 2 * L->inter : L->inter, L->inter, swiglu ? nullptr : L->b1,
+    void *xg = w.slot_out;  // gathered rows, dead before fc2 could write its outputs there
+    f1.prob[0] = PersistProblem{xg, L->hidden, work.offsets, L->n_experts, LE->w1,
+                                swiglu ? 2 * L->inter : L->inter, L->inter, swiglu ? nullptr : LE->b1,
                                 w.h, L->inter, L->inter, L->hidden, (int)max_rows};
-    f2.prob[0] = PersistProblem{w.h, L->inter, w.offsets, L->n_experts, L->w2, L->hidden, 0,
-                                swiglu ? nullptr : L->b2, w.slot_out, L->hidden, L->hidden, L->inter, (int)max_rows};
+    f2.prob[0] = PersistProblem{w.h, L->inter, work.offsets, L->n_experts, LE->w2, L->hidden, 0,
+                                swiglu ? nullptr : LE->b2, work.rows, L->hidden, L->hidden, L->inter,
+                                (int)max_rows};
     f1.n_problems = f2.n_problems = 1;
     if (L->shared_inter > 0) {
       const int si = L->shared_inter;
@@ -307,8 +354,8 @@ extern "C" int dice_moe_forward(const dice_moe_layer_t *L, const void *x, int64_
     // Where the kernel can address the activation rows through the permutation
     // itself, the gathered copy is skipped.
     PersistBatch f1g = f1;
-    f1g.prob[0].a = x;
-    f1g.prob[0].a_rows = w.perm;
+    f1g.prob[0].a = work.x;
+    f1g.prob[0].a_rows = work.perm;
     f1g.prob[0].a_div = L->top_k;
     f1g.prob[0].a_src_rows = (int)n_tokens;
     const bool fused_gather = persist_supported(f1g, m1) && persist_supported(f2, kFc2);
@@ -316,7 +363,8 @@ extern "C" int dice_moe_forward(const dice_moe_layer_t *L, const void *x, int64_
       if (fused_gather) {
         f1 = f1g;
       } else {
-        rc = gather_rows_impl(x, L->act_dtype, w.perm, L->top_k, max_rows, L->hidden, xg, nullptr, 0, stream);
+        rc = gather_rows_impl(work.x, L->act_dtype, work.perm, L->top_k, max_rows, L->hidden, xg, nullptr, 0,
+                              stream);
         if (rc) return rc;
       }
       stamp(3, s);
@@ -326,28 +374,55 @@ extern "C" int dice_moe_forward(const dice_moe_layer_t *L, const void *x, int64_
       rc = launch_grouped_gemm_persist(f2, kFc2, s);
       if (rc) return rc;
       stamp(5, s);
-      rc = dice_combine(w.slot_out, w.inv_perm, wt, w.shared_out, mask, mode == 2 ? cache_in : nullptr,
-                        mode == 1 ? cache_out : nullptr, y, L->act_dtype, n_tokens, L->top_k, L->hidden,
-                        stream);
-      stamp(6, s);
-      return rc;
+      done = true;
     }
   }
-
-  rc = dice_grouped_mlp(x, L->act_dtype, w.perm, L->top_k, w.offsets, L->n_experts, max_rows,
-                        L->hidden, L->inter, L->w1, L->b1, L->w2, L->b2, L->w1_scale, L->w2_scale,
-                        L->w_dtype, L->act_variant, w.h, w.slot_out, 1, stream);
-  if (rc) return rc;
-  if (L->shared_inter > 0) {
-    rc = dice_grouped_mlp(x, L->act_dtype, nullptr, 1, w.shared_offsets, 1, n_tokens, L->hidden,
-                          L->shared_inter, L->shared_w1, L->shared_b1, L->shared_w2, L->shared_b2,
-                          nullptr, nullptr, L->act_dtype, L->act_variant, w.shared_h, w.shared_out, 0,
-                          stream);
+  if (!done) {
+    rc = dice_grouped_mlp(work.x, L->act_dtype, work.perm, L->top_k, work.offsets, L->n_experts, max_rows,
+                          L->hidden, L->inter, LE->w1, LE->b1, LE->w2, LE->b2, LE->w1_scale, LE->w2_scale,
+                          LE->w_dtype, L->act_variant, w.h, work.rows, 0, stream);
     if (rc) return rc;
+    if (L->shared_inter > 0) {
+      rc = dice_grouped_mlp(x, L->act_dtype, nullptr, 1, w.shared_offsets, 1, n_tokens, L->hidden,
+                            L->shared_inter, L->shared_w1, L->shared_b1, L->shared_w2, L->shared_b2,
+                            nullptr, nullptr, L->act_dtype, L->act_variant, w.shared_h, w.shared_out, 0,
+                            stream);
+      if (rc) return rc;
+    }
   }
-  return dice_combine(w.slot_out, nullptr, wt, w.shared_out, mode == 0 ? nullptr : skip_mask,
-                      mode == 2 ? cache_in : nullptr, mode == 1 ? cache_out : nullptr, y,
-                      L->act_dtype, n_tokens, L->top_k, L->hidden, stream);
+  rc = dice_combine(emit.rows, emit.inv_perm, combine_wt, w.shared_out, mask,
+                    combine_mode == 2 ? cache_in : nullptr, combine_mode == 1 ? cache_out : nullptr, y,
+                    L->act_dtype, n_tokens, L->top_k, L->hidden, stream);
+  if (done) stamp(6, s);
+  return rc;
+}
+}  // namespace
+}  // namespace dice
+
+extern "C" int dice_moe_forward(const dice_moe_layer_t *L, const void *x, int64_t n_tokens,
+                                int mode, const uint8_t *skip_mask, const void *cache_in,
+                                void *cache_out, void *y, int32_t *topk_idx_out,
+                                float *topk_weight_out, void *workspace, size_t workspace_bytes,
+                                void *stream) {
+  DICE_REQUIRE(mode >= 0 && mode <= 2, DICE_ERR_BAD_ARG, "dice_moe_forward: mode %d", mode);
+  return dice::forward_impl("dice_moe_forward", L, L, x, n_tokens, mode == 2, skip_mask, nullptr, nullptr,
+                            nullptr, mode, cache_in, cache_out, false, y, topk_idx_out, topk_weight_out,
+                            workspace, workspace_bytes, stream);
+}
+
+extern "C" int dice_moe_forward_lagged(const dice_moe_layer_t *L, const dice_moe_layer_t *experts_of,
+                                       const void *x, int64_t n_tokens, int drop_skipped,
+                                       const uint8_t *skip_mask, dice_moe_lag_entry_t *put,
+                                       const dice_moe_lag_entry_t *work, const dice_moe_lag_entry_t *emit,
+                                       int combine_mode, const void *cache_in, void *cache_out,
+                                       int use_latest_weights, void *y, int32_t *topk_idx_out,
+                                       float *topk_weight_out, void *workspace, size_t workspace_bytes,
+                                       void *stream) {
+  DICE_REQUIRE(L, DICE_ERR_BAD_ARG, "dice_moe_forward_lagged: null pointer");
+  return dice::forward_impl("dice_moe_forward_lagged", L, experts_of ? experts_of : L, x, n_tokens,
+                            drop_skipped != 0, skip_mask, put, work, emit, combine_mode, cache_in, cache_out,
+                            use_latest_weights != 0, y, topk_idx_out, topk_weight_out, workspace,
+                            workspace_bytes, stream);
 }
 
 extern "C" int dice_profile_enable(int on) {

@@ -1,11 +1,16 @@
-"""Staleness ("conditional communication") control surface of the reference,
-single-GPU part: module-level state with the reference's function names
-(expertpara/diep.py:57-98,112-176) and its per-layer skip cache
-(expertpara/ep_cache.py:188-235).
+"""Staleness control surface of the reference on one GPU: module-level state
+with the reference's function names (expertpara/diep.py:36-176), its per-layer
+skip cache (expertpara/ep_cache.py:188-235) and the dispatch / combine caches
+of its asynchronous expert parallelism (expertpara/diep.py:17-28,184-289;
+expertpara/ep_cache.py:62-186).
 
-The policy is host-side and tiny; the data path (recompute only the retained
-slot of every token, blend with the cached expert output, write the cache on a
-full step) runs inside ``dice_moe_forward``.
+On one GPU every all-to-all of the reference is a copy, so what remains of
+"displaced" and "interweaved" parallelism is the step lag itself: which earlier
+call's routing the experts run on and which earlier call's result is returned.
+That bookkeeping is host-side and tiny and lives here; the data path (recompute
+only the retained slot of every token, blend with the cached expert output,
+write the cache on a full step, run the experts on a stale entry, combine an
+older one) runs inside ``dice_moe_forward`` / ``dice_moe_forward_lagged``.
 """
 from __future__ import annotations
 
@@ -14,6 +19,11 @@ from typing import List, Optional
 import torch
 
 _step = 0
+_forced_sync = False
+_async_pipeline = False
+_selective_async_strategy: Optional[str] = None
+_use_latest_expert_weights: Optional[bool] = None
+max_mem = -1
 _noskip_interval = 1
 _enable_skip = False
 _skip_mode: Optional[str] = None
@@ -54,20 +64,195 @@ class EPSkipCache:
 _diep_cache_skip = EPSkipCache(0)
 
 
+class LagEntry:
+    """One layer call's routing and what it refers to: the value tuple of the
+    reference's dispatch cache (diep.py:17-21) and, once ``rows`` is filled, of
+    its combine cache (diep.py:23-27).  ``x`` is a private copy of the layer
+    input (the reference's ``grouped_dup_inp`` is one too), ``rows`` the
+    grouped, unweighted expert outputs, ``dropped`` says the dispatch left out
+    the skipped slot of every token, ``owner`` is the block whose experts the
+    entry needs."""
+
+    __slots__ = ("x", "offsets", "perm", "inv_perm", "topk_weight", "rows", "max_rows", "dropped", "owner")
+
+    def __init__(self, x, n_experts: int, top_k: int, dropped: bool, owner=None, copy_x: bool = True):
+        n = x.shape[0]
+        dev = x.device
+        self.x = torch.empty_like(x) if copy_x else x
+        self.offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=dev)
+        self.perm = torch.empty(n * top_k, dtype=torch.int32, device=dev)
+        self.inv_perm = torch.empty(n * top_k, dtype=torch.int32, device=dev)
+        self.topk_weight = torch.empty(n * top_k, dtype=torch.float32, device=dev)
+        self.rows = None
+        self.max_rows = n * (top_k - 1) if dropped else n * top_k
+        self.dropped = dropped
+        self.owner = owner
+
+    def ensure_rows(self):
+        if self.rows is None:
+            self.rows = torch.empty((max(self.max_rows, 1), self.x.shape[-1]), dtype=self.x.dtype,
+                                    device=self.x.device)
+        return self.rows
+
+    def desc(self):
+        from .lib import LagEntryDesc, ptr
+        d = LagEntryDesc()
+        d.x, d.offsets, d.perm, d.inv_perm = ptr(self.x), ptr(self.offsets), ptr(self.perm), ptr(self.inv_perm)
+        d.topk_weight, d.rows, d.max_rows = ptr(self.topk_weight), ptr(self.rows), self.max_rows
+        return d
+
+    def tensors(self):
+        return [t for t in (self.x, self.offsets, self.perm, self.inv_perm, self.topk_weight, self.rows)
+                if isinstance(t, torch.Tensor)]
+
+
+class All2AllCache:
+    """One entry per layer; ``get`` leaves the entry in place (reference
+    ep_cache.py:62-118).  There are no handles or send buffers to collect on
+    one GPU, so the reference's ``auto_gc`` has nothing to do here."""
+
+    def __init__(self, capacity: int):
+        self.capacity = capacity
+        self.cache: List[Optional[LagEntry]] = [None] * capacity
+
+    def clear(self):
+        self.cache = [None] * self.capacity
+
+    def put(self, key: int, value: LagEntry):
+        assert isinstance(key, int) and isinstance(value, LagEntry)
+        self.cache[key] = value
+
+    def get(self, key: int) -> LagEntry:
+        assert isinstance(key, int)
+        assert isinstance(self.cache[key], LagEntry), f"no cached step for layer {key}"
+        return self.cache[key]
+
+    def contains(self, key: int) -> bool:
+        assert isinstance(key, int)
+        return self.cache[key] is not None
+
+    def wait(self):
+        """Nothing is in flight on one GPU (reference ep_cache.py:79-85)."""
+
+
+_diep_cache_dispatch = All2AllCache(0)
+_diep_cache_combine = All2AllCache(0)
+
+
 def ep_cache_init(cache_capacity, auto_gc=False, noskip_step=1, skip_mode=None,
                   async_pipeline=False, selective_async_strategy=None):
-    """Reference diep.py:112-158.  ``async_pipeline`` / ``selective_async_strategy``
-    configure the cross-GPU all-to-all caches, which do not exist here."""
+    """Reference diep.py:112-158."""
     global _noskip_interval, _enable_skip, _skip_mode, _diep_cache_skip
-    if async_pipeline or selective_async_strategy is not None:
-        raise NotImplementedError("async all-to-all staleness needs several GPUs")
+    global _async_pipeline, _selective_async_strategy, _diep_cache_dispatch, _diep_cache_combine
+    assert selective_async_strategy in [None, "shallow", "deep", "interleaved", "all"]
+    _selective_async_strategy = selective_async_strategy
+    _async_pipeline = async_pipeline
     _noskip_interval = noskip_step
     _enable_skip = noskip_step != 1
     if _enable_skip:
         assert skip_mode is not None
     _skip_mode = skip_mode
+    _diep_cache_dispatch = All2AllCache(cache_capacity)
+    _diep_cache_combine = All2AllCache(cache_capacity)
     _diep_cache_skip = EPSkipCache(capacity=cache_capacity if _enable_skip else 0)
     _mask_cache.clear()
+
+
+def use_latest_expert_weights(val):
+    """Reference ep_fwd.py:12-15: True scales a lagged result with the routing
+    weights of the current step, False with those cached beside it."""
+    global _use_latest_expert_weights
+    assert val in [True, False], "val must be a boolean"
+    _use_latest_expert_weights = val
+
+
+def latest_expert_weights() -> bool:
+    return bool(_use_latest_expert_weights)
+
+
+def diep_force_sync():
+    """Reference diep.py:100-103: the calls that follow are synchronous and
+    (re)fill the caches; the caller clears them first (rectified_flow.py:100-105)."""
+    global _forced_sync
+    assert not _forced_sync
+    _forced_sync = True
+
+
+def diep_cancel_sync():
+    global _forced_sync
+    assert _forced_sync
+    _forced_sync = False
+
+
+def diep_forced_sync() -> bool:
+    return _forced_sync
+
+
+def ep_wait():
+    _diep_cache_dispatch.wait()
+    _diep_cache_combine.wait()
+
+
+def layer_is_async(ep_async_mode, layer_idx, total_layers) -> bool:
+    """Which layers run step-lagged (reference models.py:328-338)."""
+    if ep_async_mode == "shallow":
+        return layer_idx < total_layers // 2
+    if ep_async_mode == "deep":
+        return layer_idx >= total_layers // 2
+    if ep_async_mode == "all":
+        return True
+    if ep_async_mode == "interleaved":
+        return layer_idx % 2 == 0
+    raise ValueError(f"Invalid ep_async_mode: {ep_async_mode}")
+
+
+def _past_layer_key(key):
+    """Reference diep.py:184-194: the lagged layer that ran before ``key``."""
+    total_layers = _diep_cache_dispatch.capacity
+    if _selective_async_strategy == "all":
+        return (key - 1) % total_layers
+    if _selective_async_strategy == "shallow":
+        return (key - 1) % (total_layers // 2)
+    if _selective_async_strategy == "deep":
+        return (key - 1) % (total_layers // 2) + total_layers // 2
+    if _selective_async_strategy == "interleaved":
+        return (key - 2) % total_layers
+    raise ValueError(f"Unknown selective async strategy: {_selective_async_strategy}")
+
+
+def lag_roles(cache_key: int, new_entry: LagEntry):
+    """Books ``new_entry`` (this call's routing) into the caches and returns
+    ``(work, emit)``: the entry whose experts run in this call and the entry
+    this call returns (reference global_dispatch_async diep.py:196-254 and
+    global_combine_async :256-289).  On a forced-sync step both are the new
+    entry.  Otherwise ``work`` is what the dispatch cache holds for this layer
+    (displaced) or for the previous lagged layer (interweaved), and ``emit`` is
+    what the combine cache holds for this layer; ``work`` takes the combine
+    cache slot of the layer it belongs to."""
+    global max_mem
+    assert cache_key is not None
+    if _forced_sync:
+        assert not _diep_cache_dispatch.contains(cache_key)
+        assert not _diep_cache_combine.contains(cache_key)
+        _diep_cache_dispatch.put(cache_key, new_entry)
+        _diep_cache_combine.put(cache_key, new_entry)
+        return new_entry, new_entry
+    if _async_pipeline:
+        past_key = _past_layer_key(cache_key)
+        assert _diep_cache_dispatch.contains(past_key)
+        assert _diep_cache_combine.contains(cache_key)
+    else:
+        past_key = cache_key
+    work = _diep_cache_dispatch.get(past_key)
+    _diep_cache_dispatch.put(cache_key, new_entry)
+    emit = _diep_cache_combine.get(cache_key)
+    _diep_cache_combine.put(past_key, work)
+    max_mem = max(max_mem, ep_cached_tensors_size())
+    return work, emit
+
+
+def ep_get_max_mem():
+    return max_mem
 
 
 def ep_set_step(step):
@@ -119,6 +304,8 @@ def ep_set_rand_mask(mask: Optional[torch.Tensor]):
 
 
 def ep_cache_clear():
+    _diep_cache_dispatch.clear()
+    _diep_cache_combine.clear()
     _diep_cache_skip.clear()
 
 
@@ -135,8 +322,24 @@ def ep_skip_cached_tensors_size():
     return _diep_cache_skip.tensors_size()
 
 
+def ep_all2all_cached_tensors_size():
+    """Bytes held by the dispatch and combine caches (reference diep.py:44-48).
+    An entry that sits in both caches is counted once; an entry keeps the layer
+    input itself ([N, D]) where the reference keeps its k-fold gathered copy."""
+    seen, total = set(), 0
+    for cache in (_diep_cache_dispatch, _diep_cache_combine):
+        for e in cache.cache:
+            if e is None:
+                continue
+            for t in e.tensors():
+                if id(t) not in seen:
+                    seen.add(id(t))
+                    total += t.element_size() * t.numel()
+    return total
+
+
 def ep_cached_tensors_size():
-    return ep_skip_cached_tensors_size()
+    return ep_all2all_cached_tensors_size() + ep_skip_cached_tensors_size()
 
 
 def ep_forced_sync(i, sample_steps, ep_async_warm_up=0, strided_sync=0, ep_async_cool_down=0):

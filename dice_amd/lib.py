@@ -44,6 +44,7 @@ EXPORTS = [
     "dice_quantize_fp8_rowwise",
     "dice_moe_workspace_bytes",
     "dice_moe_forward",
+    "dice_moe_forward_lagged",
 ]
 
 
@@ -63,6 +64,15 @@ class MoeLayerDesc(Structure):
         ("b1", c_void_p), ("b2", c_void_p), ("w1_scale", c_void_p), ("w2_scale", c_void_p),
         ("shared_w1", c_void_p), ("shared_w2", c_void_p),
         ("shared_b1", c_void_p), ("shared_b2", c_void_p),
+    ]
+
+
+class LagEntryDesc(Structure):
+    """Mirror of ``dice_moe_lag_entry_t``."""
+
+    _fields_ = [
+        ("x", c_void_p), ("offsets", c_void_p), ("perm", c_void_p), ("inv_perm", c_void_p),
+        ("topk_weight", c_void_p), ("rows", c_void_p), ("max_rows", c_int64),
     ]
 
 
@@ -107,6 +117,11 @@ def load() -> ctypes.CDLL:
     lib.dice_moe_forward.restype = c_int
     lib.dice_moe_forward.argtypes = [POINTER(MoeLayerDesc), c_void_p, c_int64, c_int, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]
+    lib.dice_moe_forward_lagged.restype = c_int
+    lib.dice_moe_forward_lagged.argtypes = [POINTER(MoeLayerDesc), POINTER(MoeLayerDesc), c_void_p, c_int64,
+                                            c_int, c_void_p, POINTER(LagEntryDesc), POINTER(LagEntryDesc),
+                                            POINTER(LagEntryDesc), c_int, c_void_p, c_void_p, c_int,
+                                            c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]
     lib.dice_profile_enable.restype = c_int
     lib.dice_profile_enable.argtypes = [c_int]
     lib.dice_profile_stage_count.restype = c_int

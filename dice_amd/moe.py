@@ -22,24 +22,34 @@ from .lib import (DICE_ACT_GELU_TANH, DICE_ACT_SWIGLU, MODE_PLAIN, MODE_PUT, MOD
 
 
 class ParaMode:
-    """Value object of the reference (models.py:34-55), reduced to what the MoE
-    block reads: ``ep`` selects the ``moe_infer_ep`` data flow (and with it the
-    staleness cache); anything that needs a second GPU is refused."""
+    """Value object of the reference (models.py:34-70).  ``ep`` selects the
+    ``moe_infer_ep`` data flow (and with it the staleness caches), ``ep_async``
+    its step-lagged variants; sequence parallelism needs several GPUs and is
+    refused."""
 
-    def __init__(self, ep=False, ep_async=False, sp=False, sp_async=False, **kwargs):
-        if ep_async or sp or sp_async:
-            raise DiceError("async expert parallelism and sequence parallelism need several GPUs "
-                            "and are outside this single-GPU build")
+    def __init__(self, ep=False, ep_async=False, sp=False, sp_async=False, num_sampling_steps=None,
+                 ep_async_warm_up=None, strided_sync=None, ep_async_cool_down=None,
+                 sp_async_warm_up=None, ep_async_mode=None):
+        if sp or sp_async:
+            raise DiceError("sequence parallelism needs several GPUs and is outside this single-GPU build")
         self.ep = ep
-        self.ep_async = False
+        self.ep_async = ep_async
+        if ep_async:
+            assert ep
         self.sp = False
         self.sp_async = False
         self.dp = not ep
-        for k, v in kwargs.items():
-            setattr(self, k, v)
+        self.num_sampling_steps = num_sampling_steps
+        self.ep_async_warm_up = ep_async_warm_up
+        self.strided_sync = strided_sync
+        self.sp_async_warm_up = sp_async_warm_up
+        self.ep_async_cool_down = ep_async_cool_down
+        self.ep_async_mode = ep_async_mode
 
     def verbose(self):
-        return "DP" if self.dp else "EP"
+        if self.dp:
+            return "DP"
+        return "DiEP" if self.ep_async else "EP"
 
 
 class MoEGate(nn.Module):
@@ -262,11 +272,21 @@ class SparseMoeBlock(nn.Module):
             raise DiceError("SparseMoeBlock: only the inference branch is implemented (call .eval())")
         orig_shape = hidden_states.shape
         x = hidden_states.reshape(-1, orig_shape[-1]).contiguous()
-        mode, mask, cache_in, cache_out = MODE_PLAIN, None, None, None
-        if self.para_mode.ep and diep.ep_skip_enabled():
-            # conditional communication: reference models.py:342-353, ep_fwd.py:49-66,176-188
+        if not self.para_mode.ep:
+            return self.run(x).view(*orig_shape)
+        # reference models.py:325-354
+        async_op = bool(self.para_mode.ep_async) and diep.layer_is_async(
+            self.para_mode.ep_async_mode, self.layer_idx, self.total_layers)
+        mask, skip_now = None, None
+        if diep.ep_skip_enabled():
             mask = diep.ep_skip_mask(x.shape[0] * self.num_experts_per_tok).to(x.device)
-            if diep.ep_skip_now(self.layer_idx):
+            skip_now = diep.ep_skip_now(self.layer_idx)
+        if async_op:
+            return self._run_lagged(x, mask, skip_now).view(*orig_shape)
+        mode, cache_in, cache_out = MODE_PLAIN, None, None
+        if mask is not None:
+            # conditional communication: reference ep_fwd.py:49-66,176-188
+            if skip_now:
                 mode, cache_in = MODE_SKIP, diep.ep_skip_get(self.layer_idx)
             else:
                 mode = MODE_PUT
@@ -275,6 +295,47 @@ class SparseMoeBlock(nn.Module):
         if mode == MODE_PUT:
             diep.ep_skip_put(self.layer_idx, cache_out)
         return y.view(*orig_shape)
+
+    @torch.no_grad()
+    def _run_lagged(self, x, mask, skip_now, topk_idx_out=None, topk_weight_out=None):
+        """Step-lagged call (reference ep_fwd.py:133-195 with async_op=True):
+        this call's routing is booked into the caches, the routed experts run on
+        the entry ``diep.lag_roles`` hands back and an older entry is returned.
+        The blend with / write of the skip cache follows the EMITTED entry: it
+        takes the cache when that entry was dispatched without the skipped
+        slots (ep_fwd.py:177-185), else it refills the cache (:186-188)."""
+        desc = self._ensure(x)
+        n = x.shape[0]
+        ws = self._workspace(desc, n, x.device)
+        new = diep.LagEntry(x, len(self.experts), self.num_experts_per_tok, bool(skip_now), owner=self)
+        work, emit = diep.lag_roles(self.layer_idx, new)
+        work.ensure_rows()
+        if emit.rows is None:
+            raise DiceError("the cached step to return has never been through the experts")
+        mode, cache_in, cache_out = MODE_PLAIN, None, None
+        if mask is not None:
+            if emit.dropped:
+                mode, cache_in = MODE_SKIP, diep.ep_skip_get(self.layer_idx)
+                if cache_in is None:
+                    raise DiceError(f"layer {self.layer_idx}: a step dispatched without its skipped slots "
+                                    "came back but the skip cache is empty")
+            else:
+                mode, cache_out = MODE_PUT, torch.empty_like(x)
+            if mask.dtype == torch.bool:
+                mask = mask.view(torch.uint8)
+        owner = work.owner if work.owner is not None else self
+        experts_of = owner._ensure(x)
+        put_d, work_d, emit_d = new.desc(), work.desc(), emit.desc()
+        y = torch.empty_like(x)
+        check(load().dice_moe_forward_lagged(
+            ctypes.byref(desc), ctypes.byref(experts_of), ptr(x), n, int(bool(skip_now)), ptr(mask),
+            ctypes.byref(put_d), None if work is new else ctypes.byref(work_d),
+            None if emit is work else ctypes.byref(emit_d), mode, ptr(cache_in), ptr(cache_out),
+            int(diep.latest_expert_weights()), ptr(y), ptr(topk_idx_out), ptr(topk_weight_out),
+            ptr(ws), ws.numel(), stream_ptr()))
+        if mode == MODE_PUT:
+            diep.ep_skip_put(self.layer_idx, cache_out)
+        return y
 
     @torch.no_grad()
     def run(self, x, mode=MODE_PLAIN, skip_mask=None, cache_in=None, cache_out=None,

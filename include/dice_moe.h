@@ -213,6 +213,56 @@ int dice_moe_forward(const dice_moe_layer_t *layer, const void *x,
                      void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Step-lagged layer call.  Replaces moe_infer_ep with async_op=True
+ * (expertpara/ep_fwd.py:133-172) and the dispatch / combine caches behind
+ * global_dispatch_async / global_combine_async (expertpara/diep.py:17-28,
+ * 196-289) on one GPU, where every all-to-all is a copy and what is left of the
+ * asynchrony is its step lag: the routed experts run on an entry an earlier
+ * call left behind, and the call returns the entry before that one.
+ *
+ * A dice_moe_lag_entry_t is one call's routing and what it refers to; it moves
+ * through three roles, each in a different call unless the caller forces a
+ * synchronous step by leaving `work` and `emit` NULL:
+ *   put  - filled by this call: x (copy of the layer input; may alias x, then
+ *          no copy is made and the caller keeps x unchanged while the entry
+ *          lives), offsets, perm, inv_perm (dice_dispatch tables), topk_weight
+ *          and, on the host, max_rows = n_tokens*top_k, or n_tokens when
+ *          drop_skipped
+ *   work - its routed experts run now: reads x, offsets, perm, max_rows (host
+ *          bound on offsets[n_experts]); writes rows [max_rows, hidden],
+ *          grouped and unweighted
+ *   emit - combined into y: reads rows, inv_perm and, unless
+ *          use_latest_weights, topk_weight (ep_fwd.py:190-193)
+ * NULL roles default to the entry one stage earlier (work = put or the
+ * workspace, emit = work), so all-NULL is dice_moe_forward.
+ *   experts_of    layer whose routed expert weights the `work` entry needs (the
+ *                 interweaved mode runs the previous lagged layer's experts,
+ *                 diep.py:184-194,221-226); NULL = `layer`.  Gate and shared
+ *                 expert always come from `layer` and run on x.
+ *   drop_skipped  this call's dispatch leaves out slots with skip_mask != 0
+ *                 (skip_now of ep_fwd.py:57-66)
+ *   combine_mode  0 plain; 1 also write cache_out from the emitted entry; 2 the
+ *                 emitted entry was produced with drop_skipped: masked slots
+ *                 take cache_in (ep_fwd.py:176-188)
+ */
+typedef struct dice_moe_lag_entry {
+  void *x;
+  int32_t *offsets, *perm, *inv_perm;
+  float *topk_weight;
+  void *rows;
+  int64_t max_rows;
+} dice_moe_lag_entry_t;
+
+int dice_moe_forward_lagged(const dice_moe_layer_t *layer, const dice_moe_layer_t *experts_of,
+                            const void *x, int64_t n_tokens, int drop_skipped,
+                            const uint8_t *skip_mask, dice_moe_lag_entry_t *put,
+                            const dice_moe_lag_entry_t *work, const dice_moe_lag_entry_t *emit,
+                            int combine_mode, const void *cache_in, void *cache_out,
+                            int use_latest_weights, void *y, int32_t *topk_idx_out,
+                            float *topk_weight_out, void *workspace, size_t workspace_bytes,
+                            void *stream);
+
+/*
  * Stage timers.  Replace the reference's CudaProfiler scopes around the MoE
  * layer ("moe.gate", "moe.mlp", "moe.mlp_shared": models.py:305,356,375;
  * cudaprof/prof.py:19-60, expertpara/prof_analyse.py:3-17).  When enabled,

@@ -29,6 +29,19 @@ Pinning status (what independently fixes each function's result):
                           swap symmetry.  The reference never tests its skip
                           path, so beyond these identities it is
                           "parity unpinned" by any reference-held vector.
+* ``moe_infer_ep_async``- the reference's own recipe and assertion
+                          (tests/test_ep.py:79-124, seeds 42/43): after a
+                          forced-sync first step, step 1 returns step 0's
+                          result and step t>=2 returns step t-2's, checked
+                          against the float64 per-token fixtures.  Pipelined
+                          ("interweaved") mode has no reference test; it is
+                          pinned by the closed form its key arithmetic implies
+                          (every lagged layer returns its own result of the
+                          previous step, computed with its own experts), by the
+                          forced-sync step being exact, and by the latest- vs
+                          stale-weight switch changing only the scale factors.
+                          Its combination with the skip cache is exercised only
+                          as a state machine: "parity unpinned".
 * bf16 / fp8 variants   - no reference code or vector exists for them
                           ("parity unpinned" by the reference); they are the
                           same functions evaluated in that dtype.
@@ -353,6 +366,215 @@ def moe_infer_ep_local(
     return expert_out
 
 
+# --------------------------------------------------------------------------- #
+# Step-lagged ("displaced" / "interweaved") expert parallelism on one worker
+# --------------------------------------------------------------------------- #
+class All2AllCache:
+    """Restates ``All2AllCache`` (expertpara/ep_cache.py:62-186) at world size
+    1: one tuple per layer; ``get`` leaves the entry in place (:110-118)."""
+
+    def __init__(self, capacity: int):
+        self.capacity = capacity
+        self.cache: List[Optional[tuple]] = [None] * capacity
+
+    def clear(self):
+        self.cache = [None] * self.capacity
+
+    def put(self, key: int, value: tuple):
+        assert isinstance(key, int)
+        self.cache[key] = value
+
+    def get(self, key: int) -> tuple:
+        assert isinstance(key, int)
+        assert isinstance(self.cache[key][0], torch.Tensor)
+        return self.cache[key]
+
+    def contains(self, key: int) -> bool:
+        return self.cache[key] is not None
+
+
+class DiepState:
+    """The module-level state of expertpara/diep.py (:17-34,100-158) and the
+    ``_use_latest_expert_weights`` switch of expertpara/ep_fwd.py:10-15 as one
+    object: dispatch / combine / skip caches with one entry per layer, the
+    forced-sync flag, the pipeline ("interweaved") switch and the selective
+    strategy that fixes which earlier layer a pipelined layer works for."""
+
+    def __init__(self, cache_capacity: int, noskip_step: int = 1, skip_mode: Optional[str] = None,
+                 async_pipeline: bool = False, selective_async_strategy: Optional[str] = None,
+                 use_latest_expert_weights: Optional[bool] = None):
+        assert selective_async_strategy in [None, "shallow", "deep", "interleaved", "all"]
+        self.selective_async_strategy = selective_async_strategy
+        self.async_pipeline = async_pipeline
+        self.noskip_interval = noskip_step
+        self.enable_skip = noskip_step != 1
+        if self.enable_skip:
+            assert skip_mode is not None
+        self.skip_mode = skip_mode
+        self.dispatch = All2AllCache(cache_capacity)
+        self.combine = All2AllCache(cache_capacity)
+        self.skip = EPSkipCache(cache_capacity if self.enable_skip else 0)
+        self.forced_sync = False
+        self.use_latest_expert_weights = use_latest_expert_weights
+        self.step = 0
+
+    def force_sync(self):  # diep.py:100-103
+        assert not self.forced_sync
+        self.forced_sync = True
+
+    def cancel_sync(self):  # diep.py:105-108
+        assert self.forced_sync
+        self.forced_sync = False
+
+    def cache_clear(self):  # diep.py:160-163
+        self.dispatch.clear()
+        self.combine.clear()
+        self.skip.clear()
+
+    def past_layer_key(self, key: int) -> int:
+        """Restates ``_past_layer_key`` (diep.py:184-194)."""
+        total_layers = self.dispatch.capacity
+        s = self.selective_async_strategy
+        if s == "all":
+            return (key - 1) % total_layers
+        if s == "shallow":
+            return (key - 1) % (total_layers // 2)
+        if s == "deep":
+            return (key - 1) % (total_layers // 2) + total_layers // 2
+        if s == "interleaved":
+            return (key - 2) % total_layers
+        raise ValueError(f"Unknown selective async strategy: {s}")
+
+
+def layer_is_async(mode: Optional[str], layer_idx: int, total_layers: int) -> bool:
+    """Which layers run step-lagged under ``ep_async_mode`` (models.py:328-338)."""
+    if mode == "shallow":
+        return layer_idx < total_layers // 2
+    if mode == "deep":
+        return layer_idx >= total_layers // 2
+    if mode == "all":
+        return True
+    if mode == "interleaved":
+        return layer_idx % 2 == 0
+    raise ValueError(f"Invalid ep_async_mode: {mode}")
+
+
+@torch.no_grad()
+def moe_infer_ep_async(
+    state: DiepState,
+    inp: torch.Tensor,
+    experts: Sequence,
+    flat_expert_indices: torch.Tensor,
+    flat_expert_weights: torch.Tensor,
+    num_experts_per_tok: int,
+    async_op: bool,
+    skip_mask_: Optional[torch.Tensor] = None,
+    skip_now_: Optional[bool] = None,
+    cache_key: int = 0,
+) -> torch.Tensor:
+    """Restates ``moe_infer_ep`` (expertpara/ep_fwd.py:19-197) at world size 1
+    with ``global_dispatch_async`` / ``global_combine_async``
+    (expertpara/diep.py:196-289), every all-to-all reduced to a copy.
+
+    What remains of the asynchrony on one worker is the step lag: outside a
+    forced-sync step the experts run on the dispatch entry an earlier call left
+    behind (same layer one step ago, or the previous pipelined layer), and the
+    call returns the combine entry an earlier call left behind, un-permuted and
+    weighted with ITS routing tables - and with its routing weights too unless
+    ``use_latest_expert_weights`` is set (ep_fwd.py:190-193).
+    """
+    num_total_experts = len(experts)
+    partial_skip = skip_mask_ is not None
+    retain_mask = ~skip_mask_ if partial_skip else None
+    if skip_now_:
+        assert partial_skip, "skip is not enabled"
+        assert num_experts_per_tok == 2, "only support num_experts_per_tok == 2"
+        original_k = num_experts_per_tok
+        num_experts_per_tok //= 2
+        flat_expert_indices = flat_expert_indices[retain_mask]
+        assert flat_expert_indices.size(0) == inp.size(0) * num_experts_per_tok
+    else:
+        original_k = num_experts_per_tok
+
+    counts = flat_expert_indices.bincount()
+    if counts.size(0) != num_total_experts:
+        expanded = torch.zeros(num_total_experts, dtype=counts.dtype)
+        expanded[: counts.size(0)] = counts
+        counts = expanded
+    grouped_idx_dup = flat_expert_indices.argsort(stable=True)
+    grouped_idx = grouped_idx_dup // num_experts_per_tok
+    grouped_dup_inp = torch.index_select(inp, 0, grouped_idx)
+    latest_flat_expert_weights = flat_expert_weights.clone()
+    experts_to_calc = experts
+
+    # global_dispatch_async, diep.py:196-254
+    if async_op:
+        assert cache_key is not None
+        entry = (grouped_dup_inp.clone(), counts, grouped_idx_dup, flat_expert_weights, experts)
+        if state.forced_sync:
+            assert not state.dispatch.contains(cache_key)
+            state.dispatch.put(cache_key, entry)
+            mlp_inp = entry[0]
+        else:
+            if state.async_pipeline:
+                key_to_get = state.past_layer_key(cache_key)
+                assert state.dispatch.contains(key_to_get)
+            else:
+                key_to_get = cache_key
+            mlp_inp, counts, grouped_idx_dup, flat_expert_weights, experts_to_calc = state.dispatch.get(key_to_get)
+            state.dispatch.put(cache_key, entry)
+    else:
+        mlp_inp = grouped_dup_inp
+
+    # proc_experts, ep_fwd.py:200-211
+    mlp_outp = torch.empty_like(mlp_inp)
+    start = 0
+    for e in range(num_total_experts):
+        c = int(counts[e])
+        if c:
+            mlp_outp[start:start + c] = experts_to_calc[e](mlp_inp[start:start + c])
+        start += c
+    assert start == mlp_inp.size(0)
+
+    # global_combine_async, diep.py:256-289
+    grouped_dup_outp = mlp_outp
+    if async_op:
+        if state.forced_sync:
+            assert not state.combine.contains(cache_key)
+            state.combine.put(cache_key, (mlp_outp.clone(), grouped_idx_dup, flat_expert_weights))
+        else:
+            if state.async_pipeline:
+                assert state.combine.contains(cache_key)
+                key_to_put = state.past_layer_key(cache_key)
+            else:
+                key_to_put = cache_key
+            prev = state.combine.get(cache_key)
+            state.combine.put(key_to_put, (mlp_outp.clone(), grouped_idx_dup, flat_expert_weights))
+            grouped_dup_outp, grouped_idx_dup, flat_expert_weights = prev
+
+    # _local_combine, ep_fwd.py:350-354
+    outp_dup = torch.zeros(grouped_dup_outp.size(0), inp.shape[-1], dtype=grouped_dup_outp.dtype)
+    outp_dup.index_copy_(0, grouped_idx_dup, grouped_dup_outp)
+
+    final_outp = outp_dup
+    if partial_skip:
+        if outp_dup.size(0) != inp.size(0) * original_k:
+            assert outp_dup.size(0) == inp.size(0) * original_k // 2
+            dropped = state.skip.get(cache_key)
+            final_outp = outp_dup.new_empty((outp_dup.size(0) * 2, outp_dup.size(1)))
+            final_outp[retain_mask] = outp_dup
+            final_outp[skip_mask_] = dropped
+        else:
+            state.skip.put(cache_key, outp_dup[skip_mask_])
+    if state.use_latest_expert_weights:
+        final_outp = final_outp * latest_flat_expert_weights
+    else:
+        final_outp = final_outp * flat_expert_weights
+    expert_out = final_outp.view(inp.size(0), original_k, inp.size(1)).sum(dim=1)
+    assert expert_out.shape == inp.shape
+    return expert_out
+
+
 @torch.no_grad()
 def dense_moe(x, experts, topk_idx, topk_weight):
     """Per-token brute force: ``y[t] = sum_j w[t,j] * E_{idx[t,j]}(x[t])``.
@@ -440,6 +662,8 @@ def sparse_moe_block_forward(
     cache: Optional[EPSkipCache] = None,
     cache_key: int = 0,
     fp32_gate: bool = True,
+    state: Optional[DiepState] = None,
+    async_op: bool = False,
 ):
     """Restates ``SparseMoeBlock.forward`` inference branch
     (models.py:302-312,321-358): gate -> flatten -> ``moe_infer`` (or the EP
@@ -457,7 +681,17 @@ def sparse_moe_block_forward(
     x = hidden_states.reshape(-1, orig_shape[-1])
     flat_idx = topk_idx.reshape(-1)
     flat_w = topk_weight.to(x.dtype).reshape(-1, 1)
-    if use_ep_path or skip_mask_ is not None:
+    if state is not None:
+        # models.py:325-354: mask / skip decision come from the shared state
+        partial_skip = state.enable_skip
+        mask = None
+        now = None
+        if partial_skip:
+            mask = skip_mask_ if skip_mask_ is not None else skip_mask(flat_idx.size(0), state.skip_mode)
+            now = skip_now(True, state.skip, cache_key, state.step, state.noskip_interval)
+        y = moe_infer_ep_async(state, x, params.experts, flat_idx, flat_w, params.top_k, async_op,
+                               mask, now, cache_key)
+    elif use_ep_path or skip_mask_ is not None:
         y = moe_infer_ep_local(x, params.experts, flat_idx, flat_w, params.top_k,
                                skip_mask_, skip_now_, cache, cache_key)
     else:

@@ -10,7 +10,7 @@ def rel_l2(a: torch.Tensor, b: torch.Tensor) -> float:
 
 
 def block_from_params(p: O.MoEBlockParams, D, variant="swiglu", dtype=torch.float32, device="cuda",
-                      ep=False, layer_idx=0):
+                      ep=False, layer_idx=0, total_layers=1, para_mode=None):
     """Builds the product module and loads the oracle's weights through the
     reference's state-dict key layout."""
     from dice_amd import ParaMode, SparseMoeBlock
@@ -21,8 +21,9 @@ def block_from_params(p: O.MoEBlockParams, D, variant="swiglu", dtype=torch.floa
         si = p.shared.gate_proj.shape[0] if variant == "swiglu" else p.shared.fc1_w.shape[0]
         n_shared = si // D
     blk = SparseMoeBlock(D, mlp_ratio=inter // D, num_experts=E, num_experts_per_tok=p.top_k,
-                         pretraining_tp=1, layer_idx=layer_idx, total_layers=1,
-                         para_mode=ParaMode(ep=ep), variant=variant, n_shared_experts=n_shared)
+                         pretraining_tp=1, layer_idx=layer_idx, total_layers=total_layers,
+                         para_mode=para_mode if para_mode is not None else ParaMode(ep=ep),
+                         variant=variant, n_shared_experts=n_shared)
     sd = {"gate.weight": p.gate_weight}
     def put(prefix, ex):
         if variant == "swiglu":

@@ -84,9 +84,66 @@ def test_module_interface_and_state_dict_keys():
 def test_multi_gpu_modes_are_refused():
     from dice_amd import DiceError, ParaMode
     with pytest.raises(DiceError):
-        ParaMode(ep=True, ep_async=True)
-    with pytest.raises(DiceError):
         ParaMode(sp=True)
+    with pytest.raises(AssertionError):
+        ParaMode(ep_async=True)          # models.py:40-41: async needs ep
+    pm = ParaMode(ep=True, ep_async=True, ep_async_mode="all", ep_async_warm_up=2)
+    assert pm.verbose() == "DiEP" and not pm.dp and pm.ep_async_warm_up == 2
+
+
+@pytest.mark.parametrize("pipeline,strategy", [(False, "all"), (True, "all"), (True, "shallow"),
+                                               (True, "deep"), (True, "interleaved")])
+def test_lag_bookkeeping_matches_oracle_state_machine(pipeline, strategy):
+    """Host side of the step-lagged calls: which cached entry the experts run on
+    and which one is returned must be the ones the oracle's restatement of the
+    reference caches (diep.py:196-289) consumes.  Entries are told apart by a
+    tag stored in their x tensor; the oracle's 'experts' return the tag of the
+    layer that owns them, so a wrong owner shows as well."""
+    from dice_amd import diep
+    from oracle import dice_oracle as O
+    L, E, n, d = 4, 4, 6, 2
+    diep.ep_cache_init(cache_capacity=L, async_pipeline=pipeline, selective_async_strategy=strategy)
+    state = O.DiepState(L, async_pipeline=pipeline, selective_async_strategy=strategy)
+
+    class Tagger:
+        """Expert stand-in: adds 1000 * (owning layer + 1) to its input."""
+        def __init__(self, layer):
+            self.layer = layer
+        def __call__(self, x):
+            return x + 1000.0 * (self.layer + 1)
+
+    idx = torch.arange(2 * n) % E
+    w = torch.ones(2 * n, 1)
+    try:
+        for step in range(5):
+            forced = step in (0, 3)
+            if forced:
+                diep.diep_force_sync()
+                diep.ep_cache_clear()
+                state.force_sync()
+                state.cache_clear()
+            for l in range(L):
+                if not O.layer_is_async(strategy, l, L):
+                    assert not diep.layer_is_async(strategy, l, L)
+                    continue
+                assert diep.layer_is_async(strategy, l, L)
+                tag = float(10 * step + l + 1)
+                x = torch.full((n, d), tag)
+                got = O.moe_infer_ep_async(state, x, [Tagger(l)] * E, idx, w, 2, True, cache_key=l)
+                new = diep.LagEntry(x, E, 2, False, owner=l, copy_x=False)
+                work, emit = diep.lag_roles(l, new)
+                work.rows = work.x + 1000.0 * (work.owner + 1)       # what the kernel call would leave
+                # the oracle returned 2 * (emitted tag + 1000 * (owner + 1)): both slots, weight 1
+                assert torch.equal(got, 2 * emit.rows), (step, l)
+            if forced:
+                diep.diep_cancel_sync()
+                state.cancel_sync()
+        assert diep.ep_all2all_cached_tensors_size() > 0
+        assert diep.ep_get_max_mem() > 0
+    finally:
+        if diep.diep_forced_sync():
+            diep.diep_cancel_sync()
+        diep.ep_cache_init(cache_capacity=1)
 
 
 def test_skip_policy_matches_oracle():

@@ -229,3 +229,114 @@ def test_fp8_rowwise_quantiser_properties():
     assert rel.max() <= 2 ** -4 + 1e-6
     big = w.abs() > amax[:, None] / 16
     assert ((deq - w).abs()[big] <= w.abs()[big] * 2 ** -4 + 1e-9).all()
+
+
+# --------------------------------------------------------------------------- #
+# step-lagged expert parallelism (displaced / interweaved) on one worker
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("seed", [42, 43])
+def test_displaced_lag_matches_reference_recipe(golden_dir, seed):
+    """tests/test_ep.py:79-124 with async_op=True: iteration 0 is a forced-sync
+    step, iteration 1 returns iteration 0's result and iteration t >= 2 returns
+    iteration t-2's; expected values are the float64 per-token fixtures."""
+    z = np.load(os.path.join(golden_dir, f"ep_recipe_seed{seed}.npz"))
+    experts = [LinearExpert(z["expert_w"][e], z["expert_b"][e]) for e in range(8)]
+    state = O.DiepState(1)
+    for it in range(4):
+        if it == 0:
+            state.force_sync()
+        elif it == 1:
+            state.cancel_sync()
+        x = torch.from_numpy(z[f"inp{it}"])
+        idx = torch.from_numpy(z[f"idx{it}"])
+        w = torch.from_numpy(z[f"w{it}"])
+        got = O.moe_infer_ep_async(state, x, experts, idx, w, 2, True, cache_key=0)
+        src = 0 if it < 2 else it - 2
+        want = torch.from_numpy(z[f"y{src}"]).float()
+        assert torch.allclose(got, want, atol=1e-6, rtol=1e-5), (it, src)
+
+
+def _per_token(x, experts, idx, w, idx_for_experts=None):
+    """float64 numpy definition y[t] = sum_j w[t,j] * E_{idx[t,j]}(x[t]) for
+    LinearExpert lists."""
+    x64 = x.double().numpy()
+    n = x.shape[0]
+    y = np.zeros((n, x.shape[1]))
+    ids = idx if idx_for_experts is None else idx_for_experts
+    for t in range(n):
+        for j in range(2):
+            e = experts[int(ids[2 * t + j])]
+            y[t] += float(w[2 * t + j]) * (e.w.double().numpy() @ x64[t] + e.b.double().numpy())
+    return torch.from_numpy(y).float()
+
+
+def _rand_linear_experts(gen, n, d):
+    return [LinearExpert(torch.rand(d, d, generator=gen).numpy(), torch.rand(d, generator=gen).numpy())
+            for _ in range(n)]
+
+
+@pytest.mark.parametrize("strategy", ["all", "shallow", "deep", "interleaved"])
+@pytest.mark.parametrize("latest", [False, True])
+def test_interweaved_lag_closed_form(strategy, latest):
+    """Pipelined mode: a lagged layer returns its own previous-step result
+    (own experts, own previous input, previous routing; the routing WEIGHTS are
+    the current ones iff use_latest_expert_weights), layers outside the
+    selective strategy stay exact, and a forced-sync step is exact everywhere."""
+    L, n, d, E = 4, 24, 12, 4
+    gen = torch.Generator().manual_seed(3)
+    layers = [_rand_linear_experts(gen, E, d) for _ in range(L)]
+    state = O.DiepState(L, async_pipeline=True, selective_async_strategy=strategy,
+                        use_latest_expert_weights=latest)
+    hist = []
+    for step in range(4):
+        forced = step == 0
+        if forced:
+            state.force_sync()
+            state.cache_clear()
+        cur = []
+        for l in range(L):
+            x = torch.randn(n, d, generator=gen)
+            idx = torch.randint(0, E, (2 * n,), generator=gen)
+            w = torch.rand(2 * n, 1, generator=gen)
+            cur.append((x, idx, w))
+            lagged = O.layer_is_async(strategy, l, L)
+            got = O.moe_infer_ep_async(state, x, layers[l], idx, w, 2, lagged, cache_key=l)
+            if forced or not lagged:
+                want = _per_token(x, layers[l], idx, w)
+            else:
+                px, pidx, pw = hist[-1][l]
+                want = _per_token(px, layers[l], pidx, w if latest else pw)
+            assert torch.allclose(got, want, atol=1e-5, rtol=1e-5), (step, l)
+        hist.append(cur)
+        if forced:
+            state.cancel_sync()
+
+
+def test_displaced_with_skip_cache_state_machine():
+    """Displaced lag together with conditional communication, interval 2, on
+    the reference schedule: the sizes that flow through the caches stay
+    consistent (every call returns [N, D]) and, because the lag of two steps
+    preserves the full/skip parity, a skip-step entry always meets a skip cache
+    entry.  Values: with identical inputs every step the lagged result equals
+    the synchronous full result."""
+    n, d, E = 16, 8, 4
+    gen = torch.Generator().manual_seed(5)
+    experts = _rand_linear_experts(gen, E, d)
+    x = torch.randn(n, d, generator=gen)
+    idx = torch.stack([torch.randperm(E, generator=gen)[:2] for _ in range(n)]).reshape(-1)
+    w = torch.rand(2 * n, 1, generator=gen)
+    want = _per_token(x, experts, idx, w)
+    state = O.DiepState(1, noskip_step=2, skip_mode="low")
+    mask = O.skip_mask(2 * n, "low")
+    for i in range(10, 0, -1):
+        state.step = i
+        forced = i == 10
+        if forced:
+            state.force_sync()
+            state.cache_clear()
+        now = O.skip_now(True, state.skip, 0, i, 2)
+        got = O.moe_infer_ep_async(state, x, experts, idx, w, 2, True, mask, now, 0)
+        if forced:
+            state.cancel_sync()
+        assert got.shape == x.shape
+        assert torch.allclose(got, want, atol=1e-5, rtol=1e-5), i
