@@ -29,15 +29,15 @@ FC1_HBM_TRAFFIC_BYTES = 1.148e9
 N_TOKENS, D, E, TOPK, RATIO = 8192, 1152, 8, 2, 4
 
 
-def make_block(variant, dev):
+def make_block(variant, dev, layer_idx=0, total_layers=1, para_mode=None):
     """Seeded synthetic weights: router N(0, 0.02), experts Xavier-uniform."""
     from dice_amd import ParaMode, SparseMoeBlock
     # swiglu: the reference's shared expert (one SwiGLU MLP of width 2D, models.py:292-296);
     # gelu_tanh: two always-on experts of the routed shape = one MLP of width 2*4D.
     n_shared = 2 if variant == "swiglu" else 2 * RATIO
-    torch.manual_seed(0)
-    blk = SparseMoeBlock(D, RATIO, E, TOPK, pretraining_tp=1, layer_idx=0, total_layers=1,
-                         para_mode=ParaMode(), variant=variant, n_shared_experts=n_shared)
+    torch.manual_seed(layer_idx)
+    blk = SparseMoeBlock(D, RATIO, E, TOPK, pretraining_tp=1, layer_idx=layer_idx, total_layers=total_layers,
+                         para_mode=para_mode or ParaMode(), variant=variant, n_shared_experts=n_shared)
     for m in blk.modules():
         if isinstance(m, torch.nn.Linear):
             torch.nn.init.xavier_uniform_(m.weight)
@@ -134,6 +134,39 @@ def time_stages(blk, x, steps):
     return {names[i]: acc[i] / steps for i in range(n)}
 
 
+def time_lagged(variant, dev, x, steps, warmup, pipeline):
+    """ms per layer call of the step-lagged modes on the same block shape: two
+    layers, a forced-sync first step, then `steps` lagged steps (displaced: each
+    layer two steps behind itself; interweaved: each layer runs the other one's
+    experts and is one step behind).  Includes the per-call copy of the layer
+    input and the allocation of the cached entry on the host side."""
+    from dice_amd import ParaMode, diep
+    pm = ParaMode(ep=True, ep_async=True, ep_async_mode="all")
+    blks = [make_block(variant, dev, l, 2, pm) for l in range(2)]
+    diep.ep_cache_init(cache_capacity=2, async_pipeline=pipeline, selective_async_strategy="all")
+    diep.use_latest_expert_weights(True)
+    xv = x.view(1, N_TOKENS, D)
+    try:
+        diep.diep_force_sync()
+        diep.ep_cache_clear()
+        for b in blks:
+            b(xv)
+        diep.diep_cancel_sync()
+        for _ in range(warmup):
+            for b in blks:
+                b(xv)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            for b in blks:
+                b(xv)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / (steps * len(blks)) * 1e3
+    finally:
+        diep.ep_cache_init(cache_capacity=1)
+        diep.use_latest_expert_weights(False)
+
+
 def cpu_baseline(variant, budget_s=20.0):
     """The oracle (a torch restatement of the reference block) timed on the
     host cores on a bounded token sample of the same workload."""
@@ -177,6 +210,7 @@ def main():
     ap.add_argument("--fc2-cfg", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-stages", action="store_true", help="skip the per-kernel timing pass")
+    ap.add_argument("--no-lagged", action="store_true", help="skip the step-lagged (displaced / interweaved) pass")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a known-size kernel to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
@@ -252,6 +286,11 @@ def main():
                "moe.combine": (slots * D + 2 * N_TOKENS * D) * bf + slots * 8}
         out["hbm_stage_gbs"] = {s: hbm[s] / (st[s] * 1e-3) / 1e9 for s in hbm}
         out["hbm_stage_frac_of_peak"] = {s: v / PEAK_HBM_GBS for s, v in out["hbm_stage_gbs"].items()}
+    if not args.no_lagged:
+        # the same layer under the reference's step-lagged schedules (not part of `value`)
+        out["step_lag_ms_per_layer_call"] = {
+            "displaced": time_lagged(args.variant, dev, x, args.steps, args.warmup, False),
+            "interweaved": time_lagged(args.variant, dev, x, args.steps, args.warmup, True)}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.variant)
     print(json.dumps(out))
