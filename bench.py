@@ -167,6 +167,43 @@ def time_lagged(variant, dev, x, steps, warmup, pipeline):
         diep.use_latest_expert_weights(False)
 
 
+def time_caller(blk, x, steps, warmup):
+    """The MoE line of the reference's DiTBlock.forward, x + gate * moe(modulate(norm2(x))),
+    on 32 samples x 256 tokens: ms per call with the prologue / epilogue inside the library,
+    with them as torch eager ops around the plain layer call (what the reference's DiTBlock
+    does), and the prologue kernel alone with its share of the 8 TB/s HBM peak."""
+    import torch.nn.functional as F
+    from dice_amd import ops
+    B, T = 32, N_TOKENS // 32
+    g = torch.Generator().manual_seed(1)
+    xs = x.view(B, T, D)
+    shift, scale, gate = ((torch.randn(B, D, generator=g) * 0.3).bfloat16().to(x.device) for _ in range(3))
+    out = torch.empty_like(xs)
+
+    def fused():
+        blk.forward_modulated(xs, shift, scale, gate, out=out)
+
+    def eager():
+        h = F.layer_norm(xs, (D,), None, None, 1e-6) * (1 + scale.unsqueeze(1)) + shift.unsqueeze(1)
+        return xs + gate.unsqueeze(1) * blk(h)
+
+    def prologue():
+        ops.ln_modulate(xs, shift, scale)
+
+    res = {}
+    for name, fn in (("fused", fused), ("eager_caller", eager), ("ln_modulate_kernel", prologue)):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        res[name] = (time.perf_counter() - t0) / steps * 1e3
+    res["ln_modulate_frac_of_hbm_peak"] = 2 * N_TOKENS * D * 2 / (res["ln_modulate_kernel"] * 1e-3) / 1e9 / PEAK_HBM_GBS
+    return res
+
+
 def cpu_baseline(variant, budget_s=20.0):
     """The oracle (a torch restatement of the reference block) timed on the
     host cores on a bounded token sample of the same workload."""
@@ -210,6 +247,7 @@ def main():
     ap.add_argument("--fc2-cfg", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-stages", action="store_true", help="skip the per-kernel timing pass")
+    ap.add_argument("--no-caller", action="store_true", help="skip the fused-caller (LayerNorm/modulate + residual) pass")
     ap.add_argument("--no-lagged", action="store_true", help="skip the step-lagged (displaced / interweaved) pass")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a known-size kernel to scale "
@@ -286,6 +324,8 @@ def main():
                "moe.combine": (slots * D + 2 * N_TOKENS * D) * bf + slots * 8}
         out["hbm_stage_gbs"] = {s: hbm[s] / (st[s] * 1e-3) / 1e9 for s in hbm}
         out["hbm_stage_frac_of_peak"] = {s: v / PEAK_HBM_GBS for s, v in out["hbm_stage_gbs"].items()}
+    if not args.no_caller:
+        out["block_moe_half_ms"] = time_caller(blk, x, args.steps, args.warmup)
     if not args.no_lagged:
         # the same layer under the reference's step-lagged schedules (not part of `value`)
         out["step_lag_ms_per_layer_call"] = {

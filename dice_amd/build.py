@@ -22,6 +22,7 @@ SOURCES = [
     "gate.hip",
     "dispatch.hip",
     "combine.hip",
+    "modulate.hip",
     "quant.hip",
     "grouped_gemm_f32.hip",
     "grouped_gemm_bf16.hip",

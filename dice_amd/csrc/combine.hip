@@ -11,6 +11,12 @@
 // and writes y (and the cache row on a "put" step).  Accumulation is fp32 in
 // slot order with a single rounding, no atomics, so the result is
 // deterministic.
+//
+// Optionally also the caller's epilogue, out = resid + gate[b] * y
+// (x + gate_mlp.unsqueeze(1) * self.moe(...) of DiTBlock.forward, reference
+// models.py:519; b = token / tokens_per_sample), applied to the fp32 sum before
+// the one rounding: two more reads per element instead of the reference's two
+// extra elementwise kernels over [N, D].
 #include "common.h"
 
 namespace dice {
@@ -44,7 +50,8 @@ __global__ __launch_bounds__(256) void combine_kernel(
     const float *__restrict__ topk_weight, const Pack<T> *__restrict__ shared_out,
     const uint8_t *__restrict__ skip_mask, const Pack<T> *__restrict__ cache_in,
     Pack<T> *__restrict__ cache_out, Pack<T> *__restrict__ y, int64_t n_tokens, int top_k,
-    int vec_per_row) {
+    int vec_per_row, const Pack<T> *__restrict__ resid, const Pack<T> *__restrict__ gate,
+    int64_t tokens_per_sample) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n_tokens * vec_per_row) return;
   const int64_t t = i / vec_per_row;
@@ -72,6 +79,12 @@ __global__ __launch_bounds__(256) void combine_kernel(
 #pragma unroll
     for (int e = 0; e < Pack<T>::kN; ++e) acc[e] += sh.get(e);
   }
+  if (resid) {
+    const Pack<T> r = resid[i];
+    const Pack<T> g = gate[(t / tokens_per_sample) * vec_per_row + c];
+#pragma unroll
+    for (int e = 0; e < Pack<T>::kN; ++e) acc[e] = fmaf(g.get(e), acc[e], r.get(e));
+  }
   Pack<T> o;
 #pragma unroll
   for (int e = 0; e < Pack<T>::kN; ++e) o.set(e, acc[e]);
@@ -82,26 +95,23 @@ template <typename T>
 int launch_combine(const void *slot_out, const int32_t *inv_perm, const float *w,
                    const void *shared_out, const uint8_t *skip, const void *cache_in,
                    void *cache_out, void *y, int64_t n_tokens, int top_k, int hidden,
-                   hipStream_t s) {
+                   const void *resid, const void *gate, int64_t tokens_per_sample, hipStream_t s) {
   const int vec_per_row = hidden / Pack<T>::kN;
   const int64_t total = n_tokens * vec_per_row;
   const int64_t blocks = (total + 255) / 256;
   hipLaunchKernelGGL(combine_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s,
                      (const Pack<T> *)slot_out, inv_perm, w, (const Pack<T> *)shared_out, skip,
                      (const Pack<T> *)cache_in, (Pack<T> *)cache_out, (Pack<T> *)y, n_tokens, top_k,
-                     vec_per_row);
+                     vec_per_row, (const Pack<T> *)resid, (const Pack<T> *)gate, tokens_per_sample);
   return launch_status("dice_combine");
 }
 
 }  // namespace
-}  // namespace dice
 
-extern "C" int dice_combine(const void *slot_out, const int32_t *inv_perm,
-                            const float *topk_weight, const void *shared_out,
-                            const uint8_t *skip_mask, const void *cache_in, void *cache_out,
-                            void *y, int dtype, int64_t n_tokens, int top_k, int hidden,
-                            void *stream) {
-  using namespace dice;
+int combine_impl(const void *slot_out, const int32_t *inv_perm, const float *topk_weight,
+                 const void *shared_out, const uint8_t *skip_mask, const void *cache_in, void *cache_out,
+                 void *y, int dtype, int64_t n_tokens, int top_k, int hidden, const void *resid,
+                 const void *gate, int64_t tokens_per_sample, void *stream) {
   DICE_REQUIRE(slot_out && topk_weight && y, DICE_ERR_BAD_ARG, "dice_combine: null pointer");
   DICE_REQUIRE(top_k >= 1 && top_k <= kMaxTopK, DICE_ERR_BAD_ARG, "dice_combine: top_k %d outside [1, %d]",
                top_k, kMaxTopK);
@@ -109,6 +119,9 @@ extern "C" int dice_combine(const void *slot_out, const int32_t *inv_perm,
                "dice_combine: a cache pointer needs skip_mask");
   DICE_REQUIRE(!(cache_in && cache_out), DICE_ERR_BAD_ARG,
                "dice_combine: a step either reads (skip) or writes (put) the cache, not both");
+  DICE_REQUIRE(!resid == !gate, DICE_ERR_BAD_ARG, "dice_combine: residual and gate come together");
+  DICE_REQUIRE(!resid || tokens_per_sample >= 1, DICE_ERR_BAD_ARG,
+               "dice_combine: tokens_per_sample %lld < 1", (long long)tokens_per_sample);
   const size_t es = dtype_size(dtype);
   DICE_REQUIRE(es == 2 || es == 4, DICE_ERR_UNSUPPORTED, "dice_combine: dtype %d", dtype);
   DICE_REQUIRE(hidden > 0 && ((size_t)hidden * es) % 16 == 0, DICE_ERR_BAD_ARG,
@@ -118,13 +131,36 @@ extern "C" int dice_combine(const void *slot_out, const int32_t *inv_perm,
   switch (dtype) {
     case DICE_F32:
       return launch_combine<float>(slot_out, inv_perm, topk_weight, shared_out, skip_mask, cache_in,
-                                   cache_out, y, n_tokens, top_k, hidden, s);
+                                   cache_out, y, n_tokens, top_k, hidden, resid, gate, tokens_per_sample, s);
     case DICE_BF16:
       return launch_combine<bf16_t>(slot_out, inv_perm, topk_weight, shared_out, skip_mask, cache_in,
-                                    cache_out, y, n_tokens, top_k, hidden, s);
+                                    cache_out, y, n_tokens, top_k, hidden, resid, gate, tokens_per_sample, s);
     case DICE_F16:
       return launch_combine<f16_t>(slot_out, inv_perm, topk_weight, shared_out, skip_mask, cache_in,
-                                   cache_out, y, n_tokens, top_k, hidden, s);
+                                   cache_out, y, n_tokens, top_k, hidden, resid, gate, tokens_per_sample, s);
   }
   return fail(DICE_ERR_UNSUPPORTED, "dice_combine: dtype %d", dtype);
+}
+
+}  // namespace dice
+
+extern "C" int dice_combine(const void *slot_out, const int32_t *inv_perm,
+                            const float *topk_weight, const void *shared_out,
+                            const uint8_t *skip_mask, const void *cache_in, void *cache_out,
+                            void *y, int dtype, int64_t n_tokens, int top_k, int hidden,
+                            void *stream) {
+  return dice::combine_impl(slot_out, inv_perm, topk_weight, shared_out, skip_mask, cache_in, cache_out, y,
+                            dtype, n_tokens, top_k, hidden, nullptr, nullptr, 1, stream);
+}
+
+extern "C" int dice_combine_residual(const void *slot_out, const int32_t *inv_perm,
+                                     const float *topk_weight, const void *shared_out,
+                                     const uint8_t *skip_mask, const void *cache_in, void *cache_out,
+                                     const void *resid, const void *gate, int64_t tokens_per_sample,
+                                     void *out, int dtype, int64_t n_tokens, int top_k, int hidden,
+                                     void *stream) {
+  using namespace dice;
+  DICE_REQUIRE(resid && gate, DICE_ERR_BAD_ARG, "dice_combine_residual: null pointer");
+  return combine_impl(slot_out, inv_perm, topk_weight, shared_out, skip_mask, cache_in, cache_out, out, dtype,
+                      n_tokens, top_k, hidden, resid, gate, tokens_per_sample, stream);
 }

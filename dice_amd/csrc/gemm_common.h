@@ -147,6 +147,15 @@ bool persist_supported(const PersistBatch &b, int mode);
 bool gemm_config_wants_persistent();  // tuning hook state: both stages set to the persistent kernel
 int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s);
 
+// LayerNorm + adaLN modulation in front of the layer, and the combine with the
+// caller's residual / gate epilogue behind it (modulate.hip, combine.hip).
+int ln_modulate_impl(const void *x, const void *shift, const void *scale, void *out, int dtype,
+                     int64_t n_tokens, int hidden, int64_t tokens_per_sample, float eps, void *stream);
+int combine_impl(const void *slot_out, const int32_t *inv_perm, const float *topk_weight,
+                 const void *shared_out, const uint8_t *skip_mask, const void *cache_in, void *cache_out,
+                 void *y, int dtype, int64_t n_tokens, int top_k, int hidden, const void *resid,
+                 const void *gate, int64_t tokens_per_sample, void *stream);
+
 int dispatch_impl(const int32_t *flat_idx, const uint8_t *skip_mask, int64_t n_slots, int n_experts,
                   int32_t *counts, int32_t *offsets, int32_t *perm, int32_t *inv_perm, void *workspace,
                   size_t workspace_bytes, int32_t *range_out, int32_t range_n, void *stream);

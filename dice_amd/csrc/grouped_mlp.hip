@@ -27,7 +27,7 @@ struct LayerWorkspace {
   int32_t *counts, *offsets, *perm, *inv_perm;
   void *dispatch_ws;
   size_t dispatch_ws_bytes;
-  void *h, *slot_out, *shared_h, *shared_out;
+  void *h, *slot_out, *shared_h, *shared_out, *modulated;
   int32_t *shared_offsets;
   size_t total;
 };
@@ -54,6 +54,7 @@ LayerWorkspace carve_layer(const dice_moe_layer_t *L, int64_t n_tokens, void *ws
   } else {
     w.shared_h = w.shared_out = nullptr;
   }
+  w.modulated = c.take_bytes((size_t)n_tokens * L->hidden * es);  // layer input when the caller's prologue runs here
   w.total = c.used;
   return w;
 }
@@ -239,9 +240,13 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
                  int64_t n_tokens, bool drop_skipped, const uint8_t *skip_mask,
                  dice_moe_lag_entry_t *put, const dice_moe_lag_entry_t *work_in,
                  const dice_moe_lag_entry_t *emit_in, int combine_mode, const void *cache_in,
-                 void *cache_out, bool use_latest_weights, void *y, int32_t *topk_idx_out,
-                 float *topk_weight_out, void *workspace, size_t workspace_bytes, void *stream) {
+                 void *cache_out, bool use_latest_weights, const dice_moe_caller_t *caller, void *y,
+                 int32_t *topk_idx_out, float *topk_weight_out, void *workspace, size_t workspace_bytes,
+                 void *stream) {
   DICE_REQUIRE(L && x && y, DICE_ERR_BAD_ARG, "%s: null pointer", who);
+  if (caller)
+    DICE_REQUIRE(caller->shift && caller->scale && caller->gate && caller->tokens_per_sample >= 1,
+                 DICE_ERR_BAD_ARG, "%s: the caller's shift / scale / gate or tokens_per_sample", who);
   DICE_REQUIRE(combine_mode >= 0 && combine_mode <= 2, DICE_ERR_BAD_ARG, "%s: mode %d", who, combine_mode);
   DICE_REQUIRE(L->gate_w && LE->w1 && LE->w2, DICE_ERR_BAD_ARG, "%s: null weights", who);
   DICE_REQUIRE(L->top_k >= 1 && L->top_k <= 8 && L->top_k <= L->n_experts, DICE_ERR_BAD_ARG,
@@ -299,6 +304,19 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
 
   g_timers.recorded = false;
   stamp(0, s);
+  // With the caller's prologue the layer input is LN(x) modulated, written
+  // straight into the entry that outlives the call when there is one; x itself
+  // is then only the residual of the epilogue.
+  const void *resid = nullptr;
+  if (caller) {
+    void *hm = put ? put->x : w.modulated;
+    DICE_REQUIRE(hm != x, DICE_ERR_BAD_ARG, "%s: the entry's input buffer aliases x", who);
+    rc = ln_modulate_impl(x, caller->shift, caller->scale, hm, L->act_dtype, n_tokens, L->hidden,
+                          caller->tokens_per_sample, caller->ln_eps, stream);
+    if (rc) return rc;
+    resid = x;
+    x = hm;
+  }
   rc = dice_gate_topk(x, L->act_dtype, L->gate_w, L->gate_w_dtype, L->gate_bias, n_tokens, L->hidden,
                       L->n_experts, L->top_k, L->norm_topk_prob, idx, nullptr, wt, nullptr, stream);
   if (rc) return rc;
@@ -390,9 +408,10 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
       if (rc) return rc;
     }
   }
-  rc = dice_combine(emit.rows, emit.inv_perm, combine_wt, w.shared_out, mask,
+  rc = combine_impl(emit.rows, emit.inv_perm, combine_wt, w.shared_out, mask,
                     combine_mode == 2 ? cache_in : nullptr, combine_mode == 1 ? cache_out : nullptr, y,
-                    L->act_dtype, n_tokens, L->top_k, L->hidden, stream);
+                    L->act_dtype, n_tokens, L->top_k, L->hidden, resid, caller ? caller->gate : nullptr,
+                    caller ? caller->tokens_per_sample : 1, stream);
   if (done) stamp(6, s);
   return rc;
 }
@@ -406,8 +425,20 @@ extern "C" int dice_moe_forward(const dice_moe_layer_t *L, const void *x, int64_
                                 void *stream) {
   DICE_REQUIRE(mode >= 0 && mode <= 2, DICE_ERR_BAD_ARG, "dice_moe_forward: mode %d", mode);
   return dice::forward_impl("dice_moe_forward", L, L, x, n_tokens, mode == 2, skip_mask, nullptr, nullptr,
-                            nullptr, mode, cache_in, cache_out, false, y, topk_idx_out, topk_weight_out,
-                            workspace, workspace_bytes, stream);
+                            nullptr, mode, cache_in, cache_out, false, nullptr, y, topk_idx_out,
+                            topk_weight_out, workspace, workspace_bytes, stream);
+}
+
+extern "C" int dice_moe_forward_modulated(const dice_moe_layer_t *L, const dice_moe_caller_t *caller,
+                                          const void *x, int64_t n_tokens, int mode,
+                                          const uint8_t *skip_mask, const void *cache_in, void *cache_out,
+                                          void *out, int32_t *topk_idx_out, float *topk_weight_out,
+                                          void *workspace, size_t workspace_bytes, void *stream) {
+  DICE_REQUIRE(caller, DICE_ERR_BAD_ARG, "dice_moe_forward_modulated: null pointer");
+  DICE_REQUIRE(mode >= 0 && mode <= 2, DICE_ERR_BAD_ARG, "dice_moe_forward_modulated: mode %d", mode);
+  return dice::forward_impl("dice_moe_forward_modulated", L, L, x, n_tokens, mode == 2, skip_mask, nullptr,
+                            nullptr, nullptr, mode, cache_in, cache_out, false, caller, out, topk_idx_out,
+                            topk_weight_out, workspace, workspace_bytes, stream);
 }
 
 extern "C" int dice_moe_forward_lagged(const dice_moe_layer_t *L, const dice_moe_layer_t *experts_of,
@@ -415,13 +446,13 @@ extern "C" int dice_moe_forward_lagged(const dice_moe_layer_t *L, const dice_moe
                                        const uint8_t *skip_mask, dice_moe_lag_entry_t *put,
                                        const dice_moe_lag_entry_t *work, const dice_moe_lag_entry_t *emit,
                                        int combine_mode, const void *cache_in, void *cache_out,
-                                       int use_latest_weights, void *y, int32_t *topk_idx_out,
-                                       float *topk_weight_out, void *workspace, size_t workspace_bytes,
-                                       void *stream) {
+                                       int use_latest_weights, const dice_moe_caller_t *caller, void *y,
+                                       int32_t *topk_idx_out, float *topk_weight_out, void *workspace,
+                                       size_t workspace_bytes, void *stream) {
   DICE_REQUIRE(L, DICE_ERR_BAD_ARG, "dice_moe_forward_lagged: null pointer");
   return dice::forward_impl("dice_moe_forward_lagged", L, experts_of ? experts_of : L, x, n_tokens,
                             drop_skipped != 0, skip_mask, put, work, emit, combine_mode, cache_in, cache_out,
-                            use_latest_weights != 0, y, topk_idx_out, topk_weight_out, workspace,
+                            use_latest_weights != 0, caller, y, topk_idx_out, topk_weight_out, workspace,
                             workspace_bytes, stream);
 }
 

@@ -45,6 +45,9 @@ EXPORTS = [
     "dice_moe_workspace_bytes",
     "dice_moe_forward",
     "dice_moe_forward_lagged",
+    "dice_ln_modulate",
+    "dice_combine_residual",
+    "dice_moe_forward_modulated",
 ]
 
 
@@ -74,6 +77,13 @@ class LagEntryDesc(Structure):
         ("x", c_void_p), ("offsets", c_void_p), ("perm", c_void_p), ("inv_perm", c_void_p),
         ("topk_weight", c_void_p), ("rows", c_void_p), ("max_rows", c_int64),
     ]
+
+
+class CallerDesc(Structure):
+    """Mirror of ``dice_moe_caller_t``."""
+
+    _fields_ = [("shift", c_void_p), ("scale", c_void_p), ("gate", c_void_p),
+                ("tokens_per_sample", c_int64), ("ln_eps", c_float)]
 
 
 _lib: Optional[ctypes.CDLL] = None
@@ -121,7 +131,19 @@ def load() -> ctypes.CDLL:
     lib.dice_moe_forward_lagged.argtypes = [POINTER(MoeLayerDesc), POINTER(MoeLayerDesc), c_void_p, c_int64,
                                             c_int, c_void_p, POINTER(LagEntryDesc), POINTER(LagEntryDesc),
                                             POINTER(LagEntryDesc), c_int, c_void_p, c_void_p, c_int,
-                                            c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]
+                                            POINTER(CallerDesc), c_void_p, c_void_p, c_void_p, c_void_p,
+                                            c_size_t, c_void_p]
+    lib.dice_ln_modulate.restype = c_int
+    lib.dice_ln_modulate.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_int64,
+                                     c_float, c_void_p]
+    lib.dice_combine_residual.restype = c_int
+    lib.dice_combine_residual.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                          c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int64, c_int, c_int,
+                                          c_void_p]
+    lib.dice_moe_forward_modulated.restype = c_int
+    lib.dice_moe_forward_modulated.argtypes = [POINTER(MoeLayerDesc), POINTER(CallerDesc), c_void_p, c_int64,
+                                               c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                               c_void_p, c_void_p, c_size_t, c_void_p]
     lib.dice_profile_enable.restype = c_int
     lib.dice_profile_enable.argtypes = [c_int]
     lib.dice_profile_stage_count.restype = c_int

@@ -17,7 +17,7 @@ import torch
 import torch.nn as nn
 
 from . import diep, ops
-from .lib import (DICE_ACT_GELU_TANH, DICE_ACT_SWIGLU, MODE_PLAIN, MODE_PUT, MODE_SKIP, DiceError,
+from .lib import (DICE_ACT_GELU_TANH, DICE_ACT_SWIGLU, MODE_PLAIN, MODE_PUT, MODE_SKIP, CallerDesc, DiceError,
                   MoeLayerDesc, check, dtype_code, load, ptr, stream_ptr)
 
 
@@ -268,12 +268,33 @@ class SparseMoeBlock(nn.Module):
     @torch.no_grad()
     def forward(self, hidden_states):
         """``[B, T, D] -> [B, T, D]`` (reference models.py:302-358)."""
+        return self._forward(hidden_states, None)
+
+    @torch.no_grad()
+    def forward_modulated(self, x, shift, scale, gate, eps: float = 1e-6, out=None):
+        """The MoE line of the reference's ``DiTBlock.forward`` (models.py:519)
+        in one call: ``x + gate.unsqueeze(1) * moe(modulate(norm2(x), shift, scale))``
+        with ``norm2 = LayerNorm(D, elementwise_affine=False, eps)`` (models.py:497)
+        and ``modulate`` of models.py:75-76.  ``x [B, T, D]``; ``shift``, ``scale``,
+        ``gate`` ``[B, D]`` (chunks of adaLN_modulation's output are fine: they are
+        made contiguous here).  ``out`` may be ``x`` itself."""
+        if x.dim() != 3 or shift.shape != (x.shape[0], x.shape[2]):
+            raise DiceError("forward_modulated needs x [B, T, D] and shift / scale / gate [B, D]")
+        c = CallerDesc()
+        keep = [t.to(x.dtype).contiguous() for t in (shift, scale, gate)]
+        c.shift, c.scale, c.gate = (ptr(t) for t in keep)
+        c.tokens_per_sample = x.shape[1]
+        c.ln_eps = eps
+        return self._forward(x, c, out)
+
+    def _forward(self, hidden_states, caller, out=None):
         if self.training:
             raise DiceError("SparseMoeBlock: only the inference branch is implemented (call .eval())")
         orig_shape = hidden_states.shape
         x = hidden_states.reshape(-1, orig_shape[-1]).contiguous()
+        y = None if out is None else out.view(-1, orig_shape[-1])
         if not self.para_mode.ep:
-            return self.run(x).view(*orig_shape)
+            return self.run(x, y=y, caller=caller).view(*orig_shape)
         # reference models.py:325-354
         async_op = bool(self.para_mode.ep_async) and diep.layer_is_async(
             self.para_mode.ep_async_mode, self.layer_idx, self.total_layers)
@@ -282,7 +303,7 @@ class SparseMoeBlock(nn.Module):
             mask = diep.ep_skip_mask(x.shape[0] * self.num_experts_per_tok).to(x.device)
             skip_now = diep.ep_skip_now(self.layer_idx)
         if async_op:
-            return self._run_lagged(x, mask, skip_now).view(*orig_shape)
+            return self._run_lagged(x, mask, skip_now, caller=caller, y=y).view(*orig_shape)
         mode, cache_in, cache_out = MODE_PLAIN, None, None
         if mask is not None:
             # conditional communication: reference ep_fwd.py:49-66,176-188
@@ -291,13 +312,13 @@ class SparseMoeBlock(nn.Module):
             else:
                 mode = MODE_PUT
                 cache_out = torch.empty_like(x)
-        y = self.run(x, mode, mask, cache_in, cache_out)
+        y = self.run(x, mode, mask, cache_in, cache_out, y=y, caller=caller)
         if mode == MODE_PUT:
             diep.ep_skip_put(self.layer_idx, cache_out)
         return y.view(*orig_shape)
 
     @torch.no_grad()
-    def _run_lagged(self, x, mask, skip_now, topk_idx_out=None, topk_weight_out=None):
+    def _run_lagged(self, x, mask, skip_now, topk_idx_out=None, topk_weight_out=None, caller=None, y=None):
         """Step-lagged call (reference ep_fwd.py:133-195 with async_op=True):
         this call's routing is booked into the caches, the routed experts run on
         the entry ``diep.lag_roles`` hands back and an older entry is returned.
@@ -326,21 +347,24 @@ class SparseMoeBlock(nn.Module):
         owner = work.owner if work.owner is not None else self
         experts_of = owner._ensure(x)
         put_d, work_d, emit_d = new.desc(), work.desc(), emit.desc()
-        y = torch.empty_like(x)
+        if y is None:
+            y = torch.empty_like(x)
         check(load().dice_moe_forward_lagged(
             ctypes.byref(desc), ctypes.byref(experts_of), ptr(x), n, int(bool(skip_now)), ptr(mask),
             ctypes.byref(put_d), None if work is new else ctypes.byref(work_d),
             None if emit is work else ctypes.byref(emit_d), mode, ptr(cache_in), ptr(cache_out),
-            int(diep.latest_expert_weights()), ptr(y), ptr(topk_idx_out), ptr(topk_weight_out),
-            ptr(ws), ws.numel(), stream_ptr()))
+            int(diep.latest_expert_weights()), None if caller is None else ctypes.byref(caller), ptr(y),
+            ptr(topk_idx_out), ptr(topk_weight_out), ptr(ws), ws.numel(), stream_ptr()))
         if mode == MODE_PUT:
             diep.ep_skip_put(self.layer_idx, cache_out)
         return y
 
     @torch.no_grad()
     def run(self, x, mode=MODE_PLAIN, skip_mask=None, cache_in=None, cache_out=None,
-            topk_idx_out=None, topk_weight_out=None, y=None):
-        """One call of ``dice_moe_forward`` on ``x [N, D]``."""
+            topk_idx_out=None, topk_weight_out=None, y=None, caller=None):
+        """One call of ``dice_moe_forward`` on ``x [N, D]`` (of
+        ``dice_moe_forward_modulated`` when the caller's prologue / epilogue come
+        along: ``x`` is then the residual stream)."""
         desc = self._ensure(x)
         n = x.shape[0]
         ws = self._workspace(desc, n, x.device)
@@ -348,9 +372,15 @@ class SparseMoeBlock(nn.Module):
             y = torch.empty_like(x)
         if skip_mask is not None and skip_mask.dtype == torch.bool:
             skip_mask = skip_mask.view(torch.uint8)
-        check(load().dice_moe_forward(ctypes.byref(desc), ptr(x), n, mode, ptr(skip_mask), ptr(cache_in),
-                                      ptr(cache_out), ptr(y), ptr(topk_idx_out), ptr(topk_weight_out),
-                                      ptr(ws), ws.numel(), stream_ptr()))
+        if caller is None:
+            check(load().dice_moe_forward(ctypes.byref(desc), ptr(x), n, mode, ptr(skip_mask), ptr(cache_in),
+                                          ptr(cache_out), ptr(y), ptr(topk_idx_out), ptr(topk_weight_out),
+                                          ptr(ws), ws.numel(), stream_ptr()))
+        else:
+            check(load().dice_moe_forward_modulated(
+                ctypes.byref(desc), ctypes.byref(caller), ptr(x), n, mode, ptr(skip_mask), ptr(cache_in),
+                ptr(cache_out), ptr(y), ptr(topk_idx_out), ptr(topk_weight_out), ptr(ws), ws.numel(),
+                stream_ptr()))
         return y
 
     @torch.no_grad()

@@ -112,6 +112,18 @@ def combine(slot_out: torch.Tensor, topk_weight: torch.Tensor, n_tokens: int, to
     return y
 
 
+def ln_modulate(x: torch.Tensor, shift: torch.Tensor, scale: torch.Tensor, eps: float = 1e-6):
+    """``LayerNorm(x) * (1 + scale[:, None]) + shift[:, None]`` without affine
+    parameters (reference models.py:75-76,497,519).  ``x [B, T, D]``, ``shift``
+    and ``scale`` ``[B, D]``."""
+    b, t, d = x.shape
+    x = x.contiguous()
+    out = torch.empty_like(x)
+    check(load().dice_ln_modulate(ptr(x), ptr(shift.contiguous()), ptr(scale.contiguous()), ptr(out),
+                                  dtype_code(x.dtype), b * t, d, t, eps, stream_ptr()))
+    return out
+
+
 def quantize_fp8_rowwise(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """Per-output-channel e4m3fn quantisation of a ``[..., rows, cols]`` weight.
     Returns ``(q float8_e4m3fn same shape, scale fp32 [..., rows])``."""

@@ -213,6 +213,48 @@ int dice_moe_forward(const dice_moe_layer_t *layer, const void *x,
                      void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * The layer's caller, fused.  Replaces the MoE line of DiTBlock.forward
+ * (models.py:519)
+ *   x = x + gate_mlp.unsqueeze(1) * self.moe(modulate(self.norm2(x), shift_mlp, scale_mlp))
+ * with norm2 = LayerNorm(hidden, elementwise_affine=False, eps=1e-6)
+ * (models.py:497) and modulate(x, shift, scale) = x*(1+scale)+shift per sample
+ * (models.py:75-76).
+ *
+ * dice_ln_modulate is the prologue alone: out[t] = LN(x[t]) * (1 + scale[b]) +
+ * shift[b], b = t / tokens_per_sample; statistics and arithmetic in fp32
+ * (biased variance around the mean, eps inside the square root), one rounding
+ * to `dtype`.   x, out [n_tokens, hidden]; shift, scale [n_samples, hidden].
+ *
+ * dice_combine_residual is dice_combine followed by the epilogue
+ * out[t] = resid[t] + gate[b] * y[t], applied to the fp32 sum before the one
+ * rounding; `out` may alias `resid`.
+ *
+ * dice_moe_forward_modulated is dice_moe_forward between the two: x is the
+ * residual stream, the layer runs on the modulated rows (kept in the
+ * workspace) and `out` (which may alias x) receives the updated stream.
+ */
+typedef struct dice_moe_caller {
+  const void *shift, *scale, *gate; /* [n_samples, hidden], activation dtype */
+  int64_t tokens_per_sample;        /* T of x [B, T, hidden] */
+  float ln_eps;                     /* 1e-6 in the reference */
+} dice_moe_caller_t;
+
+int dice_ln_modulate(const void *x, const void *shift, const void *scale, void *out,
+                     int dtype, int64_t n_tokens, int hidden, int64_t tokens_per_sample,
+                     float eps, void *stream);
+int dice_combine_residual(const void *slot_out, const int32_t *inv_perm,
+                          const float *topk_weight, const void *shared_out,
+                          const uint8_t *skip_mask, const void *cache_in, void *cache_out,
+                          const void *resid, const void *gate, int64_t tokens_per_sample,
+                          void *out, int dtype, int64_t n_tokens, int top_k, int hidden,
+                          void *stream);
+int dice_moe_forward_modulated(const dice_moe_layer_t *layer, const dice_moe_caller_t *caller,
+                               const void *x, int64_t n_tokens, int mode,
+                               const uint8_t *skip_mask, const void *cache_in, void *cache_out,
+                               void *out, int32_t *topk_idx_out, float *topk_weight_out,
+                               void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Step-lagged layer call.  Replaces moe_infer_ep with async_op=True
  * (expertpara/ep_fwd.py:133-172) and the dispatch / combine caches behind
  * global_dispatch_async / global_combine_async (expertpara/diep.py:17-28,
@@ -244,6 +286,9 @@ int dice_moe_forward(const dice_moe_layer_t *layer, const void *x,
  *   combine_mode  0 plain; 1 also write cache_out from the emitted entry; 2 the
  *                 emitted entry was produced with drop_skipped: masked slots
  *                 take cache_in (ep_fwd.py:176-188)
+ *   caller        NULL, or the fused caller above: x is then the residual
+ *                 stream, the entry's x receives the modulated rows directly
+ *                 (no copy) and y the updated stream
  */
 typedef struct dice_moe_lag_entry {
   void *x;
@@ -258,7 +303,8 @@ int dice_moe_forward_lagged(const dice_moe_layer_t *layer, const dice_moe_layer_
                             const uint8_t *skip_mask, dice_moe_lag_entry_t *put,
                             const dice_moe_lag_entry_t *work, const dice_moe_lag_entry_t *emit,
                             int combine_mode, const void *cache_in, void *cache_out,
-                            int use_latest_weights, void *y, int32_t *topk_idx_out,
+                            int use_latest_weights, const dice_moe_caller_t *caller,
+                            void *y, int32_t *topk_idx_out,
                             float *topk_weight_out, void *workspace, size_t workspace_bytes,
                             void *stream);
 

@@ -42,6 +42,12 @@ Pinning status (what independently fixes each function's result):
                           stale-weight switch changing only the scale factors.
                           Its combination with the skip cache is exercised only
                           as a state machine: "parity unpinned".
+* ``norm_modulate`` /    - float64 numpy definition of LayerNorm (biased variance
+  ``dit_block_moe_half``  around the mean, eps inside the root) and of the two
+                          affine maps on small inputs; constant rows give
+                          exactly ``shift``; scale = -1 removes x altogether;
+                          gate = 0 returns x.  The reference has no test of its
+                          DiTBlock: beyond these, "parity unpinned".
 * bf16 / fp8 variants   - no reference code or vector exists for them
                           ("parity unpinned" by the reference); they are the
                           same functions evaluated in that dtype.
@@ -700,6 +706,48 @@ def sparse_moe_block_forward(
     if params.shared is not None:
         y = y + params.shared(identity)
     return y, topk_idx, topk_weight, logits
+
+
+# --------------------------------------------------------------------------- #
+# The block's caller
+# --------------------------------------------------------------------------- #
+def modulate(x: torch.Tensor, shift: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    """Restates ``modulate`` (models.py:75-76)."""
+    return x * (1 + scale.unsqueeze(1)) + shift.unsqueeze(1)
+
+
+def norm_modulate(x: torch.Tensor, shift: torch.Tensor, scale: torch.Tensor, eps: float = 1e-6,
+                  single_rounding: bool = False) -> torch.Tensor:
+    """``modulate(self.norm2(x), shift_mlp, scale_mlp)`` with ``norm2 =
+    nn.LayerNorm(hidden, elementwise_affine=False, eps=1e-6)`` (models.py:497,519).
+
+    ``single_rounding=False`` is the literal op sequence in the tensors' dtype
+    (LayerNorm output, ``1 + scale``, the product and the sum are each rounded
+    to it); ``True`` evaluates the same expression in fp32 and rounds once,
+    which is what one fused pass computes.  The two coincide in fp32."""
+    d = x.shape[-1]
+    if single_rounding:
+        h = F.layer_norm(x.float(), (d,), None, None, eps)
+        return modulate(h, shift.float(), scale.float()).to(x.dtype)
+    return modulate(F.layer_norm(x, (d,), None, None, eps), shift, scale)
+
+
+@torch.no_grad()
+def dit_block_moe_half(params: "MoEBlockParams", x: torch.Tensor, shift: torch.Tensor, scale: torch.Tensor,
+                       gate: torch.Tensor, eps: float = 1e-6, single_rounding: bool = False, **block_kw):
+    """Restates the MoE line of ``DiTBlock.forward`` (models.py:519):
+    ``x + gate_mlp.unsqueeze(1) * self.moe(modulate(self.norm2(x), shift_mlp, scale_mlp))``.
+
+    Returns ``(out, h, topk_idx, topk_weight, logits)``; ``h`` is the layer input.
+    With ``single_rounding`` the epilogue too is evaluated in fp32 from the
+    block's output and rounded once."""
+    h = norm_modulate(x, shift, scale, eps, single_rounding)
+    y, idx, wt, logits = sparse_moe_block_forward(params, h, **block_kw)
+    if single_rounding:
+        out = (x.float() + gate.float().unsqueeze(1) * y.float()).to(x.dtype)
+    else:
+        out = x + gate.unsqueeze(1) * y
+    return out, h, idx, wt, logits
 
 
 # --------------------------------------------------------------------------- #

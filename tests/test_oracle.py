@@ -340,3 +340,51 @@ def test_displaced_with_skip_cache_state_machine():
             state.cancel_sync()
         assert got.shape == x.shape
         assert torch.allclose(got, want, atol=1e-5, rtol=1e-5), i
+
+
+# --------------------------------------------------------------------------- #
+# the block's caller: LayerNorm + modulate prologue, gated residual epilogue
+# --------------------------------------------------------------------------- #
+def test_norm_modulate_against_float64_definition():
+    rng = np.random.default_rng(11)
+    B, T, D = 3, 5, 48
+    x = (rng.standard_normal((B, T, D)) * 3 + 2).astype(np.float32)
+    shift = rng.standard_normal((B, D)).astype(np.float32)
+    scale = rng.standard_normal((B, D)).astype(np.float32)
+    x64 = x.astype(np.float64)
+    mean = x64.mean(-1, keepdims=True)
+    var = ((x64 - mean) ** 2).mean(-1, keepdims=True)          # biased
+    want = (x64 - mean) / np.sqrt(var + 1e-6) * (1 + scale[:, None, :]) + shift[:, None, :]
+    for single in (False, True):
+        got = O.norm_modulate(torch.from_numpy(x), torch.from_numpy(shift), torch.from_numpy(scale),
+                              single_rounding=single)
+        assert np.allclose(got.double().numpy(), want, atol=2e-5, rtol=1e-5)
+    # an unbiased variance or eps outside the root would miss by far more than the tolerance
+    wrong = (x64 - mean) / np.sqrt(var * D / (D - 1) + 1e-6) * (1 + scale[:, None, :]) + shift[:, None, :]
+    assert not np.allclose(wrong, want, atol=2e-5, rtol=1e-5)
+    # constant rows normalise to zero: the output is the shift alone
+    const = torch.full((B, T, D), 4.0)
+    got = O.norm_modulate(const, torch.from_numpy(shift), torch.from_numpy(scale))
+    assert torch.allclose(got, torch.from_numpy(shift)[:, None, :].expand(B, T, D), atol=1e-6)
+
+
+def test_block_caller_identities():
+    p = _small_block()
+    g = torch.Generator().manual_seed(2)
+    B, T, D = 2, 9, 64
+    x = torch.randn(B, T, D, generator=g)
+    shift, scale, gate = (torch.randn(B, D, generator=g) * 0.3 for _ in range(3))
+    out, h, idx, wt, _ = O.dit_block_moe_half(p, x, shift, scale, gate)
+    # definition, with the already pinned block on the already pinned prologue
+    y, idx2, _, _ = O.sparse_moe_block_forward(p, h)
+    assert torch.equal(idx, idx2)
+    want = x.double() + gate.double()[:, None, :] * y.double()
+    assert torch.allclose(out.double(), want, atol=1e-6)
+    # gate = 0 leaves the stream untouched; scale = -1 feeds the layer the shift only
+    out0, *_ = O.dit_block_moe_half(p, x, shift, scale, torch.zeros(B, D))
+    assert torch.equal(out0, x)
+    _, h1, *_ = O.dit_block_moe_half(p, x, shift, -torch.ones(B, D), gate)
+    assert torch.allclose(h1, shift[:, None, :].expand(B, T, D), atol=1e-6)
+    # fp32: one rounding or four, same result
+    out_s, *_ = O.dit_block_moe_half(p, x, shift, scale, gate, single_rounding=True)
+    assert torch.allclose(out_s, out, atol=1e-5)
