@@ -749,11 +749,24 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
 
   // This workgroup's tiles, described once and parked in LDS behind the epilogue's
   // staging rows; lane f of a table read gets word f of the description.
-  constexpr int kTableBytes = kTableTurns * kTileWords * 4, kRowSlotBytes = GATHER ? kPBM * 4 : 0;
-  static_assert(kQWaves * Epi::WAVE_BYTES + kTableBytes + kRowSlotBytes <= kPStageArea, "no room for the tile table");
+  constexpr int kTableBytes = kTableTurns * kTileWords * 4, kRowSlotBytes = kPBM * 4;
+  // A 256-wide biased tile starts its accumulators from the bias (64 values per
+  // lane that the epilogue then need not hold: it would spill); its epilogue
+  // stages 16-row bands, which leaves room for two bias buffers of one tile's
+  // columns each beside the tile table.  A 192-wide tile (48 values) adds the
+  // bias in the epilogue.
+  constexpr bool kBiasInAcc = HAS_BIAS && BN == 256;
+  constexpr int kBiasBufFloats = 256, kBiasBytes = 2 * kBiasBufFloats * 4;
+  static_assert(kQWaves * Epi::WAVE_BYTES + kTableBytes + (GATHER ? kRowSlotBytes : 0) +
+                        (kBiasInAcc ? kRowSlotBytes + kBiasBytes : 0) <= kPStageArea,
+                "no room for the tile table");
   uint32_t *const tile_table = reinterpret_cast<uint32_t *>(lds_stage + kPStageArea - kTableBytes);
   // (gathered activations) the slots of the 256 rows of the tile the load side opens next
-  int32_t *const lds_row_slots = reinterpret_cast<int32_t *>(lds_stage + kPStageArea - kTableBytes - kPBM * 4);
+  int32_t *const lds_row_slots = reinterpret_cast<int32_t *>(lds_stage + kPStageArea - kTableBytes - kRowSlotBytes);
+  // The first wave copies a tile's bias in (one global->LDS instruction) a whole
+  // tile before the accumulators of that tile are initialised with it.
+  float *const lds_bias =
+      reinterpret_cast<float *>(lds_stage + kPStageArea - kTableBytes - kRowSlotBytes - kBiasBytes);
   if (wave == 0) {
     TileWalker<BN_OUT> walk(batch, lane);
     walk.build_table(batch, lane, kQBK, tile_table);
@@ -791,6 +804,20 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
             __builtin_amdgcn_make_buffer_rsrc((void *)ptr, 0, (uint32_t)rows * 4, kRsrcFlags);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void *)lds_row_slots, 16,
                                                  lane * 16, 0, 0, 0);
+      }
+    }
+  };
+  auto copy_bias = [&](const PackedTile &pk, int buf) {
+    if constexpr (kBiasInAcc) {
+      const uint64_t ptr = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane(pk.words, 9) << 32) |
+                           (uint32_t)__builtin_amdgcn_readlane(pk.words, 8);
+      const int n0 = __builtin_amdgcn_readlane(pk.words, 16), n = __builtin_amdgcn_readlane(pk.words, 17);
+      if (wave == 0 && ptr != 0) {
+        // columns past the matrix read as 0 (their products are never stored)
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(ptr + (uint64_t)n0 * 4), 0, (uint32_t)(n - n0) * 4, kRsrcFlags);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rs, (__attribute__((address_space(3))) void *)(lds_bias + buf * kBiasBufFloats), 16, lane * 16, 0, 0, 0);
       }
     }
   };
@@ -840,8 +867,29 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
       af[buf][i] = *reinterpret_cast<const bf16x8_t *>(base + rd_a[KK] + i * 32 * 128);
   };
 
+  const int wave_col0 = SWIGLU ? wn * (WTN / 2) : wn * WTN;
   f32x16_t acc[TM][TN];
-  auto zero_acc = [&]() {
+  // (256-wide biased tiles) the accumulators start from the bias of their columns:
+  // every 32-row block of a column block gets the same 16 values per lane.
+  auto init_acc = [&](const Tile &t, int buf) {
+    if constexpr (kBiasInAcc) {
+      if (uni((int)(t.bias != nullptr))) {
+        const float *src = lds_bias + buf * kBiasBufFloats + wave_col0 + frag_half * 4;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          f32x16_t b;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const f32x4_t v = *reinterpret_cast<const f32x4_t *>(src + j * 32 + q * 8);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) b[q * 4 + r] = v[r];
+          }
+#pragma unroll
+          for (int i = 0; i < TM; ++i) acc[i][j] = b;
+        }
+        return;
+      }
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -865,8 +913,10 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   PackedTile nxt = fetch_tile(next_turn++);
   Tile ld = unpack_tile(nxt);                     // tile being loaded
   if (!ld.valid) return;                          // nothing to do for this workgroup
-  if constexpr (GATHER) {
+  int bias_buf = 0;                               // buffer that holds the bias of the tile being multiplied
+  if constexpr (GATHER || kBiasInAcc) {
     copy_row_slots(nxt);
+    copy_bias(nxt, 0);
     pwait_vmcnt<0>();
     phase_barrier();
   }
@@ -879,6 +929,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
     phase_barrier();
     copy_row_slots(nxt);
   }
+  copy_bias(nxt, 1);
   auto advance_copy = [&]() {
     if (++ld_kt == ld.steps) {
       ld = unpack_tile(nxt);
@@ -941,14 +992,13 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   load_step(c0);           // step 2
   write_quarter(c1, c0);
   load_quarter(c1, c0);    // first quarter of step 3; the stage keeps quarters 1..3 of step 1
-  zero_acc();
+  init_acc(cp, 0);
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   phase_barrier();
   read_frags(c0, c0, 0);
   __builtin_amdgcn_sched_barrier(0);
 
   unsigned char *const stage_rows = lds_stage + wave * Epi::WAVE_BYTES;
-  const int wave_col0 = SWIGLU ? wn * (WTN / 2) : wn * WTN;
 
   while (true) {  // one tile per iteration
     // Every tile has an even number of steps, so a tile always starts in slot 0.
@@ -989,7 +1039,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
       step(c0);
       step(c1);
     }
-    tile_epilogue<MODE, HAS_BIAS, kQWaves, TM, TN>(cp, acc, stage_rows, wm * WTM, wave_col0, lane);
+    tile_epilogue<MODE, HAS_BIAS && !kBiasInAcc, kQWaves, TM, TN>(cp, acc, stage_rows, wm * WTM, wave_col0, lane);
     // The load side is within the next tile here (every tile has at least
     // kQMinSteps steps).
     cp = ld;
@@ -1001,7 +1051,11 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
     // for those (at most 32 newer loads are ever in flight) cover it long before
     // the load side opens `nxt`, at least two steps from here.
     copy_row_slots(nxt);
-    zero_acc();
+    // (the bias buffer written here was last read a whole tile ago, the one read
+    // below was filled a whole tile ago: the same ordering as for the row slots)
+    copy_bias(nxt, bias_buf);
+    bias_buf ^= 1;
+    init_acc(cp, bias_buf);
     // The last block above already fetched these fragments; reading them again
     // here keeps 32 registers free during the epilogue.
     read_frags(c0, c0, 0);
@@ -1062,7 +1116,8 @@ bool persist64_ok(const PersistBatch &b, int mode) {
   for (int i = 0; i < b.n_problems; ++i) {
     const PersistProblem &p = b.prob[i];
     if (p.k < kQBK * kQMinSteps) return false;
-    if (p.a_rows) {  // gathered activation rows: SwiGLU instantiation only
+    if (p.a_rows) {  // gathered activation rows: SwiGLU instantiation only (the GELU one would
+                     // spill, and measures no faster than a gathered copy plus the plain kernel)
       if (mode != kFc1Swiglu) return false;
       if (p.a_div < 1 || p.a_div > 16 || (int64_t)p.a_src_rows * p.a_div >= (1ll << 28)) return false;
       if ((size_t)p.a_src_rows * p.lda * 2 >= (1ull << 31)) return false;

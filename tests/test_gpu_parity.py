@@ -300,6 +300,13 @@ def test_mlp_bf16_persistent_kernels(dev, variant, cfg):
     _check_mlp_persistent(dev, 512, 512, 8, 2, variant, cfg, counts=[1024, 0, 0, 0, 0, 0, 0, 0])
 
 
+def test_mlp_bf16_biased_tiles_across_experts(dev):
+    """GELU experts with non-zero biases at XL width, enough rows that every
+    workgroup multiplies several tiles in a row, of different experts and
+    column blocks: the 256-wide tiles start their accumulators from a bias that
+    is staged one tile ahead, alternating between two buffers."""
+    _check_mlp_persistent(dev, 4096, 1152, 8, 4, "gelu_tanh", 21)
+
 
 
 @pytest.mark.parametrize("cfg", [0, 1, 2])
