@@ -381,12 +381,36 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
         }
     }
   }
+#define DICE_EPI_VALUE(v, j, e)                        \
+  do {                                                 \
+    if (SWIGLU) {                                      \
+      v = silu_fast(v) * up[e];                        \
+    } else {                                           \
+      if (HAS_BIAS) v += bias_v[j][e];                 \
+      if (MODE == kFc1Gelu) v = gelu_tanh_fast(v);     \
+    }                                                  \
+  } while (0)
+#define DICE_EPI_STORE_BAND(band)                                                                          \
+  do {                                                                                                     \
+    wave_lds_sync();                                                                                       \
+    _Pragma("unroll") for (int ps = 0; ps < G::PASSES; ++ps) {                                             \
+      int r = ps * G::ROWS_PER_PASS + rd_row;                                                              \
+      bool live = true;                                                                                    \
+      if (!G::EXACT) {                                                                                     \
+        live = rd_row < G::ROWS_PER_PASS && r < BAND;                                                      \
+        r = live ? r : 0;                                                                                  \
+      }                                                                                                    \
+      const u32x4_t v = *reinterpret_cast<const u32x4_any_t *>(stage + r * PITCH + rd_chunk * 16);         \
+      const int m = wave_row0 + (band) * BAND + r;                                                         \
+      const int n = col_base + rd_chunk * 8;                                                               \
+      const uint32_t voff = (live && n < cp.n) ? (uint32_t)m * cp.c_pitch + (uint32_t)n * 2 : kOutOfRange; \
+      __builtin_amdgcn_raw_buffer_store_b128(v, crs, voff, 0, 0);                                          \
+    }                                                                                                      \
+    wave_lds_sync(); /* the next band overwrites the staging rows */                                       \
+  } while (0)
 #pragma unroll
-  for (int band = 0; band < TM * 32 / BAND; ++band) {
-    const int i = band * BAND / 32;             // 32-row block the band lies in
-    const int half = (band * BAND % 32) / 16;   // which 16 rows of it (BAND == 16 only)
-    if (BAND == 32 || (frag_row >> 4) == half) {
-      const int srow = BAND == 32 ? frag_row : (frag_row & 15);
+  for (int i = 0; i < TM; ++i) {
+    if constexpr (BAND == 32) {
 #pragma unroll
       for (int j = 0; j < OUT_BLOCKS; ++j) {
         const f32x16_t blk = acc_block<WAVES == 4>(acc[i][j]);
@@ -399,39 +423,54 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             float v = blk[q * 4 + r];
-            if (SWIGLU) {
-              v = silu_fast(v) * up[q * 4 + r];
-            } else {
-              if (HAS_BIAS) v += bias_v[j][q * 4 + r];
-              if (MODE == kFc1Gelu) v = gelu_tanh_fast(v);
-            }
+            DICE_EPI_VALUE(v, j, q * 4 + r);
             o[r] = (bf16_t)v;
           }
-          *reinterpret_cast<u32x2_any_t *>(stage + srow * PITCH + col * 2) = __builtin_bit_cast(u32x2_t, o);
+          *reinterpret_cast<u32x2_any_t *>(stage + frag_row * PITCH + col * 2) = __builtin_bit_cast(u32x2_t, o);
         }
       }
-    }
-    wave_lds_sync();
+      DICE_EPI_STORE_BAND(i);
+    } else {
+      // The staging rows hold 16 rows at a time.  The activation of the whole
+      // 32-row block is worked out once, with every lane at work (per band only
+      // half the lanes own rows), and kept packed while its two bands go out.
+      bf16x4_t packed[OUT_BLOCKS][4];
 #pragma unroll
-    for (int ps = 0; ps < G::PASSES; ++ps) {
-      int r = ps * G::ROWS_PER_PASS + rd_row;
-      bool live = true;
-      if (!G::EXACT) {
-        live = rd_row < G::ROWS_PER_PASS && r < BAND;
-        r = live ? r : 0;
+      for (int j = 0; j < OUT_BLOCKS; ++j) {
+        const f32x16_t blk = acc_block<WAVES == 4>(acc[i][j]);
+        f32x16_t up;
+        if (SWIGLU) up = acc_block<WAVES == 4>(acc[i][j + OUT_BLOCKS]);
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float v = blk[q * 4 + r];
+            DICE_EPI_VALUE(v, j, q * 4 + r);
+            packed[j][q][r] = (bf16_t)v;
+          }
       }
-      const u32x4_t v = *reinterpret_cast<const u32x4_any_t *>(stage + r * PITCH + rd_chunk * 16);
-      const int m = wave_row0 + band * BAND + r;
-      const int n = col_base + rd_chunk * 8;
-      const uint32_t voff = (live && n < cp.n) ? (uint32_t)m * cp.c_pitch + (uint32_t)n * 2 : kOutOfRange;
-      __builtin_amdgcn_raw_buffer_store_b128(v, crs, voff, 0, 0);
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        if ((frag_row >> 4) == half) {
+#pragma unroll
+          for (int j = 0; j < OUT_BLOCKS; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int col = j * 32 + frag_half * 4 + q * 8;
+              *reinterpret_cast<u32x2_any_t *>(stage + (frag_row & 15) * PITCH + col * 2) =
+                  __builtin_bit_cast(u32x2_t, packed[j][q]);
+            }
+        }
+        DICE_EPI_STORE_BAND(2 * i + half);
+      }
     }
-    wave_lds_sync();  // the next band overwrites the staging rows
-    // Keeps the bands apart: hoisting the next band's accumulator reads over this
-    // one's stores only lengthens live ranges (register spills cost far more
-    // here than the lost overlap).
+    // Keeps the 32-row blocks apart: hoisting the next block's accumulator reads
+    // over this one's stores only lengthens live ranges (register spills cost far
+    // more here than the lost overlap).
     __builtin_amdgcn_sched_barrier(0);
   }
+#undef DICE_EPI_VALUE
+#undef DICE_EPI_STORE_BAND
 }
 
 // HAS_BIAS is a compile-time switch so that the bias-free (reference SwiGLU)
