@@ -119,8 +119,8 @@ __device__ __forceinline__ float gelu_tanh_fast(float x) {
 
 // One grouped GEMM of a persistent launch: grouped activation rows (row r of
 // expert e = a + (offsets[e] + r) * lda, or, with a_rows, the source row
-// a_rows[offsets[e] + r] / a_div of a), bf16 weights [n_experts, w_rows, k],
-// output rows in grouped order.
+// a_rows[offsets[e] + r] / a_div of a), bf16 (or, with w_scale, fp8) weights
+// [n_experts, w_rows, k], output rows in grouped order.
 struct PersistProblem {
   const void *a;
   int lda;
@@ -137,6 +137,7 @@ struct PersistProblem {
   const int32_t *a_rows;   // grouped row -> slot (the dispatch permutation), or NULL: rows are contiguous
   int a_div;               // slots per source row (top-k)
   int a_src_rows;          // rows of the source matrix (range check of the gather)
+  const float *w_scale;    // [n_experts, w_rows] per-output-channel scales: the weights are fp8 (e4m3) bytes; NULL: bf16
 };
 constexpr int kMaxPersistProblems = 3;
 struct PersistBatch {

@@ -197,7 +197,7 @@ struct TileWalker {
   // that a tile switch inside the kernel is a single LDS read.  Turns past the
   // XCD's run give descriptions that cover no bytes.  Called by one wave.
   __device__ __forceinline__ void build_table(const PersistBatch &batch, int lane, int bk,
-                                              uint32_t *table) const {
+                                              uint32_t *table, bool w8 = false) const {
     const int w = (lane & 1) ? wgs_per_xcd - 1 - wg_in_xcd : wg_in_xcd;
     const int id = run_begin + lane * wgs_per_xcd + w;
     const bool valid = id < run_end;
@@ -231,7 +231,10 @@ struct TileWalker {
     const int n0 = n_tile * BN_OUT;
     const int cols_left = n - n0;
     const int wrows = cols_left < BN_OUT ? cols_left : BN_OUT;
-    const uint32_t a_pitch = (uint32_t)lda * 2, b_pitch = (uint32_t)k * 2, c_pitch = (uint32_t)ldc * 2;
+    // (fp8 weights: one byte per element, and word 22 carries the row of the
+    // per-output-channel scale table instead of the gather's reciprocal, which a
+    // single-problem launch takes from its arguments)
+    const uint32_t a_pitch = (uint32_t)lda * 2, b_pitch = (uint32_t)k * (w8 ? 1 : 2), c_pitch = (uint32_t)ldc * 2;
     const uint64_t wexp = pw + (uint64_t)expert * w_rows * b_pitch;
     // Gathered rows are addressed from the start of the source matrix.
     const uint64_t ptrs[5] = {prows ? pa : pa + (uint64_t)(row0 + m_tile * kPBM) * a_pitch, wexp + (uint64_t)n0 * b_pitch,
@@ -253,7 +256,8 @@ struct TileWalker {
     const uint64_t tile_rows = prows ? prows + (uint64_t)(row0 + m_tile * kPBM) * sizeof(int32_t) : 0;
     entry[20] = (uint32_t)tile_rows;
     entry[21] = (uint32_t)(tile_rows >> 32);
-    entry[22] = (uint32_t)(0xffffffffull / (uint32_t)a_div + 1);  // mulhi(slot, .) = slot / a_div for slot < 2^28, a_div <= 16
+    entry[22] = w8 ? (uint32_t)(expert * w_rows + n0)
+                   : (uint32_t)(0xffffffffull / (uint32_t)a_div + 1);  // mulhi(slot, .) = slot / a_div for slot < 2^28, a_div <= 16
     entry[23] = (uint32_t)(valid ? rows : 0);
   }
 
@@ -320,13 +324,14 @@ struct TileWalker {
 // Geometry of one wave's epilogue: its TM x TN accumulator blocks become
 // OUT_COLS output columns (SwiGLU folds gate and up blocks), staged BAND rows at
 // a time through WAVE_BYTES of LDS and stored as whole 16-byte row chunks.
-template <int MODE, int WAVES, int TM, int TN>
+template <int MODE, int WAVES, int TM, int TN, int RESERVE = 0>
 struct EpiGeom {
   static constexpr bool SWIGLU = MODE == kFc1Swiglu;
   static constexpr int OUT_BLOCKS = SWIGLU ? TN / 2 : TN;
   static constexpr int OUT_COLS = OUT_BLOCKS * 32;
   static constexpr int PITCH = OUT_COLS * 2 + 16;
-  static constexpr int BAND = (WAVES * 32 * PITCH <= kPStageArea) ? 32 : 16;  // rows staged at a time
+  // rows staged at a time (RESERVE: bytes of the staging area that other tables take)
+  static constexpr int BAND = (WAVES * 32 * PITCH + RESERVE <= kPStageArea) ? 32 : 16;
   static constexpr int LANES_PER_ROW = OUT_COLS * 2 / 16;
   static constexpr int ROWS_PER_PASS = kWave / LANES_PER_ROW;   // lanes past ROWS_PER_PASS rows idle
   static constexpr int PASSES = (BAND + ROWS_PER_PASS - 1) / ROWS_PER_PASS;
@@ -353,10 +358,13 @@ __device__ __forceinline__ f32x16_t acc_block(const f32x16_t &a) {
 // the wave's LDS staging rows, row-segment stores.  Rows past the group's end are
 // dropped by the descriptor's range check, columns past the problem's n by an
 // offset no descriptor covers.
-template <int MODE, bool HAS_BIAS, int WAVES, int TM, int TN>
+// HAS_SCALE: the weights were fp8; column c of the product is multiplied by
+// scale_lds[c - n0] (SwiGLU: gate columns first, the up columns 128 floats on).
+template <int MODE, bool HAS_BIAS, int WAVES, int TM, int TN, bool HAS_SCALE = false, int RESERVE = 0>
 __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM][TN], unsigned char *stage,
-                                              int wave_row0, int wave_col0, int lane) {
-  using G = EpiGeom<MODE, WAVES, TM, TN>;
+                                              int wave_row0, int wave_col0, int lane,
+                                              const float *scale_lds = nullptr) {
+  using G = EpiGeom<MODE, WAVES, TM, TN, RESERVE>;
   constexpr bool SWIGLU = G::SWIGLU;
   constexpr int OUT_BLOCKS = G::OUT_BLOCKS, PITCH = G::PITCH, BAND = G::BAND;
   const int frag_row = lane & 31, frag_half = lane >> 5;
@@ -381,14 +389,24 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
         }
     }
   }
-#define DICE_EPI_VALUE(v, j, e)                        \
-  do {                                                 \
-    if (SWIGLU) {                                      \
-      v = silu_fast(v) * up[e];                        \
-    } else {                                           \
-      if (HAS_BIAS) v += bias_v[j][e];                 \
-      if (MODE == kFc1Gelu) v = gelu_tanh_fast(v);     \
-    }                                                  \
+#define DICE_EPI_SCALES(j, q)                                                                         \
+  f32x4_t sg, su;                                                                                     \
+  if (HAS_SCALE) {                                                                                    \
+    const float *sp = scale_lds + wave_col0 + (j) * 32 + frag_half * 4 + (q) * 8;                       \
+    sg = *reinterpret_cast<const f32x4_t *>(sp);                                                      \
+    if (SWIGLU) su = *reinterpret_cast<const f32x4_t *>(sp + 128);                                    \
+  }
+#define DICE_EPI_VALUE(v, j, q, r)                          \
+  do {                                                      \
+    if (HAS_SCALE) v *= sg[r];                              \
+    if (SWIGLU) {                                           \
+      float u = up[(q) * 4 + (r)];                          \
+      if (HAS_SCALE) u *= su[r];                            \
+      v = silu_fast(v) * u;                                 \
+    } else {                                                \
+      if (HAS_BIAS) v += bias_v[j][(q) * 4 + (r)];          \
+      if (MODE == kFc1Gelu) v = gelu_tanh_fast(v);          \
+    }                                                       \
   } while (0)
 #define DICE_EPI_STORE_BAND(band)                                                                          \
   do {                                                                                                     \
@@ -420,10 +438,11 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
         for (int q = 0; q < 4; ++q) {
           const int col = j * 32 + frag_half * 4 + q * 8;
           bf16x4_t o;
+          DICE_EPI_SCALES(j, q)
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             float v = blk[q * 4 + r];
-            DICE_EPI_VALUE(v, j, q * 4 + r);
+            DICE_EPI_VALUE(v, j, q, r);
             o[r] = (bf16_t)v;
           }
           *reinterpret_cast<u32x2_any_t *>(stage + frag_row * PITCH + col * 2) = __builtin_bit_cast(u32x2_t, o);
@@ -441,13 +460,15 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
         f32x16_t up;
         if (SWIGLU) up = acc_block<WAVES == 4>(acc[i][j + OUT_BLOCKS]);
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
+        for (int q = 0; q < 4; ++q) {
+          DICE_EPI_SCALES(j, q)
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             float v = blk[q * 4 + r];
-            DICE_EPI_VALUE(v, j, q * 4 + r);
+            DICE_EPI_VALUE(v, j, q, r);
             packed[j][q][r] = (bf16_t)v;
           }
+        }
       }
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
@@ -470,6 +491,7 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
     __builtin_amdgcn_sched_barrier(0);
   }
 #undef DICE_EPI_VALUE
+#undef DICE_EPI_SCALES
 #undef DICE_EPI_STORE_BAND
 }
 
@@ -764,16 +786,29 @@ __device__ __forceinline__ void qsched_block() {
 // 192 divides and 256 does not (1152 = 6 x 192: no padded columns to multiply).
 // GATHER: activation rows may be addressed through a row table (the dispatch
 // permutation), which saves the separate gathered copy of the activations.
-template <int MODE, bool HAS_BIAS, int BN, bool GATHER>
+// W8: the weights are fp8 (e4m3) bytes with one fp32 scale per output channel
+// (single-problem launches only).  A 16-byte load then holds 16 elements of a
+// row; they are widened to bf16 (exactly) on their way into LDS, so the slots,
+// the fragment reads and the MFMAs are those of the bf16 kernel; the scale
+// multiplies the fp32 sums in the epilogue.
+template <int MODE, bool HAS_BIAS, int BN, bool GATHER, bool W8 = false>
 __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   constexpr bool SWIGLU = MODE == kFc1Swiglu;
   static_assert(BN == 256 || (BN == 192 && !SWIGLU), "tile widths");
   constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
   constexpr int WTM = 128, WTN = BN / 2, TM = 4, TN = WTN / 32;
-  constexpr int kCopiesA = kPBM / 8 / kQWaves, kCopiesB = BN / 8 / kQWaves;  // 16-byte-per-lane loads, 8 rows each
+  // 16-byte-per-lane loads: 8 rows of 128 bytes each (fp8 weights: 16 rows of 64 bytes)
+  constexpr int kRowsPerCopyB = W8 ? 16 : 8;
+  constexpr int kCopiesA = kPBM / 8 / kQWaves, kCopiesB = BN / kRowsPerCopyB / kQWaves;
   constexpr int kQCopies = kCopiesA + kCopiesB;
-  static_assert(kCopiesA % 2 == 0 && kCopiesB % 2 == 0, "a step is four quarters: two of A, two of B");
-  using Epi = EpiGeom<MODE, kQWaves, TM, TN>;
+  static_assert(kCopiesA % 2 == 0, "a step is four quarters: two of A, two of B");
+  // (three scale buffers: the epilogue of a tile reads its scales while the first
+  // wave, a little ahead, may already copy in those of the tile after the next)
+  constexpr int kScaleBufFloats = 256, kScaleBytes = W8 ? 3 * kScaleBufFloats * 4 : 0;
+  constexpr int kSlotUsed = (kPBM + BN) * 128;
+  constexpr bool kScaleInSlot = W8 && kSlotUsed + kScaleBytes <= kQSlotBytes;  // 192-wide tiles leave a slot's tail free
+  constexpr int kEpiReserve = kTableTurns * kTileWords * 4 + (W8 && !kScaleInSlot ? kScaleBytes + kPBM * 4 : 0);
+  using Epi = EpiGeom<MODE, kQWaves, TM, TN, W8 ? kEpiReserve : 0>;
   const template_int<0> c0; const template_int<1> c1; const template_int<2> c2; const template_int<3> c3;
 
   // Three separate LDS objects, so that the compiler knows that fragment reads of
@@ -797,7 +832,8 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   constexpr bool kBiasInAcc = HAS_BIAS && BN == 256;
   constexpr int kBiasBufFloats = 256, kBiasBytes = 2 * kBiasBufFloats * 4;
   static_assert(kQWaves * Epi::WAVE_BYTES + kTableBytes + (GATHER ? kRowSlotBytes : 0) +
-                        (kBiasInAcc ? kRowSlotBytes + kBiasBytes : 0) <= kPStageArea,
+                        (kBiasInAcc ? kRowSlotBytes + kBiasBytes : 0) +
+                        (W8 && !kScaleInSlot ? kRowSlotBytes + kBiasBytes + kScaleBytes : 0) <= kPStageArea,
                 "no room for the tile table");
   uint32_t *const tile_table = reinterpret_cast<uint32_t *>(lds_stage + kPStageArea - kTableBytes);
   // (gathered activations) the slots of the 256 rows of the tile the load side opens next
@@ -806,9 +842,13 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   // tile before the accumulators of that tile are initialised with it.
   float *const lds_bias =
       reinterpret_cast<float *>(lds_stage + kPStageArea - kTableBytes - kRowSlotBytes - kBiasBytes);
+  // (fp8 weights) the scales of a tile's columns, copied in like the bias
+  float *const lds_scale = reinterpret_cast<float *>(
+      kScaleInSlot ? lds_slot1 + kSlotUsed
+                   : lds_stage + kPStageArea - kTableBytes - kRowSlotBytes - kBiasBytes - 3 * kScaleBufFloats * 4);
   if (wave == 0) {
     TileWalker<BN_OUT> walk(batch, lane);
-    walk.build_table(batch, lane, kQBK, tile_table);
+    walk.build_table(batch, lane, kQBK, tile_table, W8);
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   phase_barrier();
@@ -825,6 +865,14 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   // reads, are the same for every l)
   uint32_t wr_off = qring_off(cp_row0, cp_chunk);
   asm volatile("" : "+v"(wr_off));
+  // fp8 weights: 4 lanes per 64-byte row, 16 rows per load; a lane's 16 bytes
+  // become chunks 2c and 2c + 1 of the bf16 row in LDS.
+  const int cpb_row0 = W8 ? wave * 16 + (lane >> 2) : cp_row0;
+  const int cpb_chunk = W8 ? (lane & 3) : cp_chunk;
+  uint32_t wr_off_b8 = W8 ? qring_off(cpb_row0, 2 * cpb_chunk) : 0;
+  uint32_t wr_off_b8_hi = W8 ? qring_off(cpb_row0, 2 * cpb_chunk + 1) : 0;
+  if constexpr (W8) asm volatile("" : "+v"(wr_off_b8), "+v"(wr_off_b8_hi));
+  const uint32_t w8_magic = W8 ? (uint32_t)(0xffffffffull / (uint32_t)(batch.prob[0].a_div > 0 ? batch.prob[0].a_div : 1) + 1) : 0;
   // Per-lane byte offsets inside the tile being loaded.  Without a row table
   // load i of the activations is row cp_row0 + 32 i: one offset plus a scalar
   // stride.  With one, each of a lane's kCopiesA rows has its own offset, worked
@@ -860,9 +908,25 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
       }
     }
   };
+  auto copy_scale = [&](const PackedTile &pk, int buf) {
+    if constexpr (W8) {
+      const uint32_t row = (uint32_t)__builtin_amdgcn_readlane(pk.words, 22);
+      const int n0 = __builtin_amdgcn_readlane(pk.words, 16), n = __builtin_amdgcn_readlane(pk.words, 17);
+      if (wave == 0) {
+        const float *base = batch.prob[0].w_scale + row;
+        // SwiGLU: 128 gate scales, then the 128 up scales up_offset rows further on;
+        // otherwise the tile's columns, those past the matrix reading as 0
+        const uint32_t bytes = SWIGLU ? (uint32_t)(batch.prob[0].up_offset + 128) * 4 : (uint32_t)(n - n0) * 4;
+        const uint32_t voff = SWIGLU && lane >= 32 ? (uint32_t)batch.prob[0].up_offset * 4 + (lane - 32) * 16 : lane * 16;
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, bytes, kRsrcFlags);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rs, (__attribute__((address_space(3))) void *)(lds_scale + buf * kScaleBufFloats), 16, voff, 0, 0, 0);
+      }
+    }
+  };
   auto set_copy_offsets = [&](const Tile &t) {
     ld_voff_a = (uint32_t)cp_row0 * t.a_pitch + cp_chunk * 16;
-    ld_voff_b = (uint32_t)cp_row0 * t.b_pitch + cp_chunk * 16;
+    ld_voff_b = (uint32_t)cpb_row0 * t.b_pitch + cpb_chunk * 16;
     asm volatile("" : "+v"(ld_voff_a), "+v"(ld_voff_b));
     if constexpr (GATHER) {
 #pragma unroll
@@ -871,7 +935,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
         uint32_t off = ld_voff_a + (uint32_t)(32 * i) * t.a_pitch;
         if (t.a_rows) {
           const uint32_t slot = (uint32_t)lds_row_slots[r];
-          off = r < t.rows ? __umulhi(slot, t.a_magic) * t.a_pitch + cp_chunk * 16 : kOutOfRange;
+          off = r < t.rows ? __umulhi(slot, W8 ? w8_magic : t.a_magic) * t.a_pitch + cp_chunk * 16 : kOutOfRange;
         }
         ld_voff_rows[i] = off;
         asm volatile("" : "+v"(ld_voff_rows[i]));
@@ -910,7 +974,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   f32x16_t acc[TM][TN];
   // (256-wide biased tiles) the accumulators start from the bias of their columns:
   // every 32-row block of a column block gets the same 16 values per lane.
-  auto init_acc = [&](const Tile &t, int buf) {
+  auto init_acc = [&](const Tile &t, int buf, int sbuf) {
     if constexpr (kBiasInAcc) {
       if (uni((int)(t.bias != nullptr))) {
         const float *src = lds_bias + buf * kBiasBufFloats + wave_col0 + frag_half * 4;
@@ -919,7 +983,13 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
           f32x16_t b;
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            const f32x4_t v = *reinterpret_cast<const f32x4_t *>(src + j * 32 + q * 8);
+            f32x4_t v = *reinterpret_cast<const f32x4_t *>(src + j * 32 + q * 8);
+            if constexpr (W8) {  // the epilogue multiplies the sums by the scale
+              const f32x4_t sc = *reinterpret_cast<const f32x4_t *>(
+                  lds_scale + sbuf * kScaleBufFloats + wave_col0 + frag_half * 4 + j * 32 + q * 8);
+#pragma unroll
+              for (int r = 0; r < 4; ++r) v[r] = v[r] / sc[r];
+            }
 #pragma unroll
             for (int r = 0; r < 4; ++r) b[q * 4 + r] = v[r];
           }
@@ -953,9 +1023,11 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   Tile ld = unpack_tile(nxt);                     // tile being loaded
   if (!ld.valid) return;                          // nothing to do for this workgroup
   int bias_buf = 0;                               // buffer that holds the bias of the tile being multiplied
-  if constexpr (GATHER || kBiasInAcc) {
+  int scale_buf = 0;                              // ... and its scales (one of three)
+  if constexpr (GATHER || kBiasInAcc || W8) {
     copy_row_slots(nxt);
     copy_bias(nxt, 0);
+    copy_scale(nxt, 0);
     pwait_vmcnt<0>();
     phase_barrier();
   }
@@ -969,6 +1041,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
     copy_row_slots(nxt);
   }
   copy_bias(nxt, 1);
+  copy_scale(nxt, 1);
   auto advance_copy = [&]() {
     if (++ld_kt == ld.steps) {
       ld = unpack_tile(nxt);
@@ -979,7 +1052,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   // A step's loads in four quarters: the two halves of the activation rows, then
   // the two halves of the weight rows.  first(q) .. first(q + 1) are quarter q's
   // indices into the register stage.
-  auto quarter_first = [](int q) { return q <= 2 ? q * (kCopiesA / 2) : kCopiesA + kCopiesB / 2; };
+  auto quarter_first = [](int q) { return q <= 2 ? q * (kCopiesA / 2) : kCopiesA + (kCopiesB + 1) / 2; };
   // Quarter q of the step the load side stands at, into register stage P.
   auto load_quarter = [&](auto stage_c, auto q_c) {
     constexpr int P = decltype(stage_c)::value, Q = decltype(q_c)::value;
@@ -995,12 +1068,13 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
         stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, uni(ld_kt * 128), 0);
       } else {
         const int i = l - kCopiesA;
-        const bool up_half = SWIGLU && 32 * i >= BN / 2;  // wave * 8 + 7 < 32 never crosses the halves
-        const int row = up_half ? 32 * i - BN / 2 : 32 * i;
+        constexpr int kStride = kRowsPerCopyB * kQWaves;  // weight rows between a lane's consecutive loads
+        const bool up_half = SWIGLU && kStride * i >= BN / 2;  // a wave's rows of one load never cross the halves
+        const int row = up_half ? kStride * i - BN / 2 : kStride * i;
         const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
             (void *)uni(up_half ? ld.b1 : ld.b0), 0, uni(ld.b_bytes), kRsrcFlags);
         stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(
-            rs, ld_voff_b + (uint32_t)row * uni(ld.b_pitch), uni(ld_kt * 128), 0);
+            rs, ld_voff_b + (uint32_t)row * uni(ld.b_pitch), uni(ld_kt * (W8 ? 64 : 128)), 0);
       }
     }
   };
@@ -1010,8 +1084,23 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
 #pragma unroll
     for (int l = quarter_first(Q); l < (Q == 3 ? kQCopies : quarter_first(Q + 1)); ++l) {
       const int i = l < kCopiesA ? l : l - kCopiesA;
-      unsigned char *dst = (P == 0 ? lds_slot0 : lds_slot1) + (l < kCopiesA ? 0 : kPBM * 128) + i * 32 * 128 + wr_off;
-      *reinterpret_cast<u32x4_any_t *>(dst) = stage_regs[P][l];
+      if (W8 && l >= kCopiesA) {
+        unsigned char *row = (P == 0 ? lds_slot0 : lds_slot1) + kPBM * 128 + i * (kRowsPerCopyB * kQWaves) * 128;
+        const u32x4_t src = stage_regs[P][l];
+        u32x4_t lo, hi;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          lo[2 * q] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(src[q], 1.0f, false));
+          lo[2 * q + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(src[q], 1.0f, true));
+          hi[2 * q] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(src[q + 2], 1.0f, false));
+          hi[2 * q + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(src[q + 2], 1.0f, true));
+        }
+        *reinterpret_cast<u32x4_any_t *>(row + wr_off_b8) = lo;
+        *reinterpret_cast<u32x4_any_t *>(row + wr_off_b8_hi) = hi;
+      } else {
+        unsigned char *dst = (P == 0 ? lds_slot0 : lds_slot1) + (l < kCopiesA ? 0 : kPBM * 128) + i * 32 * 128 + wr_off;
+        *reinterpret_cast<u32x4_any_t *>(dst) = stage_regs[P][l];
+      }
     }
   };
   auto load_step = [&](auto stage_c) {
@@ -1031,7 +1120,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   load_step(c0);           // step 2
   write_quarter(c1, c0);
   load_quarter(c1, c0);    // first quarter of step 3; the stage keeps quarters 1..3 of step 1
-  init_acc(cp, 0);
+  init_acc(cp, 0, 0);
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   phase_barrier();
   read_frags(c0, c0, 0);
@@ -1078,7 +1167,8 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
       step(c0);
       step(c1);
     }
-    tile_epilogue<MODE, HAS_BIAS && !kBiasInAcc, kQWaves, TM, TN>(cp, acc, stage_rows, wm * WTM, wave_col0, lane);
+    tile_epilogue<MODE, HAS_BIAS && !kBiasInAcc, kQWaves, TM, TN, W8, W8 ? kEpiReserve : 0>(
+        cp, acc, stage_rows, wm * WTM, wave_col0, lane, lds_scale + scale_buf * kScaleBufFloats);
     // The load side is within the next tile here (every tile has at least
     // kQMinSteps steps).
     cp = ld;
@@ -1094,7 +1184,9 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
     // below was filled a whole tile ago: the same ordering as for the row slots)
     copy_bias(nxt, bias_buf);
     bias_buf ^= 1;
-    init_acc(cp, bias_buf);
+    scale_buf = scale_buf == 2 ? 0 : scale_buf + 1;       // the tile multiplied next
+    copy_scale(nxt, scale_buf == 2 ? 0 : scale_buf + 1);  // the one after it
+    init_acc(cp, bias_buf, scale_buf);
     // The last block above already fetched these fragments; reading them again
     // here keeps 32 registers free during the epilogue.
     read_frags(c0, c0, 0);
@@ -1109,9 +1201,9 @@ __global__ __launch_bounds__(8 * kWave, 1) void gemm_persist_kernel8(PersistBatc
   gemm_persist_body<MODE, HAS_BIAS, 8>(batch);
 }
 // Four waves, one per SIMD, each with the whole 512-entry register file.
-template <int MODE, bool HAS_BIAS, int BN, bool GATHER>
+template <int MODE, bool HAS_BIAS, int BN, bool GATHER, bool W8 = false>
 __global__ __launch_bounds__(4 * kWave, 1) void gemm_persist_kernel4(PersistBatch batch) {
-  gemm_persist64_body<MODE, HAS_BIAS, BN, GATHER>(batch);
+  gemm_persist64_body<MODE, HAS_BIAS, BN, GATHER, W8>(batch);
 }
 
 }  // namespace
@@ -1155,6 +1247,7 @@ bool persist64_ok(const PersistBatch &b, int mode) {
   for (int i = 0; i < b.n_problems; ++i) {
     const PersistProblem &p = b.prob[i];
     if (p.k < kQBK * kQMinSteps) return false;
+    if (p.w_scale && b.n_problems != 1) return false;  // fp8 weights: single-problem launches
     if (p.a_rows) {  // gathered activation rows: SwiGLU instantiation only (the GELU one would
                      // spill, and measures no faster than a gathered copy plus the plain kernel)
       if (mode != kFc1Swiglu) return false;
@@ -1177,7 +1270,7 @@ int persist_variant(const PersistBatch &b, int mode) {
   if (!persist_common_ok(b, mode)) return 0;
   if (g_persist_waves == 4 && persist64_ok(b, mode)) return 4;
   for (int i = 0; i < b.n_problems; ++i)
-    if (b.prob[i].a_rows) return 0;  // the 32-k kernel wants contiguous rows
+    if (b.prob[i].a_rows || b.prob[i].w_scale) return 0;  // the 32-k kernel wants contiguous rows and bf16 weights
   return 8;
 }
 
@@ -1199,7 +1292,23 @@ int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s) 
   bool narrow = mode != kFc1Swiglu;
   for (int i = 0; i < b.n_problems; ++i)
     narrow = narrow && b.prob[i].n % 192 == 0 && b.prob[i].n % 256 != 0;
-  if (waves == 4 && narrow) {
+  const bool w8 = b.prob[0].w_scale != nullptr;
+  if (waves == 4 && w8) {
+    if (narrow) {
+      switch (mode) {
+        case kFc1Gelu: kern = has_bias ? gemm_persist_kernel4<kFc1Gelu, true, 192, false, true> : gemm_persist_kernel4<kFc1Gelu, false, 192, false, true>; break;
+        default: kern = has_bias ? gemm_persist_kernel4<kFc2, true, 192, false, true> : gemm_persist_kernel4<kFc2, false, 192, false, true>; break;
+      }
+    } else {
+      switch (mode) {
+        case kFc1Swiglu:
+          kern = gathered ? gemm_persist_kernel4<kFc1Swiglu, false, 256, true, true> : gemm_persist_kernel4<kFc1Swiglu, false, 256, false, true>;
+          break;
+        case kFc1Gelu: kern = has_bias ? gemm_persist_kernel4<kFc1Gelu, true, 256, false, true> : gemm_persist_kernel4<kFc1Gelu, false, 256, false, true>; break;
+        default: kern = has_bias ? gemm_persist_kernel4<kFc2, true, 256, false, true> : gemm_persist_kernel4<kFc2, false, 256, false, true>; break;
+      }
+    }
+  } else if (waves == 4 && narrow) {
     switch (mode) {
       case kFc1Gelu: kern = has_bias ? gemm_persist_kernel4<kFc1Gelu, true, 192, false> : gemm_persist_kernel4<kFc1Gelu, false, 192, false>; break;
       default: kern = has_bias ? gemm_persist_kernel4<kFc2, true, 192, false> : gemm_persist_kernel4<kFc2, false, 192, false>; break;

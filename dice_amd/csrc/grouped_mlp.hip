@@ -134,7 +134,8 @@ int grouped_mlp_impl(int stages, const void *x, int act_dtype, const int32_t *pe
   const bool swiglu = act_variant == DICE_ACT_SWIGLU;
 
   // Contiguous grouped rows + bf16 weights: the persistent kernel applies.
-  if (!perm && act_dtype == DICE_BF16 && w_dtype == DICE_BF16 && gemm_config_wants_persistent()) {
+  if (!perm && act_dtype == DICE_BF16 && (w_dtype == DICE_BF16 || w_dtype == DICE_FP8_E4M3) &&
+      gemm_config_wants_persistent()) {
     PersistBatch pb1{};
     pb1.n_problems = 1;
     pb1.prob[0] = PersistProblem{x, hidden, offsets, n_experts, w1, swiglu ? 2 * inter : inter, inter,
@@ -143,6 +144,10 @@ int grouped_mlp_impl(int stages, const void *x, int act_dtype, const int32_t *pe
     pb2.n_problems = 1;
     pb2.prob[0] = PersistProblem{h, inter, offsets, n_experts, w2, hidden, 0, swiglu ? nullptr : b2,
                                  out, hidden, hidden, inter, (int)max_rows};
+    if (w_dtype == DICE_FP8_E4M3) {
+      pb1.prob[0].w_scale = w1_scale;
+      pb2.prob[0].w_scale = w2_scale;
+    }
     const int m1 = swiglu ? kFc1Swiglu : kFc1Gelu;
     if (persist_supported(pb1, m1) && persist_supported(pb2, kFc2)) {
       if (stages & 1) {
@@ -346,10 +351,12 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
   const uint8_t *mask = combine_mode == 0 ? nullptr : skip_mask;
   const float *combine_wt = use_latest_weights ? wt : emit.topk_weight;
 
-  // bf16 path: two persistent launches, each covering the routed experts and
-  // the shared expert together.
+  // bf16 activations: two persistent launches, each covering the routed experts
+  // and the shared expert together; with fp8 routed weights the shared expert
+  // (bf16) gets launches of its own.
   bool done = false;
-  if (L->act_dtype == DICE_BF16 && LE->w_dtype == DICE_BF16) {
+  const bool w8 = LE->w_dtype == DICE_FP8_E4M3;
+  if (L->act_dtype == DICE_BF16 && (LE->w_dtype == DICE_BF16 || (w8 && LE->w1_scale && LE->w2_scale))) {
     const bool swiglu = L->act_variant == DICE_ACT_SWIGLU;
     const int m1 = swiglu ? kFc1Swiglu : kFc1Gelu;
     PersistBatch f1{}, f2{};
@@ -361,14 +368,29 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
                                 swiglu ? nullptr : LE->b2, work.rows, L->hidden, L->hidden, L->inter,
                                 (int)max_rows};
     f1.n_problems = f2.n_problems = 1;
+    if (w8) {
+      f1.prob[0].w_scale = LE->w1_scale;
+      f2.prob[0].w_scale = LE->w2_scale;
+    }
+    PersistBatch s1{}, s2{};  // the shared expert on its own (fp8 routed weights only)
     if (L->shared_inter > 0) {
       const int si = L->shared_inter;
-      f1.prob[1] = PersistProblem{x, L->hidden, w.shared_offsets, 1, L->shared_w1, swiglu ? 2 * si : si, si,
-                                  swiglu ? nullptr : L->shared_b1, w.shared_h, si, si, L->hidden, (int)n_tokens};
-      f2.prob[1] = PersistProblem{w.shared_h, si, w.shared_offsets, 1, L->shared_w2, L->hidden, 0,
-                                  swiglu ? nullptr : L->shared_b2, w.shared_out, L->hidden, L->hidden, si, (int)n_tokens};
-      f1.n_problems = f2.n_problems = 2;
+      const PersistProblem p1{x, L->hidden, w.shared_offsets, 1, L->shared_w1, swiglu ? 2 * si : si, si,
+                              swiglu ? nullptr : L->shared_b1, w.shared_h, si, si, L->hidden, (int)n_tokens};
+      const PersistProblem p2{w.shared_h, si, w.shared_offsets, 1, L->shared_w2, L->hidden, 0,
+                              swiglu ? nullptr : L->shared_b2, w.shared_out, L->hidden, L->hidden, si, (int)n_tokens};
+      if (w8) {
+        s1.prob[0] = p1;
+        s2.prob[0] = p2;
+        s1.n_problems = s2.n_problems = 1;
+      } else {
+        f1.prob[1] = p1;
+        f2.prob[1] = p2;
+        f1.n_problems = f2.n_problems = 2;
+      }
     }
+    const bool shared_ok =
+        s1.n_problems == 0 || (persist_supported(s1, m1) && persist_supported(s2, kFc2));
     // Where the kernel can address the activation rows through the permutation
     // itself, the gathered copy is skipped.
     PersistBatch f1g = f1;
@@ -376,8 +398,8 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
     f1g.prob[0].a_rows = work.perm;
     f1g.prob[0].a_div = L->top_k;
     f1g.prob[0].a_src_rows = (int)n_tokens;
-    const bool fused_gather = persist_supported(f1g, m1) && persist_supported(f2, kFc2);
-    if (fused_gather || (persist_supported(f1, m1) && persist_supported(f2, kFc2))) {
+    const bool fused_gather = shared_ok && persist_supported(f1g, m1) && persist_supported(f2, kFc2);
+    if (fused_gather || (shared_ok && persist_supported(f1, m1) && persist_supported(f2, kFc2))) {
       if (fused_gather) {
         f1 = f1g;
       } else {
@@ -388,9 +410,17 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
       stamp(3, s);
       rc = launch_grouped_gemm_persist(f1, m1, s);
       if (rc) return rc;
+      if (s1.n_problems) {
+        rc = launch_grouped_gemm_persist(s1, m1, s);
+        if (rc) return rc;
+      }
       stamp(4, s);
       rc = launch_grouped_gemm_persist(f2, kFc2, s);
       if (rc) return rc;
+      if (s2.n_problems) {
+        rc = launch_grouped_gemm_persist(s2, kFc2, s);
+        if (rc) return rc;
+      }
       stamp(5, s);
       done = true;
     }

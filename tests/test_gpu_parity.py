@@ -372,6 +372,59 @@ def test_mlp_fp8_weights(dev, variant, cfg):
     assert rel_l2(out, want_m) < FP8_TOL
 
 
+@pytest.mark.parametrize("variant", ["swiglu", "gelu_tanh"])
+@pytest.mark.parametrize("D,ratio,counts", [
+    (1152, 4, None),                                   # XL width: 192-wide fc2 tiles, several tiles per workgroup
+    (512, 4, [0, 1, 700, 0, 257, 3, 1086, 1]),         # 256-wide fc2 tiles; empty, one-row and ragged groups
+    (2048, 2, None),                                   # DiT-G width
+])
+def test_mlp_fp8_weights_persistent_kernel(dev, variant, D, ratio, counts):
+    """fp8 weights through the 64-k persistent kernels (contiguous grouped rows):
+    the bytes are widened to bf16 on their way into LDS, the per-channel scale
+    multiplies the fp32 sums, and a bias enters the accumulators divided by it."""
+    from dice_amd import lib, ops
+    E, N = 8, 1024
+    g = _gen(31 + D)
+    p = O.make_block_params(D, E, 2, ratio, n_shared=0, seed=6, dtype=torch.bfloat16, variant=variant)
+    if variant == "gelu_tanh":
+        for e in p.experts:
+            e.fc1_b = (torch.randn(e.fc1_b.shape, generator=g) * 0.1).bfloat16()
+            e.fc2_b = (torch.randn(e.fc2_b.shape, generator=g) * 0.1).bfloat16()
+    x = torch.randn(N, D, generator=g).bfloat16()
+    if counts is None:
+        idx = torch.randint(0, E, (N * 2,), generator=g)
+    else:
+        idx = torch.cat([torch.full((c,), e) for e, c in enumerate(counts)])
+        idx = idx[torch.randperm(idx.numel(), generator=g)]
+    _, offsets, perm, _ = O.dispatch_tables(idx, E)
+    xg = x[perm // 2]
+    w1, w2, b1, b2 = _packed(p, variant, torch.bfloat16, dev)
+    q1, s1 = ops.quantize_fp8_rowwise(w1)
+    q2, s2 = ops.quantize_fp8_rowwise(w2)
+    lib.load().dice_set_gemm_config(21, 21)
+    try:
+        out = ops.grouped_mlp(xg.to(dev), None, 1, offsets.int().to(dev), N * 2, q1, q2, variant, b1, b2,
+                              s1, s2).cpu()
+    finally:
+        lib.load().dice_set_gemm_config(0, 0)
+    d1 = O.dequantize_fp8_rowwise(q1.cpu().view(-1, q1.shape[-1]), s1.cpu().view(-1)).view(w1.shape)
+    d2 = O.dequantize_fp8_rowwise(q2.cpu().view(-1, q2.shape[-1]), s2.cpu().view(-1)).view(w2.shape)
+    inter = ratio * D
+    want = torch.empty(N * 2, D)
+    for e in range(E):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        if hi == lo:
+            continue
+        xs = xg[lo:hi].float()
+        if variant == "swiglu":
+            want[lo:hi] = O.moe_mlp(xs, d1[e, :inter], d1[e, inter:], d2[e])
+        else:
+            want[lo:hi] = O.gelu_mlp(xs, d1[e], b1[e].cpu(), d2[e], b2[e].cpu())
+    assert rel_l2(out, want) < BF16_TOL, rel_l2(out, want)
+    err = (out.double() - want.double()).norm(dim=1) / want.double().norm(dim=1).clamp_min(1e-6)
+    assert err.max() < 5 * BF16_TOL, f"worst row {int(err.argmax())} rel err {float(err.max())}"
+
+
 # --------------------------------------------------------------------------- #
 # whole block
 # --------------------------------------------------------------------------- #
