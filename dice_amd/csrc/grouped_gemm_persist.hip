@@ -29,8 +29,10 @@
 // weights at the same time.
 //
 // Weights are [experts, rows, k] bf16 as in the reference's nn.Linear layout
-// (models.py:245-247); activations are grouped rows (contiguous, or rows of
-// the token matrix named by a row table).
+// (models.py:245-247), or fp8 (e4m3) bytes of the same shape with one fp32
+// scale per output channel (64-k pipeline only: widened to bf16 on the way into
+// LDS, scale applied to the fp32 sums); activations are grouped rows
+// (contiguous, or rows of the token matrix named by a row table).
 #include <type_traits>
 
 #include "gemm_common.h"
