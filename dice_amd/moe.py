@@ -330,6 +330,11 @@ class SparseMoeBlock(nn.Module):
         ws = self._workspace(desc, n, x.device)
         new = diep.LagEntry(x, len(self.experts), self.num_experts_per_tok, bool(skip_now), owner=self)
         work, emit = diep.lag_roles(self.layer_idx, new)
+        for entry in (work, emit):
+            if entry.x.shape != x.shape or entry.x.dtype != x.dtype or entry.x.device != x.device:
+                raise DiceError(f"layer {self.layer_idx}: a cached step holds {tuple(entry.x.shape)} {entry.x.dtype} "
+                                f"activations, this call {tuple(x.shape)} {x.dtype}: clear the caches and force a "
+                                "synchronous step when the batch changes")
         work.ensure_rows()
         if emit.rows is None:
             raise DiceError("the cached step to return has never been through the experts")

@@ -34,6 +34,48 @@ def test_layer_struct_matches_header_layout():
     assert ctypes.sizeof(MoeLayerDesc) == 40 + 12 * 8
 
 
+def test_lag_entry_and_caller_structs_match_header_layout():
+    from dice_amd.lib import CallerDesc, LagEntryDesc
+    # dice_moe_lag_entry_t: six pointers and an int64; dice_moe_caller_t: three pointers, int64, float (+ padding)
+    assert LagEntryDesc.max_rows.offset == 48 and ctypes.sizeof(LagEntryDesc) == 56
+    assert CallerDesc.tokens_per_sample.offset == 24 and CallerDesc.ln_eps.offset == 32
+    assert ctypes.sizeof(CallerDesc) == 40
+
+
+def test_new_entry_points_report_bad_arguments():
+    from dice_amd import lib
+    from dice_amd.lib import CallerDesc, LagEntryDesc, MoeLayerDesc
+    cdll = lib.load()
+    one = ctypes.c_void_p(16)
+    rc = cdll.dice_ln_modulate(one, one, None, one, 1, 8, 64, 4, 1e-6, None)
+    assert rc == -1 and b"null pointer" in cdll.dice_last_error()
+    rc = cdll.dice_ln_modulate(one, one, one, one, 1, 8, 64, 0, 1e-6, None)
+    assert rc == -1 and b"tokens_per_sample" in cdll.dice_last_error()
+    rc = cdll.dice_ln_modulate(one, one, one, one, 1, 8, 60, 4, 1e-6, None)
+    assert rc == -1 and b"16 bytes" in cdll.dice_last_error()
+    rc = cdll.dice_ln_modulate(one, one, one, one, 1, 8, 1 << 16, 4, 1e-6, None)
+    assert rc == -2
+    rc = cdll.dice_combine_residual(one, None, one, None, None, None, None, one, None, 4, one, 1, 8, 2, 64, None)
+    assert rc == -1
+    d = MoeLayerDesc()
+    d.hidden, d.inter, d.n_experts, d.top_k, d.act_dtype, d.w_dtype = 128, 512, 8, 2, 1, 1
+    d.gate_w = d.w1 = d.w2 = 16
+    rc = cdll.dice_moe_forward_modulated(ctypes.byref(d), None, one, 8, 0, None, None, None, one, None, None,
+                                         one, 1 << 30, None)
+    assert rc == -1
+    c = CallerDesc()            # shift / scale / gate left NULL
+    rc = cdll.dice_moe_forward_modulated(ctypes.byref(d), ctypes.byref(c), one, 8, 0, None, None, None, one, None,
+                                         None, one, 1 << 30, None)
+    assert rc == -1 and b"shift" in cdll.dice_last_error()
+    e = LagEntryDesc()          # an entry without buffers
+    rc = cdll.dice_moe_forward_lagged(ctypes.byref(d), None, one, 8, 0, None, ctypes.byref(e), None, None, 0, None,
+                                      None, 0, None, one, None, None, one, 1 << 30, None)
+    assert rc == -1 and b"lacks a buffer" in cdll.dice_last_error()
+    rc = cdll.dice_moe_forward_lagged(ctypes.byref(d), None, one, 8, 1, None, None, None, None, 0, None,
+                                      None, 0, None, one, None, None, one, 1 << 30, None)
+    assert rc == -1 and b"skip_mask" in cdll.dice_last_error()
+
+
 def test_bad_arguments_are_reported_without_touching_a_gpu():
     from dice_amd import lib
     cdll = lib.load()

@@ -167,3 +167,23 @@ def test_lagged_call_without_forced_sync_is_refused(dev):
             blk(torch.randn(1, 64, D).to(dev))
     finally:
         _reset(diep)
+
+
+def test_batch_change_between_lagged_steps_is_refused(dev):
+    """A cached step only fits calls of its own shape: a different token count
+    without a forced-sync step in between raises instead of reading the old
+    tables out of range."""
+    from dice_amd import DiceError, ParaMode, diep
+    D = 256
+    p = O.make_block_params(D, 8, 2, 4, 2, seed=1)
+    pm = ParaMode(ep=True, ep_async=True, ep_async_mode="all")
+    blk = block_from_params(p, D, "swiglu", torch.float32, dev, para_mode=pm)
+    diep.ep_cache_init(cache_capacity=1)
+    try:
+        diep.diep_force_sync()
+        blk(torch.randn(1, 64, D).to(dev))
+        diep.diep_cancel_sync()
+        with pytest.raises(DiceError, match="batch changes"):
+            blk(torch.randn(1, 96, D).to(dev))
+    finally:
+        _reset(diep)
