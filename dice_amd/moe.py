@@ -292,6 +292,8 @@ class SparseMoeBlock(nn.Module):
             raise DiceError("SparseMoeBlock: only the inference branch is implemented (call .eval())")
         orig_shape = hidden_states.shape
         x = hidden_states.reshape(-1, orig_shape[-1]).contiguous()
+        if x.shape[0] == 0:  # no tokens: nothing to route, nothing to cache
+            return out if out is not None else torch.empty_like(hidden_states)
         y = None if out is None else out.view(-1, orig_shape[-1])
         if not self.para_mode.ep:
             return self.run(x, y=y, caller=caller).view(*orig_shape)

@@ -453,6 +453,33 @@ def test_block_c1_fp32(dev, variant):
     assert rel_l2(y_n.view(-1, 384)[~ties], want_n.view(-1, 384)[~ties]) < FP32_TOL
 
 
+@pytest.mark.parametrize("N,D,E,k,dtype", [
+    (1, 768, 8, 2, torch.bfloat16),        # a single token: seven experts empty, one-row groups
+    (7, 768, 8, 2, torch.bfloat16),
+    (257, 768, 16, 2, torch.bfloat16),     # DiT-B width, 16 experts, one row past a tile
+    (1000, 1024, 16, 2, torch.bfloat16),   # DiT-L width
+    (333, 1408, 16, 2, torch.bfloat16),    # DiT-G width (11 x 128)
+    (130, 384, 8, 1, torch.float32),       # top-1
+    (130, 384, 8, 4, torch.float32),       # top-4
+    (64, 384, 64, 2, torch.float32),       # as many experts as the layer call takes
+])
+def test_block_odd_shapes(dev, N, D, E, k, dtype):
+    """Token counts that fill no tile, every model width of the reference's
+    configurations (models.py:769-806), other top-k and expert counts."""
+    p = O.make_block_params(D, E, k, 4, 2, seed=11, dtype=dtype, gate_std=0.1)
+    x = torch.randn(1, N, D, generator=_gen(N + D)).to(dtype)
+    want, widx, _, logits = O.sparse_moe_block_forward(p, x)
+    blk, y = _run_block(dev, p, x, "swiglu", dtype)
+    ok = ~O.gate_tie_rows(logits, k)
+    assert ok.float().mean() > 0.95
+    assert rel_l2(y[0][ok], want[0][ok]) < (FP32_TOL if dtype == torch.float32 else BF16_TOL)
+    idx, _, _ = blk.gate(x.to(dev))
+    assert torch.equal(idx.cpu()[ok], widx[ok])
+    # zero tokens: nothing to do, nothing launched
+    empty = blk(torch.empty(1, 0, D, dtype=dtype, device=dev))
+    assert empty.shape == (1, 0, D)
+
+
 def _subset_oracle(p, x2d, sub, dtype):
     """Tokens are independent through the block, so the oracle on a subset of
     rows must equal the same rows of the full-size result."""
