@@ -134,6 +134,50 @@ def time_stages(blk, x, steps):
     return {names[i]: acc[i] / steps for i in range(n)}
 
 
+def time_staleness(variant, dev, x, sample_steps=50):
+    """Configuration 4: the conditional-communication loop of the reference sampler
+    (diffusion/rectified_flow.py:83-105) on this layer: 50 steps counted down, the first a
+    full step, then skip steps (half of the routed slots recomputed, the other half read
+    from the per-layer cache) alternating with full steps that refill the cache; x drifts
+    by 0.05 N(0,1) per step.  Returns ms per step for each strategy and per step kind."""
+    from dice_amd import ParaMode, diep
+    blk = make_block(variant, dev, 0, 1, ParaMode(ep=True))
+    xv = x.view(1, N_TOKENS, D)
+    g = torch.Generator(device=dev).manual_seed(4)
+    noise = [0.05 * torch.randn(xv.shape, generator=g, device=dev, dtype=torch.float32) for _ in range(4)]
+    out = {}
+    try:
+        for mode in ("high", "low", "rand"):
+            diep.ep_cache_init(cache_capacity=1, noskip_step=2, skip_mode=mode)
+            diep.ep_set_rand_mask(None)
+            kinds = {"full": [0.0, 0], "skip": [0.0, 0]}
+            total = 0.0
+            for rep in range(2):            # first repetition warms up
+                xt = xv.clone()
+                for i in range(sample_steps, 0, -1):
+                    diep.ep_set_step(i)
+                    if diep.ep_forced_sync(i, sample_steps):
+                        diep.ep_cache_clear()
+                    kind = "skip" if diep.ep_skip_now(0) else "full"
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    blk(xt)
+                    torch.cuda.synchronize()
+                    dt = time.perf_counter() - t0
+                    if rep == 1:
+                        kinds[kind][0] += dt
+                        kinds[kind][1] += 1
+                        total += dt
+                    xt = (xt.float() + noise[i % 4]).to(xt.dtype)
+            out[mode] = {"ms_per_step": total / sample_steps * 1e3,
+                         "full_put_step_ms": kinds["full"][0] / max(1, kinds["full"][1]) * 1e3,
+                         "skip_step_ms": kinds["skip"][0] / max(1, kinds["skip"][1]) * 1e3,
+                         "full_steps": kinds["full"][1], "skip_steps": kinds["skip"][1]}
+    finally:
+        diep.ep_cache_init(cache_capacity=1, noskip_step=1)
+    return out
+
+
 def time_lagged(variant, dev, x, steps, warmup, pipeline):
     """ms per layer call of the step-lagged modes on the same block shape: two
     layers, a forced-sync first step, then `steps` lagged steps (displaced: each
@@ -248,6 +292,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-stages", action="store_true", help="skip the per-kernel timing pass")
     ap.add_argument("--no-caller", action="store_true", help="skip the fused-caller (LayerNorm/modulate + residual) pass")
+    ap.add_argument("--no-staleness", action="store_true", help="skip the 50-step conditional-communication loop")
     ap.add_argument("--no-lagged", action="store_true", help="skip the step-lagged (displaced / interweaved) pass")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a known-size kernel to scale "
@@ -326,6 +371,9 @@ def main():
         out["hbm_stage_frac_of_peak"] = {s: v / PEAK_HBM_GBS for s, v in out["hbm_stage_gbs"].items()}
     if not args.no_caller:
         out["block_moe_half_ms"] = time_caller(blk, x, args.steps, args.warmup)
+    if not args.no_staleness:
+        # configs[3]: the 50-step conditional-communication loop (synchronised per step: host-visible latency)
+        out["staleness_loop_50_steps"] = time_staleness(args.variant, dev, x)
     if not args.no_lagged:
         # the same layer under the reference's step-lagged schedules (not part of `value`)
         out["step_lag_ms_per_layer_call"] = {
