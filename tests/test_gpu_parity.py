@@ -425,6 +425,40 @@ def test_mlp_fp8_weights_persistent_kernel(dev, variant, D, ratio, counts):
     assert err.max() < 5 * BF16_TOL, f"worst row {int(err.argmax())} rel err {float(err.max())}"
 
 
+@pytest.mark.parametrize("variant,fp8", [("swiglu", False), ("gelu_tanh", False), ("swiglu", True), ("gelu_tanh", True)])
+def test_persistent_kernels_rerun_bit_identical(dev, variant, fp8):
+    """The persistent kernels stage tile tables, row numbers, biases and scales
+    in LDS one tile ahead of their use; every workgroup multiplies several
+    tiles in a row here, and twenty back-to-back launches on the same inputs
+    must agree bit for bit (a buffer overwritten too early would show as a
+    difference between runs)."""
+    from dice_amd import lib, ops
+    N, D, E, ratio = 4096, 1152, 8, 4
+    g = _gen(77)
+    p = O.make_block_params(D, E, 2, ratio, n_shared=0, seed=8, dtype=torch.bfloat16, variant=variant)
+    if variant == "gelu_tanh":
+        for e in p.experts:
+            e.fc1_b = (torch.randn(e.fc1_b.shape, generator=g) * 0.1).bfloat16()
+            e.fc2_b = (torch.randn(e.fc2_b.shape, generator=g) * 0.1).bfloat16()
+    x = torch.randn(N * 2, D, generator=g).bfloat16().to(dev)
+    idx = torch.randint(0, E, (N * 2,), generator=g)
+    _, offsets, _, _ = O.dispatch_tables(idx, E)
+    offsets = offsets.int().to(dev)
+    w1, w2, b1, b2 = _packed(p, variant, torch.bfloat16, dev)
+    s1 = s2 = None
+    if fp8:
+        w1, s1 = ops.quantize_fp8_rowwise(w1)
+        w2, s2 = ops.quantize_fp8_rowwise(w2)
+    lib.load().dice_set_gemm_config(21, 21)
+    try:
+        outs = [ops.grouped_mlp(x, None, 1, offsets, N * 2, w1, w2, variant, b1, b2, s1, s2) for _ in range(20)]
+        torch.cuda.synchronize()
+    finally:
+        lib.load().dice_set_gemm_config(0, 0)
+    assert all(torch.equal(o, outs[0]) for o in outs[1:])
+    assert torch.isfinite(outs[0].float()).all()
+
+
 # --------------------------------------------------------------------------- #
 # whole block
 # --------------------------------------------------------------------------- #
