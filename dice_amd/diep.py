@@ -88,6 +88,19 @@ class LagEntry:
         self.dropped = dropped
         self.owner = owner
 
+    @classmethod
+    def from_tables(cls, x, offsets, perm, inv_perm, topk_weight, top_k: int, dropped: bool, owner=None):
+        """An entry around routing tables that already exist (``x`` is kept as
+        given: pass a copy if the caller may change it)."""
+        e = cls.__new__(cls)
+        n = x.shape[0]
+        e.x, e.offsets, e.perm, e.inv_perm, e.topk_weight = x, offsets, perm, inv_perm, topk_weight
+        e.rows = None
+        e.max_rows = n * (top_k - 1) if dropped else n * top_k
+        e.dropped = dropped
+        e.owner = owner
+        return e
+
     def ensure_rows(self):
         if self.rows is None:
             self.rows = torch.empty((max(self.max_rows, 1), self.x.shape[-1]), dtype=self.x.dtype,

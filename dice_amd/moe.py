@@ -150,6 +150,8 @@ class SparseMoeBlock(nn.Module):
         else:
             raise DiceError(f"unknown expert variant {variant}")
         self.experts = nn.ModuleList([mk(inter) for _ in range(num_experts)])
+        from .ep_fwd import register_experts
+        register_experts(self.experts, self)  # lets moe_infer_ep(inp, block.experts, ...) find the packed weights
         self.gate = MoEGate(embed_dim, num_experts, num_experts_per_tok)
         self.n_shared_experts = n_shared_experts
         if self.n_shared_experts is not None:

@@ -187,3 +187,48 @@ def test_batch_change_between_lagged_steps_is_refused(dev):
             blk(torch.randn(1, 96, D).to(dev))
     finally:
         _reset(diep)
+
+
+@pytest.mark.parametrize("async_op", [False, True])
+@pytest.mark.parametrize("skip", [None, "high"])
+def test_moe_infer_ep_function_follows_oracle(dev, async_op, skip):
+    """The functional boundary of the reference (expertpara/ep_fwd.py:19) with
+    the caller's own routing, driven like the reference's test of it
+    (tests/test_ep.py:79-124): random expert ids (a token may name one expert
+    twice) and random weights per iteration, forced-sync first iteration."""
+    from dice_amd import ParaMode, diep
+    from dice_amd.ep_fwd import moe_infer_ep
+    D, E, N, k = 256, 8, 128, 2
+    p = O.make_block_params(D, E, k, 4, None, seed=21)
+    blk = block_from_params(p, D, "swiglu", torch.float32, dev, para_mode=ParaMode(ep=True))
+    noskip = 2 if skip else 1
+    diep.ep_cache_init(cache_capacity=1, noskip_step=noskip, skip_mode=skip)
+    diep.use_latest_expert_weights(False)
+    state = O.DiepState(1, noskip_step=noskip, skip_mode=skip)
+    mask = O.skip_mask(N * k, skip) if skip else None
+    g = _gen(60)
+    try:
+        for it in range(6):
+            step = 6 - it
+            diep.ep_set_step(step)
+            state.step = step
+            if it == 0:
+                diep.diep_force_sync()
+                diep.ep_cache_clear()
+                state.force_sync()
+                state.cache_clear()
+            elif it == 1:
+                diep.diep_cancel_sync()
+                state.cancel_sync()
+            x = torch.randn(N, D, generator=g)
+            idx = torch.randint(0, E, (N * k,), generator=g)
+            w = torch.rand(N * k, 1, generator=g)
+            now = O.skip_now(True, state.skip, 0, step, noskip) if skip else None
+            if skip:
+                assert diep.ep_skip_now(0) == now
+            want = O.moe_infer_ep_async(state, x, p.experts, idx, w, k, async_op, mask, now, 0)
+            got = moe_infer_ep(x.to(dev), blk.experts, idx.to(dev), w.to(dev), k, async_op,
+                               skip_mask=mask, skip_now=now, cache_key=0).cpu()
+            assert rel_l2(got, want) < FP32_TOL, f"iteration {it}"
+    finally:
+        _reset(diep)
