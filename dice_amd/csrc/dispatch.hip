@@ -305,17 +305,28 @@ __global__ __launch_bounds__(kTileWaves *kWave) void dispatch_scan_rank_kernel(
     range_out[1] = range_n;
   }
   if (unit >= units) return;
-  // per expert: total over all units and total over the units before this one
+  // per expert: total over all units and total over the units before this one.
+  // The lanes read an expert's unit counts side by side (one coalesced load per
+  // 64 units) and reduce across the wave; lane e % 64 keeps expert e's sums.
   int carry = 0;  // running exclusive offset over experts
   for (int c = 0; c < n_experts; c += kWave) {
     const int e = c + lane;
     int tot = 0, before = 0;
-    if (e < n_experts) {
-      const int32_t *rowp = unit_cnt + (size_t)e * units;
-      for (int u = 0; u < units; ++u) {
-        const int v = rowp[u];
-        tot += v;
-        before += u < unit ? v : 0;
+    const int chunk_experts = n_experts - c < kWave ? n_experts - c : kWave;
+    for (int ee = 0; ee < chunk_experts; ++ee) {
+      const int32_t *rowp = unit_cnt + (size_t)(c + ee) * units;
+      int t = 0, b = 0;
+      for (int u0 = 0; u0 < units; u0 += kWave) {
+        const int u = u0 + lane;
+        const int v = u < units ? rowp[u] : 0;
+        t += v;
+        b += u < unit ? v : 0;
+      }
+      t = wave_sum_i32(t);
+      b = wave_sum_i32(b);
+      if (lane == ee) {
+        tot = t;
+        before = b;
       }
     }
     int inc = tot;
