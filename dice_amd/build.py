@@ -26,7 +26,9 @@ SOURCES = [
     "quant.hip",
     "grouped_gemm_f32.hip",
     "grouped_gemm_bf16.hip",
+    "grouped_gemm_f16.hip",
     "grouped_gemm_persist.hip",
+    "grouped_gemm_persist_f16.hip",
     "grouped_mlp.hip",
 ]
 

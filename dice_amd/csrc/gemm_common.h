@@ -146,7 +146,8 @@ struct PersistBatch {
 };
 bool persist_supported(const PersistBatch &b, int mode);
 bool gemm_config_wants_persistent();  // tuning hook state: both stages set to the persistent kernel
-int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s);
+int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s);      // bf16
+int launch_grouped_gemm_persist_f16(const PersistBatch &b, int mode, hipStream_t s);  // fp16
 
 // LayerNorm + adaLN modulation in front of the layer, and the combine with the
 // caller's residual / gate epilogue behind it (modulate.hip, combine.hip).
@@ -167,5 +168,6 @@ int gather_rows_impl(const void *x, int dtype, const int32_t *perm, int slots_pe
 int launch_grouped_gemm_f32(const GemmParams &p, int mode, int64_t max_rows, hipStream_t s);
 int launch_grouped_gemm_bf16(const GemmParams &p, int mode, int w_dtype, int64_t max_rows,
                              hipStream_t s);
+int launch_grouped_gemm_f16(const GemmParams &p, int mode, int w_dtype, int64_t max_rows, hipStream_t s);
 
 }  // namespace dice

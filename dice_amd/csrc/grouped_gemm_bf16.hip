@@ -25,10 +25,33 @@
 // fp8 (e4m3) weights are widened to bf16 while they are copied into LDS, so
 // the MFMA loop is unchanged; the per-output-channel scale is applied to the
 // fp32 accumulator in the epilogue.
+//
+// Compiled twice, like the persistent kernels: as it stands for bf16, and with
+// DICE_GEMM_F16 (through grouped_gemm_f16.hip) for fp16 activations and weights.
 #include "gemm_common.h"
+
+#ifndef DICE_GEMM_F16
+#define DICE_GEMM_F16 0
+#endif
 
 namespace dice {
 namespace {
+
+#if DICE_GEMM_F16
+typedef f16_t h16_t;
+typedef f16x8_t h16x8_t;
+typedef _Float16 h16x4_t __attribute__((ext_vector_type(4)));
+#define DICE_MFMA_32X32X16 __builtin_amdgcn_mfma_f32_32x32x16_f16
+#define DICE_WIDEN_FP8 __builtin_amdgcn_cvt_scalef32_pk_f16_fp8
+#define DICE_GEMM_LAUNCH launch_grouped_gemm_f16
+#else
+typedef bf16_t h16_t;
+typedef bf16x8_t h16x8_t;
+typedef bf16x4_t h16x4_t;
+#define DICE_MFMA_32X32X16 __builtin_amdgcn_mfma_f32_32x32x16_bf16
+#define DICE_WIDEN_FP8 __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8
+#define DICE_GEMM_LAUNCH launch_grouped_gemm_bf16
+#endif
 
 constexpr int kBK = 64;  // bf16 elements per k step = 128 bytes per LDS row
 
@@ -58,8 +81,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
   constexpr int A_STAGE = BM * kBK, B_STAGE = BN * kBK;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  bf16_t *As = reinterpret_cast<bf16_t *>(lds_raw);
-  bf16_t *Bs = As + 2 * A_STAGE;
+  h16_t *As = reinterpret_cast<h16_t *>(lds_raw);
+  h16_t *Bs = As + 2 * A_STAGE;
 
   const TileCoord t = locate_tile<BM, BN_OUT>(p);
   if (!t.active) return;
@@ -71,7 +94,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
 
   // ---- global -> register -> LDS copy assignment ----
   const int a_chunk = tid & 7, a_row0 = tid >> 3;
-  const bf16_t *a_base = (const bf16_t *)p.a;
+  const h16_t *a_base = (const h16_t *)p.a;
   uint32_t a_src[A_PASSES];
 #pragma unroll
   for (int i = 0; i < A_PASSES; ++i) {
@@ -103,15 +126,15 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
       for (int i = 0; i < B_PASSES; ++i)
         b_reg[i] = *reinterpret_cast<const u32x4_t *>(wb + b_src[i] + k0);
     } else {
-      const bf16_t *wb = (const bf16_t *)p.w + w_expert;
+      const h16_t *wb = (const h16_t *)p.w + w_expert;
 #pragma unroll
       for (int i = 0; i < B_PASSES; ++i)
         b_reg[i] = *reinterpret_cast<const u32x4_t *>(wb + b_src[i] + k0);
     }
   };
   auto store_lds = [&](int stage) {
-    bf16_t *as = As + stage * A_STAGE;
-    bf16_t *bs = Bs + stage * B_STAGE;
+    h16_t *as = As + stage * A_STAGE;
+    h16_t *bs = Bs + stage * B_STAGE;
 #pragma unroll
     for (int i = 0; i < A_PASSES; ++i) {
       const int rt = a_row0 + i * A_ROWS_PER_PASS;
@@ -125,12 +148,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
         u32x4_t lo, hi;
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
-          bf16x2_t c0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(b_reg[i][q], 1.0f, false);
-          bf16x2_t c1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(b_reg[i][q], 1.0f, true);
+          auto c0 = DICE_WIDEN_FP8(b_reg[i][q], 1.0f, false);
+          auto c1 = DICE_WIDEN_FP8(b_reg[i][q], 1.0f, true);
           lo[2 * q] = __builtin_bit_cast(uint32_t, c0);
           lo[2 * q + 1] = __builtin_bit_cast(uint32_t, c1);
-          bf16x2_t d0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(b_reg[i][q + 2], 1.0f, false);
-          bf16x2_t d1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(b_reg[i][q + 2], 1.0f, true);
+          auto d0 = DICE_WIDEN_FP8(b_reg[i][q + 2], 1.0f, false);
+          auto d1 = DICE_WIDEN_FP8(b_reg[i][q + 2], 1.0f, true);
           hi[2 * q] = __builtin_bit_cast(uint32_t, d0);
           hi[2 * q + 1] = __builtin_bit_cast(uint32_t, d1);
         }
@@ -168,30 +191,30 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
   for (int kt = 0; kt < kt_count; ++kt) {
     const int cur = kt & 1;
     if (kt + 1 < kt_count) load_global((kt + 1) * kBK);
-    const bf16_t *as = As + cur * A_STAGE;
-    const bf16_t *bs = Bs + cur * B_STAGE;
+    const h16_t *as = As + cur * A_STAGE;
+    const h16_t *bs = Bs + cur * B_STAGE;
 #pragma unroll
     for (int kk = 0; kk < kBK / 16; ++kk) {
       const int chunk = kk * 2 + frag_half;
-      bf16x8_t wf[TN], af[TM];
+      h16x8_t wf[TN], af[TM];
 #pragma unroll
       for (int j = 0; j < TN; ++j)
-        wf[j] = *reinterpret_cast<const bf16x8_t *>(bs + lds_off(w_block_row(j) + frag_row, chunk));
+        wf[j] = *reinterpret_cast<const h16x8_t *>(bs + lds_off(w_block_row(j) + frag_row, chunk));
 #pragma unroll
       for (int i = 0; i < TM; ++i)
-        af[i] = *reinterpret_cast<const bf16x8_t *>(as + lds_off(wm * WTM + i * 32 + frag_row, chunk));
+        af[i] = *reinterpret_cast<const h16x8_t *>(as + lds_off(wm * WTM + i * 32 + frag_row, chunk));
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[j], af[i], acc[i][j], 0, 0, 0);
+          acc[i][j] = DICE_MFMA_32X32X16(wf[j], af[i], acc[i][j], 0, 0, 0);
     }
     if (kt + 1 < kt_count) store_lds(cur ^ 1);
     __syncthreads();
   }
 
   // ---- epilogue: lane holds row (lane&31), columns 8*q + 4*(lane>>5) + {0..3} of each block ----
-  bf16_t *c = (bf16_t *)p.c;
+  h16_t *c = (h16_t *)p.c;
   const float *bias = p.bias ? p.bias + (size_t)t.expert * p.n : nullptr;
   const float *scale = p.w_scale ? p.w_scale + (size_t)t.expert * p.w_rows : nullptr;
   constexpr int OUT_BLOCKS = SWIGLU ? TN / 2 : TN;
@@ -201,7 +224,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
     if (m >= t.rows_valid) continue;
     const int gr = t.row_begin + m;
     const int64_t orow = p.c_perm ? p.c_perm[gr] : gr;
-    bf16_t *crow = c + orow * p.ldc;
+    h16_t *crow = c + orow * p.ldc;
 #pragma unroll
     for (int j = 0; j < OUT_BLOCKS; ++j) {
       const int nb = t.n0 + (SWIGLU ? wn * (WTN / 2) : wn * WTN) + j * 32 + frag_half * 4;
@@ -209,7 +232,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
       for (int q = 0; q < 4; ++q) {
         const int n = nb + q * 8;
         if (n >= p.n) continue;
-        bf16x4_t o;
+        h16x4_t o;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           float v = acc[i][j][q * 4 + r];
@@ -222,9 +245,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
             if (bias) v += bias[n + r];
             if (MODE == kFc1Gelu) v = gelu_tanh_fast(v);
           }
-          o[r] = (bf16_t)v;
+          o[r] = (h16_t)v;
         }
-        *reinterpret_cast<bf16x4_t *>(crow + n) = o;
+        *reinterpret_cast<h16x4_t *>(crow + n) = o;
       }
     }
   }
@@ -234,10 +257,10 @@ template <int BM, int BN, int WAVES_M, int WAVES_N, int MODE, bool W_FP8>
 int launch_cfg(const GemmParams &p, int64_t max_rows, hipStream_t s) {
   constexpr int BN_OUT = MODE == kFc1Swiglu ? BN / 2 : BN;
   constexpr int NT = WAVES_M * WAVES_N * kWave;
-  constexpr size_t lds = 2ull * (BM + BN) * kBK * sizeof(bf16_t);
+  constexpr size_t lds = 2ull * (BM + BN) * kBK * sizeof(h16_t);
   const int64_t grid = max_tiles(max_rows, p.n_experts, p.n, BM, BN_OUT);
   if (grid <= 0) return DICE_OK;
-  if (grid >= (1ll << 31)) return fail(DICE_ERR_UNSUPPORTED, "bf16 expert GEMM: grid too large");
+  if (grid >= (1ll << 31)) return fail(DICE_ERR_UNSUPPORTED, "16-bit expert GEMM: grid too large");
   auto kern = grouped_gemm_bf16_kernel<BM, BN, WAVES_M, WAVES_N, MODE, W_FP8>;
   if (lds > 48 * 1024) {
     static thread_local bool configured = false;
@@ -245,7 +268,7 @@ int launch_cfg(const GemmParams &p, int64_t max_rows, hipStream_t s) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
       if (e != hipSuccess)
-        return fail(DICE_ERR_LAUNCH, "bf16 expert GEMM: LDS attribute: %s", hipGetErrorString(e));
+        return fail(DICE_ERR_LAUNCH, "16-bit expert GEMM: LDS attribute: %s", hipGetErrorString(e));
       configured = true;
     }
   }
@@ -253,7 +276,15 @@ int launch_cfg(const GemmParams &p, int64_t max_rows, hipStream_t s) {
   return launch_status("grouped_gemm_bf16");
 }
 
+#if DICE_GEMM_F16
+}  // namespace
+extern int g_cfg_fc1, g_cfg_fc2;
+namespace {
+#else
+}  // namespace
 int g_cfg_fc1 = 0, g_cfg_fc2 = 0;
+namespace {
+#endif
 
 template <int MODE, bool W_FP8>
 int launch_mode(const GemmParams &p, int cfg, int64_t max_rows, hipStream_t s) {
@@ -269,10 +300,9 @@ int launch_mode(const GemmParams &p, int cfg, int64_t max_rows, hipStream_t s) {
 
 }  // namespace
 
-int launch_grouped_gemm_bf16(const GemmParams &p, int mode, int w_dtype, int64_t max_rows,
-                             hipStream_t s) {
-  if (p.k % kBK != 0) return fail(DICE_ERR_UNSUPPORTED, "bf16 expert GEMM: k %d %% %d != 0", p.k, kBK);
-  if (p.n % 8 != 0) return fail(DICE_ERR_UNSUPPORTED, "bf16 expert GEMM: n %d %% 8 != 0", p.n);
+int DICE_GEMM_LAUNCH(const GemmParams &p, int mode, int w_dtype, int64_t max_rows, hipStream_t s) {
+  if (p.k % kBK != 0) return fail(DICE_ERR_UNSUPPORTED, "16-bit expert GEMM: k %d %% %d != 0", p.k, kBK);
+  if (p.n % 8 != 0) return fail(DICE_ERR_UNSUPPORTED, "16-bit expert GEMM: n %d %% 8 != 0", p.n);
   const bool fp8 = w_dtype == DICE_FP8_E4M3;
   const int cfg = mode == kFc2 ? g_cfg_fc2 : g_cfg_fc1;
   switch (mode) {
@@ -290,6 +320,7 @@ int launch_grouped_gemm_bf16(const GemmParams &p, int mode, int w_dtype, int64_t
 
 }  // namespace dice
 
+#if !DICE_GEMM_F16
 namespace dice {
 constexpr int kCfgPersistent = 20;
 extern int g_persist_waves;
@@ -309,3 +340,4 @@ extern "C" int dice_set_gemm_config(int fc1_cfg, int fc2_cfg) {
   dice::g_persist_waves = fc1_cfg == dice::kCfgPersistent ? 8 : 4;
   return DICE_OK;
 }
+#endif  // !DICE_GEMM_F16

@@ -33,12 +33,48 @@
 // scale per output channel (64-k pipeline only: widened to bf16 on the way into
 // LDS, scale applied to the fp32 sums); activations are grouped rows
 // (contiguous, or rows of the token matrix named by a row table).
+//
+// This file is compiled twice: as it stands for bf16 activations and weights,
+// and with DICE_PERSIST_F16 (through grouped_gemm_persist_f16.hip) for fp16,
+// which the reference serves its XL and G models in (sample_ddp.py:77-81,97-98).
+// Only the element type of the operands, the MFMA instruction and the fp8
+// widening differ; shared host-side helpers live in the bf16 compilation.
 #include <type_traits>
 
 #include "gemm_common.h"
 
+#ifndef DICE_PERSIST_F16
+#define DICE_PERSIST_F16 0
+#endif
+
 namespace dice {
 namespace {
+
+#if DICE_PERSIST_F16
+typedef f16_t h16_t;
+typedef f16x8_t h16x8_t;
+typedef _Float16 h16x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ f32x16_t mfma_32x32x16(h16x8_t a, h16x8_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+// two fp8 (e4m3) bytes of `src` (the low or the high pair) -> two fp16, exactly
+__device__ __forceinline__ uint32_t widen_fp8_pair(uint32_t src, bool high) {
+  return __builtin_bit_cast(uint32_t, high ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(src, 1.0f, true)
+                                           : __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(src, 1.0f, false));
+}
+#else
+typedef bf16_t h16_t;
+typedef bf16x8_t h16x8_t;
+typedef bf16x4_t h16x4_t;
+__device__ __forceinline__ f32x16_t mfma_32x32x16(h16x8_t a, h16x8_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+// two fp8 (e4m3) bytes of `src` (the low or the high pair) -> two bf16, exactly
+__device__ __forceinline__ uint32_t widen_fp8_pair(uint32_t src, bool high) {
+  return __builtin_bit_cast(uint32_t, high ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(src, 1.0f, true)
+                                           : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(src, 1.0f, false));
+}
+#endif
 
 constexpr int kPBM = 256, kPBN = 256, kPBK = 32;
 constexpr int kPWavesM = 2;
@@ -439,13 +475,13 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int col = j * 32 + frag_half * 4 + q * 8;
-          bf16x4_t o;
+          h16x4_t o;
           DICE_EPI_SCALES(j, q)
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             float v = blk[q * 4 + r];
             DICE_EPI_VALUE(v, j, q, r);
-            o[r] = (bf16_t)v;
+            o[r] = (h16_t)v;
           }
           *reinterpret_cast<u32x2_any_t *>(stage + frag_row * PITCH + col * 2) = __builtin_bit_cast(u32x2_t, o);
         }
@@ -455,7 +491,7 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
       // The staging rows hold 16 rows at a time.  The activation of the whole
       // 32-row block is worked out once, with every lane at work (per band only
       // half the lanes own rows), and kept packed while its two bands go out.
-      bf16x4_t packed[OUT_BLOCKS][4];
+      h16x4_t packed[OUT_BLOCKS][4];
 #pragma unroll
       for (int j = 0; j < OUT_BLOCKS; ++j) {
         const f32x16_t blk = acc_block<WAVES == 4>(acc[i][j]);
@@ -468,7 +504,7 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
           for (int r = 0; r < 4; ++r) {
             float v = blk[q * 4 + r];
             DICE_EPI_VALUE(v, j, q, r);
-            packed[j][q][r] = (bf16_t)v;
+            packed[j][q][r] = (h16_t)v;
           }
         }
       }
@@ -582,7 +618,7 @@ __device__ __forceinline__ void gemm_persist_body(const PersistBatch &batch) {
     return wn * WTN + j * 32;
   };
   const int frag_row = lane & 31, frag_half = lane >> 5;
-  bf16x8_t wf[2][TN], af[2][TM];
+  h16x8_t wf[2][TN], af[2][TM];
   // Lane part of the fragment addresses for the two 16-k halves of a step; the
   // 32-row block and the ring slot only add compile-time constants (the swizzle
   // uses row bits 1..3, which block offsets do not touch), so the reads of a
@@ -601,11 +637,11 @@ __device__ __forceinline__ void gemm_persist_body(const PersistBatch &batch) {
     for (int j = 0; j < TN; ++j) {
       constexpr int HALF = TN / 2;
       const int joff = (SWIGLU && j >= HALF) ? (kPBN / 2 + (j - HALF) * 32) * 64 : j * 32 * 64;
-      wf[buf][j] = *reinterpret_cast<const bf16x8_t *>(base + rd_b[kk] + joff);
+      wf[buf][j] = *reinterpret_cast<const h16x8_t *>(base + rd_b[kk] + joff);
     }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
-      af[buf][i] = *reinterpret_cast<const bf16x8_t *>(base + rd_a[kk] + i * 32 * 64);
+      af[buf][i] = *reinterpret_cast<const h16x8_t *>(base + rd_a[kk] + i * 32 * 64);
   };
 
   f32x16_t acc[TM][TN];
@@ -705,7 +741,7 @@ __device__ __forceinline__ void gemm_persist_body(const PersistBatch &batch) {
           for (int i = 0; i < TM; ++i)
   #pragma unroll
             for (int j = 0; j < TN; ++j)
-              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[kk][j], af[kk][i], acc[i][j], 0, 0, 0);
+              acc[i][j] = mfma_32x32x16(wf[kk][j], af[kk][i], acc[i][j]);
         __builtin_amdgcn_s_setprio(DICE_PRIO_MEMORY);
         if (group == 0) copies_landed();
         phase_barrier();
@@ -957,7 +993,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
     rd_b[kk] = kPBM * 128 + qring_off(b_row0 + frag_row, kk * 2 + frag_half);
     asm volatile("" : "+v"(rd_a[kk]), "+v"(rd_b[kk]));
   }
-  bf16x8_t wf[2][TN], af[2][TM];
+  h16x8_t wf[2][TN], af[2][TM];
   auto read_frags = [&](auto slot_c, auto kk_c, int buf) {
     constexpr int SLOT = decltype(slot_c)::value, KK = decltype(kk_c)::value;
     const unsigned char *base = SLOT == 0 ? lds_slot0 : lds_slot1;
@@ -965,11 +1001,11 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
     for (int j = 0; j < TN; ++j) {
       constexpr int HALF = TN / 2;
       const int jrow = (SWIGLU && j >= HALF) ? BN / 2 + (j - HALF) * 32 : j * 32;
-      wf[buf][j] = *reinterpret_cast<const bf16x8_t *>(base + rd_b[KK] + jrow * 128);
+      wf[buf][j] = *reinterpret_cast<const h16x8_t *>(base + rd_b[KK] + jrow * 128);
     }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
-      af[buf][i] = *reinterpret_cast<const bf16x8_t *>(base + rd_a[KK] + i * 32 * 128);
+      af[buf][i] = *reinterpret_cast<const h16x8_t *>(base + rd_a[KK] + i * 32 * 128);
   };
 
   const int wave_col0 = SWIGLU ? wn * (WTN / 2) : wn * WTN;
@@ -1013,7 +1049,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[buf][j], af[buf][i], acc[i][j], 0, 0, 0);
+        acc[i][j] = mfma_32x32x16(wf[buf][j], af[buf][i], acc[i][j]);
   };
 
   // ---- pipeline state ----
@@ -1092,10 +1128,10 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
         u32x4_t lo, hi;
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
-          lo[2 * q] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(src[q], 1.0f, false));
-          lo[2 * q + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(src[q], 1.0f, true));
-          hi[2 * q] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(src[q + 2], 1.0f, false));
-          hi[2 * q + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(src[q + 2], 1.0f, true));
+          lo[2 * q] = widen_fp8_pair(src[q], false);
+          lo[2 * q + 1] = widen_fp8_pair(src[q], true);
+          hi[2 * q] = widen_fp8_pair(src[q + 2], false);
+          hi[2 * q + 1] = widen_fp8_pair(src[q + 2], true);
         }
         *reinterpret_cast<u32x4_any_t *>(row + wr_off_b8) = lo;
         *reinterpret_cast<u32x4_any_t *>(row + wr_off_b8_hi) = hi;
@@ -1210,6 +1246,16 @@ __global__ __launch_bounds__(4 * kWave, 1) void gemm_persist_kernel4(PersistBatc
 
 }  // namespace
 
+#if DICE_PERSIST_F16
+extern int g_persist_waves;
+int persist_variant(const PersistBatch &b, int mode);
+int persist_cu_count();
+#define DICE_PERSIST_LAUNCH launch_grouped_gemm_persist_f16
+namespace {
+int cu_count() { return persist_cu_count(); }
+}  // namespace
+#else
+#define DICE_PERSIST_LAUNCH launch_grouped_gemm_persist
 int g_persist_waves = 4;  // tuning hook: 4 = 64-k register-staged pipeline first, 8 = 32-k ping-pong pipeline only
 
 namespace {
@@ -1268,6 +1314,9 @@ bool persist64_ok(const PersistBatch &b, int mode) {
 }
 
 // 0: neither pipeline applies; 4: the 64-k four-wave kernel; 8: the 32-k eight-wave kernel.
+}  // namespace
+int persist_cu_count() { return cu_count(); }
+// 0: neither pipeline takes the launch; 4 / 8: the waves of the one that does.
 int persist_variant(const PersistBatch &b, int mode) {
   if (!persist_common_ok(b, mode)) return 0;
   if (g_persist_waves == 4 && persist64_ok(b, mode)) return 4;
@@ -1276,11 +1325,10 @@ int persist_variant(const PersistBatch &b, int mode) {
   return 8;
 }
 
-}  // namespace
-
 bool persist_supported(const PersistBatch &b, int mode) { return persist_variant(b, mode) != 0; }
+#endif  // !DICE_PERSIST_F16
 
-int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s) {
+int DICE_PERSIST_LAUNCH(const PersistBatch &b, int mode, hipStream_t s) {
   const int waves = persist_variant(b, mode);
   if (waves == 0) return fail(DICE_ERR_UNSUPPORTED, "persistent expert GEMM: unsupported shape");
   const int grid = cu_count() / kNumXcd * kNumXcd;

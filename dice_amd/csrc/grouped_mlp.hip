@@ -7,7 +7,15 @@ namespace {
 int run_gemm(const GemmParams &p, int mode, int act_dtype, int w_dtype, int64_t max_rows,
              hipStream_t s) {
   if (act_dtype == DICE_F32) return launch_grouped_gemm_f32(p, mode, max_rows, s);
+  if (act_dtype == DICE_F16) return launch_grouped_gemm_f16(p, mode, w_dtype, max_rows, s);
   return launch_grouped_gemm_bf16(p, mode, w_dtype, max_rows, s);
+}
+
+bool is_16bit(int dtype) { return dtype == DICE_BF16 || dtype == DICE_F16; }
+
+int launch_persist(const PersistBatch &b, int mode, int act_dtype, hipStream_t s) {
+  return act_dtype == DICE_F16 ? launch_grouped_gemm_persist_f16(b, mode, s)
+                               : launch_grouped_gemm_persist(b, mode, s);
 }
 
 struct Carve {
@@ -93,9 +101,9 @@ void stamp(int i, hipStream_t s) {
 
 int check_mlp_shape(const char *who, int act_dtype, int w_dtype, int act_variant, int hidden,
                     int inter, int n_experts) {
-  DICE_REQUIRE(act_dtype == DICE_BF16 || act_dtype == DICE_F32, DICE_ERR_UNSUPPORTED,
-               "%s: act_dtype %d (BF16 or F32)", who, act_dtype);
-  DICE_REQUIRE(w_dtype == act_dtype || (w_dtype == DICE_FP8_E4M3 && act_dtype == DICE_BF16),
+  DICE_REQUIRE(is_16bit(act_dtype) || act_dtype == DICE_F32, DICE_ERR_UNSUPPORTED,
+               "%s: act_dtype %d (BF16, F16 or F32)", who, act_dtype);
+  DICE_REQUIRE(w_dtype == act_dtype || (w_dtype == DICE_FP8_E4M3 && is_16bit(act_dtype)),
                DICE_ERR_UNSUPPORTED, "%s: w_dtype %d with act_dtype %d", who, w_dtype, act_dtype);
   DICE_REQUIRE(act_variant == DICE_ACT_SWIGLU || act_variant == DICE_ACT_GELU_TANH,
                DICE_ERR_BAD_ARG, "%s: act_variant %d", who, act_variant);
@@ -134,8 +142,7 @@ int grouped_mlp_impl(int stages, const void *x, int act_dtype, const int32_t *pe
   const bool swiglu = act_variant == DICE_ACT_SWIGLU;
 
   // Contiguous grouped rows + bf16 weights: the persistent kernel applies.
-  if (!perm && act_dtype == DICE_BF16 && (w_dtype == DICE_BF16 || w_dtype == DICE_FP8_E4M3) &&
-      gemm_config_wants_persistent()) {
+  if (!perm && is_16bit(act_dtype) && gemm_config_wants_persistent()) {
     PersistBatch pb1{};
     pb1.n_problems = 1;
     pb1.prob[0] = PersistProblem{x, hidden, offsets, n_experts, w1, swiglu ? 2 * inter : inter, inter,
@@ -151,10 +158,10 @@ int grouped_mlp_impl(int stages, const void *x, int act_dtype, const int32_t *pe
     const int m1 = swiglu ? kFc1Swiglu : kFc1Gelu;
     if (persist_supported(pb1, m1) && persist_supported(pb2, kFc2)) {
       if (stages & 1) {
-        rc = launch_grouped_gemm_persist(pb1, m1, s);
+        rc = launch_persist(pb1, m1, act_dtype, s);
         if (rc) return rc;
       }
-      if (stages & 2) return launch_grouped_gemm_persist(pb2, kFc2, s);
+      if (stages & 2) return launch_persist(pb2, kFc2, act_dtype, s);
       return DICE_OK;
     }
   }
@@ -356,7 +363,7 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
   // (bf16) gets launches of its own.
   bool done = false;
   const bool w8 = LE->w_dtype == DICE_FP8_E4M3;
-  if (L->act_dtype == DICE_BF16 && (LE->w_dtype == DICE_BF16 || (w8 && LE->w1_scale && LE->w2_scale))) {
+  if (is_16bit(L->act_dtype) && (LE->w_dtype == L->act_dtype || (w8 && LE->w1_scale && LE->w2_scale))) {
     const bool swiglu = L->act_variant == DICE_ACT_SWIGLU;
     const int m1 = swiglu ? kFc1Swiglu : kFc1Gelu;
     PersistBatch f1{}, f2{};
@@ -408,17 +415,17 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
         if (rc) return rc;
       }
       stamp(3, s);
-      rc = launch_grouped_gemm_persist(f1, m1, s);
+      rc = launch_persist(f1, m1, L->act_dtype, s);
       if (rc) return rc;
       if (s1.n_problems) {
-        rc = launch_grouped_gemm_persist(s1, m1, s);
+        rc = launch_persist(s1, m1, L->act_dtype, s);
         if (rc) return rc;
       }
       stamp(4, s);
-      rc = launch_grouped_gemm_persist(f2, kFc2, s);
+      rc = launch_persist(f2, kFc2, L->act_dtype, s);
       if (rc) return rc;
       if (s2.n_problems) {
-        rc = launch_grouped_gemm_persist(s2, kFc2, s);
+        rc = launch_persist(s2, kFc2, L->act_dtype, s);
         if (rc) return rc;
       }
       stamp(5, s);

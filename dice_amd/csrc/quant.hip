@@ -54,6 +54,9 @@ extern "C" int dice_quantize_fp8_rowwise(const void *w, int in_dtype, int64_t ro
   if (in_dtype == DICE_BF16) {
     hipLaunchKernelGGL(quantize_rows_kernel<bf16_t>, dim3((unsigned)rows), dim3(256), 0, s,
                        (const bf16_t *)w, cols, q, scale);
+  } else if (in_dtype == DICE_F16) {
+    hipLaunchKernelGGL(quantize_rows_kernel<f16_t>, dim3((unsigned)rows), dim3(256), 0, s,
+                       (const f16_t *)w, cols, q, scale);
   } else if (in_dtype == DICE_F32) {
     hipLaunchKernelGGL(quantize_rows_kernel<float>, dim3((unsigned)rows), dim3(256), 0, s,
                        (const float *)w, cols, q, scale);

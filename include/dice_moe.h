@@ -105,7 +105,8 @@ int dice_gather_rows(const void *x, int dtype, const int32_t *perm,
  * MoeMLP.forward (models.py:252-273) as the expert, in two grouped GEMMs:
  *   fc1: h[r] = act(A[r] W1[e]^T)     fc2: out[dst(r)] = h[r] W2[e]^T
  * for grouped rows r in [offsets[e], offsets[e+1]).
- *   x        [n_tokens, hidden] activations (act_dtype in {BF16, F32})
+ *   x        [n_tokens, hidden] activations (act_dtype in {BF16, F16, F32}; weights
+ *            in the same type, or FP8_E4M3 with 16-bit activations)
  *   perm     [>= max_rows] int32 grouped row -> slot, or NULL (row r = token r)
  *   slots_per_token  divisor turning a slot into its token row of x
  *   offsets  [n_experts+1] int32 (device)
@@ -173,7 +174,7 @@ int dice_combine(const void *slot_out, const int32_t *inv_perm,
  * Per-output-channel fp8 quantiser for expert weights (build-defined, the
  * reference has no fp8 path): scale[r] = amax(|w[r,:]|)/448 (1 if the row is
  * all zero), q[r,c] = e4m3fn(rne(w[r,c]/scale[r])).
- *   w [rows, cols] in_dtype in {BF16, F32};  q [rows, cols] uint8;  scale [rows]
+ *   w [rows, cols] in_dtype in {BF16, F16, F32};  q [rows, cols] uint8;  scale [rows]
  */
 int dice_quantize_fp8_rowwise(const void *w, int in_dtype, int64_t rows,
                               int64_t cols, uint8_t *q, float *scale,
@@ -188,7 +189,7 @@ int dice_quantize_fp8_rowwise(const void *w, int in_dtype, int64_t rows,
  */
 typedef struct dice_moe_layer {
   int32_t hidden, inter, n_experts, top_k;
-  int32_t act_dtype;      /* DICE_BF16 or DICE_F32 */
+  int32_t act_dtype;      /* DICE_BF16, DICE_F16 or DICE_F32 */
   int32_t w_dtype;        /* act_dtype, or DICE_FP8_E4M3 for routed experts */
   int32_t act_variant;    /* DICE_ACT_* */
   int32_t norm_topk_prob; /* models.py:170: 0 in the reference */

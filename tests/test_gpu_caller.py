@@ -178,3 +178,21 @@ def test_block_half_lagged_writes_entry_in_place(dev):
         diep.use_latest_expert_weights(False)
         if diep.diep_forced_sync():
             diep.diep_cancel_sync()
+
+
+def test_block_half_f16(dev):
+    """The fused caller in fp16 (model.half() in the reference) at XL width."""
+    B, T, D = 4, 256, 1152
+    p = O.make_block_params(D, 8, 2, 4, 2, seed=2, dtype=torch.float16)
+    x, shift, scale, gate = _inputs(B, T, D, torch.float16, 15)
+    blk = block_from_params(p, D, "swiglu", torch.float16, dev)
+    got = blk.forward_modulated(x.to(dev), shift.to(dev), scale.to(dev), gate.to(dev)).cpu()
+    want, h, widx, _, logits = O.dit_block_moe_half(p, x, shift, scale, gate, single_rounding=True)
+    from dice_amd import ops
+    hd = ops.ln_modulate(x.to(dev), shift.to(dev), scale.to(dev))
+    gidx = torch.empty(B * T, 2, dtype=torch.int32, device=dev)
+    blk.run(hd.view(-1, D), topk_idx_out=gidx)
+    moved = (gidx.cpu().long() != widx).any(-1)
+    assert moved.float().mean() < 0.01
+    ok = ~moved.view(B, T)
+    assert rel_l2(got[ok], want[ok]) < 4e-3

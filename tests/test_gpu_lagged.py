@@ -232,3 +232,9 @@ def test_moe_infer_ep_function_follows_oracle(dev, async_op, skip):
             assert rel_l2(got, want) < FP32_TOL, f"iteration {it}"
     finally:
         _reset(diep)
+
+
+def test_displaced_f16_persistent_path(dev):
+    """fp16, the dtype the reference serves its XL model in."""
+    _drive(dev, torch.float16, L=2, strategy="all", pipeline=False, latest=True, steps=4, D=1152, N=1024,
+           tol=4e-3)
