@@ -282,6 +282,18 @@ class SparseMoeBlock(nn.Module):
         made contiguous here).  ``out`` may be ``x`` itself."""
         if x.dim() != 3 or shift.shape != (x.shape[0], x.shape[2]):
             raise DiceError("forward_modulated needs x [B, T, D] and shift / scale / gate [B, D]")
+        wdt = self.gate.weight.dtype
+        if x.dtype != wdt:
+            # A residual stream kept in another precision than the layer (fp32 stream, half
+            # model under autocast): prologue in the stream's type, layer in its own, epilogue
+            # as torch ops in the stream's type.
+            h = ops.ln_modulate(x, shift.to(x.dtype), scale.to(x.dtype), eps)
+            y = self._forward(h, None).to(x.dtype)
+            res = x + gate.to(x.dtype).unsqueeze(1) * y
+            if out is not None:
+                out.copy_(res)
+                return out
+            return res
         c = CallerDesc()
         keep = [t.to(x.dtype).contiguous() for t in (shift, scale, gate)]
         c.shift, c.scale, c.gate = (ptr(t) for t in keep)
@@ -294,6 +306,16 @@ class SparseMoeBlock(nn.Module):
             raise DiceError("SparseMoeBlock: only the inference branch is implemented (call .eval())")
         orig_shape = hidden_states.shape
         x = hidden_states.reshape(-1, orig_shape[-1]).contiguous()
+        wdt = self.gate.weight.dtype
+        if x.dtype != wdt:
+            # Under autocast the reference's linear layers take their inputs in the module's
+            # half type whatever the caller's tensors are (sample_ddp.py:228); without it a
+            # mismatch is an error there too.
+            if not torch.is_autocast_enabled():
+                raise DiceError(f"activations are {x.dtype} but the block's parameters {wdt} "
+                                "(cast one of them, or run under torch.autocast)")
+            x = x.to(wdt)
+            hidden_states = hidden_states.to(wdt)
         if x.shape[0] == 0:  # no tokens: nothing to route, nothing to cache
             return out if out is not None else torch.empty_like(hidden_states)
         y = None if out is None else out.view(-1, orig_shape[-1])

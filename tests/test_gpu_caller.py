@@ -196,3 +196,29 @@ def test_block_half_f16(dev):
     assert moved.float().mean() < 0.01
     ok = ~moved.view(B, T)
     assert rel_l2(got[ok], want[ok]) < 4e-3
+
+
+def test_half_model_under_autocast_with_fp32_stream(dev):
+    """The reference's serving set-up for XL / G (sample_ddp.py:97-98,228): the
+    model in fp16, activations arriving in fp32 under torch.autocast.  The
+    block casts like autocast's linear layers do and answers in fp16; the fused
+    caller keeps an fp32 residual stream in fp32."""
+    from dice_amd import DiceError
+    B, T, D = 2, 128, 1152
+    p = O.make_block_params(D, 8, 2, 4, 2, seed=4, dtype=torch.float16)
+    blk = block_from_params(p, D, "swiglu", torch.float16, dev)
+    x, shift, scale, gate = _inputs(B, T, D, torch.float32, 17)
+    with pytest.raises(DiceError, match="autocast"):
+        blk(x.to(dev))
+    with torch.autocast(device_type="cuda", dtype=torch.float16):
+        y = blk(x.to(dev))
+        out = blk.forward_modulated(x.to(dev), shift.to(dev), scale.to(dev), gate.to(dev))
+    assert y.dtype == torch.float16 and out.dtype == torch.float32
+    want_y, _, _, logits = O.sparse_moe_block_forward(p, x.half())
+    ok = ~O.gate_tie_rows(logits, 2).view(B, T)
+    assert rel_l2(y.cpu()[ok], want_y[ok]) < 4e-3
+    h = O.norm_modulate(x, shift, scale)
+    wy, _, _, logits2 = O.sparse_moe_block_forward(p, h.half())
+    want = x + gate.unsqueeze(1) * wy.float()
+    ok2 = ~O.gate_tie_rows(logits2, 2, tol=1e-3).view(B, T)
+    assert rel_l2(out.cpu()[ok2], want[ok2]) < 4e-3
