@@ -165,9 +165,9 @@ int gather_rows_impl(const void *x, int dtype, const int32_t *perm, int slots_pe
                      int64_t n_rows, int hidden, void *out, int32_t *range_out, int32_t range_n,
                      void *stream);
 
-int launch_grouped_gemm_f32(const GemmParams &p, int mode, int64_t max_rows, hipStream_t s);
 int launch_grouped_gemm_bf16(const GemmParams &p, int mode, int w_dtype, int64_t max_rows,
                              hipStream_t s);
 int launch_grouped_gemm_f16(const GemmParams &p, int mode, int w_dtype, int64_t max_rows, hipStream_t s);
+int launch_grouped_gemm_f32(const GemmParams &p, int mode, int w_dtype, int64_t max_rows, hipStream_t s);
 
 }  // namespace dice

@@ -33,11 +33,22 @@
 #ifndef DICE_GEMM_F16
 #define DICE_GEMM_F16 0
 #endif
+// ... and with DICE_GEMM_F32 (through grouped_gemm_f32.hip) for fp32
+// activations and weights, the type the reference serves its S and B models in
+// (sample_ddp.py:82-85): 32 k per step (still 128-byte LDS rows), the fp32
+// MFMA v_mfma_f32_32x32x2_f32 (fp32 products and sums), no fp8 weights.
+#ifndef DICE_GEMM_F32
+#define DICE_GEMM_F32 0
+#endif
 
 namespace dice {
 namespace {
 
-#if DICE_GEMM_F16
+#if DICE_GEMM_F32
+typedef float h16_t;
+typedef f32x4_t h16x4_t;
+#define DICE_GEMM_LAUNCH launch_grouped_gemm_f32
+#elif DICE_GEMM_F16
 typedef f16_t h16_t;
 typedef f16x8_t h16x8_t;
 typedef _Float16 h16x4_t __attribute__((ext_vector_type(4)));
@@ -53,13 +64,14 @@ typedef bf16x4_t h16x4_t;
 #define DICE_GEMM_LAUNCH launch_grouped_gemm_bf16
 #endif
 
-constexpr int kBK = 64;  // bf16 elements per k step = 128 bytes per LDS row
+constexpr int kChunkElems = 16 / (int)sizeof(h16_t);  // elements per 16-byte chunk
+constexpr int kBK = 8 * kChunkElems;                  // elements per k step = 128 bytes per LDS row
 
 __device__ __forceinline__ int swizzle(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
-// Element offset of 16-byte chunk `chunk` of row `row` inside a [rows][64] tile.
+// Element offset of 16-byte chunk `chunk` of row `row` inside a [rows][kBK] tile.
 __device__ __forceinline__ int lds_off(int row, int chunk) {
-  return row * kBK + ((chunk ^ swizzle(row)) << 3);
+  return row * kBK + ((chunk ^ swizzle(row)) * kChunkElems);
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int MODE, bool W_FP8>
@@ -71,6 +83,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
   constexpr int TM = WTM / 32, TN = WTN / 32;
   static_assert(TM >= 1 && TN >= 1, "wave tile must hold at least one 32x32 block");
   static_assert(!SWIGLU || TN % 2 == 0, "SwiGLU needs gate and up blocks in the same wave");
+  static_assert(!(DICE_GEMM_F32 && W_FP8), "fp8 weights go with 16-bit activations");
   constexpr int A_ROWS_PER_PASS = NT / 8;
   constexpr int A_PASSES = BM / A_ROWS_PER_PASS;
   // bf16 weights: 8 threads x 16 B per row; fp8: 4 threads x 16 B per row.
@@ -101,7 +114,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
     const int rt = a_row0 + i * A_ROWS_PER_PASS;
     const int gr = t.row_begin + (rt < t.rows_valid ? rt : t.rows_valid - 1);
     const int src = p.a_perm ? p.a_perm[gr] / p.a_div : gr;
-    a_src[i] = (uint32_t)src * (uint32_t)p.lda + a_chunk * 8;
+    a_src[i] = (uint32_t)src * (uint32_t)p.lda + a_chunk * kChunkElems;
   }
   const int b_chunk = tid % B_THREADS_PER_ROW, b_row0 = tid / B_THREADS_PER_ROW;
   const size_t w_expert = (size_t)t.expert * p.w_rows * p.k;
@@ -112,7 +125,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
     int col = t.n0 + (SWIGLU ? (rt % (BN / 2)) : rt);
     if (col >= p.n) col = t.n0;
     const int wrow = (SWIGLU && rt >= BN / 2) ? p.up_offset + col : col;
-    b_src[i] = (uint32_t)wrow * (uint32_t)p.k + b_chunk * (W_FP8 ? 16 : 8);
+    b_src[i] = (uint32_t)wrow * (uint32_t)p.k + b_chunk * (W_FP8 ? 16 : kChunkElems);
   }
 
   u32x4_t a_reg[A_PASSES], b_reg[B_PASSES];
@@ -143,6 +156,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
 #pragma unroll
     for (int i = 0; i < B_PASSES; ++i) {
       const int rt = b_row0 + i * B_ROWS_PER_PASS;
+#if !DICE_GEMM_F32
       if (W_FP8) {
         // 16 e4m3 bytes -> 16 bf16 = chunks 2c and 2c+1 of the row.
         u32x4_t lo, hi;
@@ -159,7 +173,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
         }
         *reinterpret_cast<u32x4_t *>(bs + lds_off(rt, 2 * b_chunk)) = lo;
         *reinterpret_cast<u32x4_t *>(bs + lds_off(rt, 2 * b_chunk + 1)) = hi;
-      } else {
+      } else
+#endif
+      {
         *reinterpret_cast<u32x4_t *>(bs + lds_off(rt, b_chunk)) = b_reg[i];
       }
     }
@@ -193,6 +209,29 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
     if (kt + 1 < kt_count) load_global((kt + 1) * kBK);
     const h16_t *as = As + cur * A_STAGE;
     const h16_t *bs = Bs + cur * B_STAGE;
+#if DICE_GEMM_F32
+    // v_mfma_f32_32x32x2_f32 takes one k per half-wave: lanes 0..31 supply k = c,
+    // lanes 32..63 k = 16 + c of the step's 32, for c = 0..15 (any pairing of the
+    // k values is a valid order of the sum as long as both operands use it).
+#pragma unroll
+    for (int cc = 0; cc < 4; ++cc) {
+      const int chunk = frag_half * 4 + cc;
+      f32x4_t wf[TN], af[TM];
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        wf[j] = *reinterpret_cast<const f32x4_t *>(bs + lds_off(w_block_row(j) + frag_row, chunk));
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        af[i] = *reinterpret_cast<const f32x4_t *>(as + lds_off(wm * WTM + i * 32 + frag_row, chunk));
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(wf[j][e], af[i][e], acc[i][j], 0, 0, 0);
+    }
+#else
 #pragma unroll
     for (int kk = 0; kk < kBK / 16; ++kk) {
       const int chunk = kk * 2 + frag_half;
@@ -209,6 +248,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
         for (int j = 0; j < TN; ++j)
           acc[i][j] = DICE_MFMA_32X32X16(wf[j], af[i], acc[i][j], 0, 0, 0);
     }
+#endif
     if (kt + 1 < kt_count) store_lds(cur ^ 1);
     __syncthreads();
   }
@@ -276,7 +316,7 @@ int launch_cfg(const GemmParams &p, int64_t max_rows, hipStream_t s) {
   return launch_status("grouped_gemm_bf16");
 }
 
-#if DICE_GEMM_F16
+#if DICE_GEMM_F16 || DICE_GEMM_F32
 }  // namespace
 extern int g_cfg_fc1, g_cfg_fc2;
 namespace {
@@ -303,8 +343,16 @@ int launch_mode(const GemmParams &p, int cfg, int64_t max_rows, hipStream_t s) {
 int DICE_GEMM_LAUNCH(const GemmParams &p, int mode, int w_dtype, int64_t max_rows, hipStream_t s) {
   if (p.k % kBK != 0) return fail(DICE_ERR_UNSUPPORTED, "16-bit expert GEMM: k %d %% %d != 0", p.k, kBK);
   if (p.n % 8 != 0) return fail(DICE_ERR_UNSUPPORTED, "16-bit expert GEMM: n %d %% 8 != 0", p.n);
-  const bool fp8 = w_dtype == DICE_FP8_E4M3;
   const int cfg = mode == kFc2 ? g_cfg_fc2 : g_cfg_fc1;
+#if DICE_GEMM_F32
+  if (w_dtype != DICE_F32) return fail(DICE_ERR_UNSUPPORTED, "fp32 expert GEMM: w_dtype %d", w_dtype);
+  switch (mode) {
+    case kFc1Swiglu: return launch_mode<kFc1Swiglu, false>(p, cfg, max_rows, s);
+    case kFc1Gelu: return launch_mode<kFc1Gelu, false>(p, cfg, max_rows, s);
+    default: return launch_mode<kFc2, false>(p, cfg, max_rows, s);
+  }
+#else
+  const bool fp8 = w_dtype == DICE_FP8_E4M3;
   switch (mode) {
     case kFc1Swiglu:
       return fp8 ? launch_mode<kFc1Swiglu, true>(p, cfg, max_rows, s)
@@ -316,11 +364,12 @@ int DICE_GEMM_LAUNCH(const GemmParams &p, int mode, int w_dtype, int64_t max_row
       return fp8 ? launch_mode<kFc2, true>(p, cfg, max_rows, s)
                  : launch_mode<kFc2, false>(p, cfg, max_rows, s);
   }
+#endif
 }
 
 }  // namespace dice
 
-#if !DICE_GEMM_F16
+#if !DICE_GEMM_F16 && !DICE_GEMM_F32
 namespace dice {
 constexpr int kCfgPersistent = 20;
 extern int g_persist_waves;
@@ -340,4 +389,4 @@ extern "C" int dice_set_gemm_config(int fc1_cfg, int fc2_cfg) {
   dice::g_persist_waves = fc1_cfg == dice::kCfgPersistent ? 8 : 4;
   return DICE_OK;
 }
-#endif  // !DICE_GEMM_F16
+#endif  // bf16 compilation only

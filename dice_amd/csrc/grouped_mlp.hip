@@ -6,7 +6,7 @@ namespace {
 
 int run_gemm(const GemmParams &p, int mode, int act_dtype, int w_dtype, int64_t max_rows,
              hipStream_t s) {
-  if (act_dtype == DICE_F32) return launch_grouped_gemm_f32(p, mode, max_rows, s);
+  if (act_dtype == DICE_F32) return launch_grouped_gemm_f32(p, mode, w_dtype, max_rows, s);
   if (act_dtype == DICE_F16) return launch_grouped_gemm_f16(p, mode, w_dtype, max_rows, s);
   return launch_grouped_gemm_bf16(p, mode, w_dtype, max_rows, s);
 }
