@@ -172,6 +172,30 @@ __device__ __forceinline__ Tile unpack_tile(const PackedTile &pk) {
 // then n-tile with the m-tile fastest; callers list the problem with the longest
 // k first.  XCD x (= blockIdx.x % 8) owns the x-th eighth of that order and its
 // workgroups take tiles of the run in turns.
+// Position of tile `r` inside one (problem, expert) group of mt x nt tiles.
+// The m-tile runs fastest, so that the workgroups of an XCD that work side by
+// side share weight tiles; a group with many m-tiles (large batches) is cut
+// into bands of about eight m-tiles, each taken through all n-tiles before the
+// next, or a round of 32 workgroups would touch 32 different activation tiles
+// and every one of them again for each n-tile.
+struct TilePos {
+  int m_tile, n_tile;
+};
+__device__ __forceinline__ TilePos tile_pos(int r, int mt, int nt) {
+  constexpr int kBandTiles = 8, kBandFrom = 12;
+  const int bands = mt > kBandFrom ? (mt + kBandTiles - 1) / kBandTiles : 1;
+  const int band_m = (mt + bands - 1) / bands;          // m-tiles per band (the last may have fewer)
+  const int per_band = band_m * nt > 0 ? band_m * nt : 1;
+  const int band = r / per_band;
+  const int r2 = r - band * per_band;
+  const int left = mt - band * band_m;
+  const int width = left < band_m ? (left > 0 ? left : 1) : (band_m > 0 ? band_m : 1);
+  TilePos p;
+  p.n_tile = r2 / width;
+  p.m_tile = band * band_m + (r2 - p.n_tile * width);
+  return p;
+}
+
 template <int BN_OUT>
 struct TileWalker {
   int g_prob = 0, g_expert = 0, g_row0 = 0, g_cnt = 0, g_mt = 0, g_base = 0, g_end = 0;
@@ -230,14 +254,15 @@ struct TileWalker {
     run_end = uni(boundary(xcd + 1));
   }
 
-  // Describes this workgroup's first 64 turns at once - lane r works out turn r -
-  // and leaves them in LDS, kTileWords dwords per turn in PackedTile order, so
+  // Describes 64 of this workgroup's turns at once - lane r works out turn
+  // turn0 + r - and leaves them in LDS, kTileWords dwords per turn in PackedTile order, so
   // that a tile switch inside the kernel is a single LDS read.  Turns past the
   // XCD's run give descriptions that cover no bytes.  Called by one wave.
   __device__ __forceinline__ void build_table(const PersistBatch &batch, int lane, int bk,
-                                              uint32_t *table, bool w8 = false) const {
-    const int w = (lane & 1) ? wgs_per_xcd - 1 - wg_in_xcd : wg_in_xcd;
-    const int id = run_begin + lane * wgs_per_xcd + w;
+                                              uint32_t *table, bool w8 = false, int turn0 = 0) const {
+    const int turn = turn0 + lane;  // entry `lane` of the table describes this turn
+    const int w = (turn & 1) ? wgs_per_xcd - 1 - wg_in_xcd : wg_in_xcd;
+    const int id = run_begin + turn * wgs_per_xcd + w;
     const bool valid = id < run_end;
     const int idc = valid ? id : 0;
     int n_groups = 0;
@@ -262,8 +287,8 @@ struct TileWalker {
       }
     }
     const int r = idc - base;
-    const int n_tile = mt > 0 ? r / mt : 0;
-    const int m_tile = r - n_tile * mt;
+    const TilePos tp = tile_pos(r, mt, (n + BN_OUT - 1) / BN_OUT);
+    const int n_tile = tp.n_tile, m_tile = tp.m_tile;
     const int left = cnt - m_tile * kPBM;
     const int rows = left < kPBM ? left : kPBM;
     const int n0 = n_tile * BN_OUT;
@@ -325,8 +350,8 @@ struct TileWalker {
     const int base = __builtin_amdgcn_readlane(g_base, g);
     const PersistProblem &pr = batch.prob[pi];
     const int r = idc - base;
-    const int n_tile = mt > 0 ? r / mt : 0;
-    const int m_tile = r - n_tile * mt;
+    const TilePos tp = tile_pos(r, mt, (pr.n + BN_OUT - 1) / BN_OUT);
+    const int n_tile = tp.n_tile, m_tile = tp.m_tile;
     const int left = cnt - m_tile * kPBM;
     const int rows = left < kPBM ? left : kPBM;
     t.n0 = n_tile * BN_OUT;
@@ -829,7 +854,11 @@ __device__ __forceinline__ void qsched_block() {
 // row; they are widened to bf16 (exactly) on their way into LDS, so the slots,
 // the fragment reads and the MFMAs are those of the bf16 kernel; the scale
 // multiplies the fp32 sums in the epilogue.
-template <int MODE, bool HAS_BIAS, int BN, bool GATHER, bool W8 = false>
+// REFILL: a workgroup may have more turns than the LDS tile table holds (very
+// large batches); the table is then rewritten every kTableTurns tiles.  A
+// separate instantiation, because even unused the rewrite costs the tile switch
+// registers (1-2 % of fc1 at 8192 tokens).
+template <int MODE, bool HAS_BIAS, int BN, bool GATHER, bool W8 = false, bool REFILL = false>
 __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   constexpr bool SWIGLU = MODE == kFc1Swiglu;
   static_assert(BN == 256 || (BN == 192 && !SWIGLU), "tile widths");
@@ -890,8 +919,22 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   phase_barrier();
+  // The table holds kTableTurns turns; a workgroup with more has its first wave
+  // describe the next kTableTurns when the last entry has been fetched: every
+  // wave arrives at that tile switch, so two barriers fence the rewrite.
   auto fetch_tile = [&](int turn) {
-    return PackedTile{tile_table[turn * kTileWords + (lane < kTileWords ? lane : 0)]};
+    if constexpr (REFILL) {
+      if (turn != 0 && (turn & (kTableTurns - 1)) == 0) {
+        phase_barrier();
+        if (wave == 0) {
+          TileWalker<BN_OUT> walk(batch, lane);
+          walk.build_table(batch, lane, kQBK, tile_table, W8, turn);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        phase_barrier();
+      }
+    }
+    return PackedTile{tile_table[(turn & (kTableTurns - 1)) * kTileWords + (lane < kTileWords ? lane : 0)]};
   };
 
   // ---- global loads: one instruction fetches 8 rows x 128 bytes (8 lanes per
@@ -1239,9 +1282,9 @@ __global__ __launch_bounds__(8 * kWave, 1) void gemm_persist_kernel8(PersistBatc
   gemm_persist_body<MODE, HAS_BIAS, 8>(batch);
 }
 // Four waves, one per SIMD, each with the whole 512-entry register file.
-template <int MODE, bool HAS_BIAS, int BN, bool GATHER, bool W8 = false>
+template <int MODE, bool HAS_BIAS, int BN, bool GATHER, bool W8 = false, bool REFILL = false>
 __global__ __launch_bounds__(4 * kWave, 1) void gemm_persist_kernel4(PersistBatch batch) {
-  gemm_persist64_body<MODE, HAS_BIAS, BN, GATHER, W8>(batch);
+  gemm_persist64_body<MODE, HAS_BIAS, BN, GATHER, W8, REFILL>(batch);
 }
 
 }  // namespace
@@ -1249,6 +1292,7 @@ __global__ __launch_bounds__(4 * kWave, 1) void gemm_persist_kernel4(PersistBatc
 #if DICE_PERSIST_F16
 extern int g_persist_waves;
 int persist_variant(const PersistBatch &b, int mode);
+bool persist_fits_table(const PersistBatch &b, int mode);
 int persist_cu_count();
 #define DICE_PERSIST_LAUNCH launch_grouped_gemm_persist_f16
 namespace {
@@ -1285,23 +1329,15 @@ bool persist_common_ok(const PersistBatch &b, int mode) {
   return groups >= 1 && groups <= kWave && cu_count() >= kNumXcd;
 }
 
-// 64-k kernel: long enough tiles, and a workgroup's tile descriptions must fit
-// the LDS table of kTableTurns entries (the last one stays an invalid tile).
-// The turns of one workgroup are bounded from the host-side row bounds: an XCD
-// gets 1/8 of the total cost, in the worst case all of it in its shortest tiles.
-bool persist64_ok(const PersistBatch &b, int mode) {
+// Whether every workgroup's turns fit the LDS tile table of the 64-k kernel
+// (the last entry stays an invalid tile), bounded from the host-side row
+// bounds: an XCD gets 1/8 of the total cost, in the worst case all of it in its
+// shortest tiles.  Launches that do not fit take the table-rewriting kernels.
+bool persist64_fits_table(const PersistBatch &b, int mode) {
   int64_t cost = 0;
   int min_k32 = 1 << 30;
   for (int i = 0; i < b.n_problems; ++i) {
     const PersistProblem &p = b.prob[i];
-    if (p.k < kQBK * kQMinSteps) return false;
-    if (p.w_scale && b.n_problems != 1) return false;  // fp8 weights: single-problem launches
-    if (p.a_rows) {  // gathered activation rows: SwiGLU instantiation only (the GELU one would
-                     // spill, and measures no faster than a gathered copy plus the plain kernel)
-      if (mode != kFc1Swiglu) return false;
-      if (p.a_div < 1 || p.a_div > 16 || (int64_t)p.a_src_rows * p.a_div >= (1ll << 28)) return false;
-      if ((size_t)p.a_src_rows * p.lda * 2 >= (1ull << 31)) return false;
-    }
     const int bn_out = mode == kFc1Swiglu ? kPBN / 2 : (p.n % 192 == 0 && p.n % 256 != 0 ? 192 : kPBN);
     const int64_t m_tiles = ((int64_t)p.max_rows + kPBM - 1) / kPBM + p.n_experts;
     const int64_t n_tiles = (p.n + bn_out - 1) / bn_out;
@@ -1313,9 +1349,26 @@ bool persist64_ok(const PersistBatch &b, int mode) {
   return (tiles_per_xcd + wgs_per_xcd - 1) / wgs_per_xcd + 2 <= kTableTurns;
 }
 
+// 64-k kernel: long enough tiles.
+bool persist64_ok(const PersistBatch &b, int mode) {
+  for (int i = 0; i < b.n_problems; ++i) {
+    const PersistProblem &p = b.prob[i];
+    if (p.k < kQBK * kQMinSteps) return false;
+    if (p.w_scale && b.n_problems != 1) return false;  // fp8 weights: single-problem launches
+    if (p.a_rows) {  // gathered activation rows: SwiGLU instantiation only (the GELU one would
+                     // spill, and measures no faster than a gathered copy plus the plain kernel)
+      if (mode != kFc1Swiglu) return false;
+      if (p.a_div < 1 || p.a_div > 16 || (int64_t)p.a_src_rows * p.a_div >= (1ll << 28)) return false;
+      if ((size_t)p.a_src_rows * p.lda * 2 >= (1ull << 31)) return false;
+    }
+  }
+  return true;
+}
+
 // 0: neither pipeline applies; 4: the 64-k four-wave kernel; 8: the 32-k eight-wave kernel.
 }  // namespace
 int persist_cu_count() { return cu_count(); }
+bool persist_fits_table(const PersistBatch &b, int mode) { return persist64_fits_table(b, mode); }
 // 0: neither pipeline takes the launch; 4 / 8: the waves of the one that does.
 int persist_variant(const PersistBatch &b, int mode) {
   if (!persist_common_ok(b, mode)) return 0;
@@ -1327,6 +1380,20 @@ int persist_variant(const PersistBatch &b, int mode) {
 
 bool persist_supported(const PersistBatch &b, int mode) { return persist_variant(b, mode) != 0; }
 #endif  // !DICE_PERSIST_F16
+
+namespace {
+typedef void (*PersistKernel)(PersistBatch);
+// The 64-k kernel for one tile shape: bf16/fp16 or fp8 weights, with or without
+// the rewriting of the tile table.
+template <int MODE, bool HAS_BIAS, int BN, bool GATHER>
+PersistKernel pick64(bool w8, bool refill) {
+  if (w8)
+    return refill ? gemm_persist_kernel4<MODE, HAS_BIAS, BN, GATHER, true, true>
+                  : gemm_persist_kernel4<MODE, HAS_BIAS, BN, GATHER, true, false>;
+  return refill ? gemm_persist_kernel4<MODE, HAS_BIAS, BN, GATHER, false, true>
+                : gemm_persist_kernel4<MODE, HAS_BIAS, BN, GATHER, false, false>;
+}
+}  // namespace
 
 int DICE_PERSIST_LAUNCH(const PersistBatch &b, int mode, hipStream_t s) {
   const int waves = persist_variant(b, mode);
@@ -1343,34 +1410,18 @@ int DICE_PERSIST_LAUNCH(const PersistBatch &b, int mode, hipStream_t s) {
   for (int i = 0; i < b.n_problems; ++i)
     narrow = narrow && b.prob[i].n % 192 == 0 && b.prob[i].n % 256 != 0;
   const bool w8 = b.prob[0].w_scale != nullptr;
-  if (waves == 4 && w8) {
-    if (narrow) {
-      switch (mode) {
-        case kFc1Gelu: kern = has_bias ? gemm_persist_kernel4<kFc1Gelu, true, 192, false, true> : gemm_persist_kernel4<kFc1Gelu, false, 192, false, true>; break;
-        default: kern = has_bias ? gemm_persist_kernel4<kFc2, true, 192, false, true> : gemm_persist_kernel4<kFc2, false, 192, false, true>; break;
-      }
-    } else {
-      switch (mode) {
-        case kFc1Swiglu:
-          kern = gathered ? gemm_persist_kernel4<kFc1Swiglu, false, 256, true, true> : gemm_persist_kernel4<kFc1Swiglu, false, 256, false, true>;
-          break;
-        case kFc1Gelu: kern = has_bias ? gemm_persist_kernel4<kFc1Gelu, true, 256, false, true> : gemm_persist_kernel4<kFc1Gelu, false, 256, false, true>; break;
-        default: kern = has_bias ? gemm_persist_kernel4<kFc2, true, 256, false, true> : gemm_persist_kernel4<kFc2, false, 256, false, true>; break;
-      }
-    }
-  } else if (waves == 4 && narrow) {
-    switch (mode) {
-      case kFc1Gelu: kern = has_bias ? gemm_persist_kernel4<kFc1Gelu, true, 192, false> : gemm_persist_kernel4<kFc1Gelu, false, 192, false>; break;
-      default: kern = has_bias ? gemm_persist_kernel4<kFc2, true, 192, false> : gemm_persist_kernel4<kFc2, false, 192, false>; break;
-    }
-  } else if (waves == 4) {
-    switch (mode) {
-      case kFc1Swiglu:
-        kern = gathered ? gemm_persist_kernel4<kFc1Swiglu, false, 256, true> : gemm_persist_kernel4<kFc1Swiglu, false, 256, false>;
-        break;
-      case kFc1Gelu: kern = has_bias ? gemm_persist_kernel4<kFc1Gelu, true, 256, false> : gemm_persist_kernel4<kFc1Gelu, false, 256, false>; break;
-      default: kern = has_bias ? gemm_persist_kernel4<kFc2, true, 256, false> : gemm_persist_kernel4<kFc2, false, 256, false>; break;
-    }
+  if (waves == 4) {
+    const bool refill = !persist_fits_table(b, mode);
+    if (mode == kFc1Swiglu)
+      kern = gathered ? pick64<kFc1Swiglu, false, 256, true>(w8, refill) : pick64<kFc1Swiglu, false, 256, false>(w8, refill);
+    else if (mode == kFc1Gelu && narrow)
+      kern = has_bias ? pick64<kFc1Gelu, true, 192, false>(w8, refill) : pick64<kFc1Gelu, false, 192, false>(w8, refill);
+    else if (mode == kFc1Gelu)
+      kern = has_bias ? pick64<kFc1Gelu, true, 256, false>(w8, refill) : pick64<kFc1Gelu, false, 256, false>(w8, refill);
+    else if (narrow)
+      kern = has_bias ? pick64<kFc2, true, 192, false>(w8, refill) : pick64<kFc2, false, 192, false>(w8, refill);
+    else
+      kern = has_bias ? pick64<kFc2, true, 256, false>(w8, refill) : pick64<kFc2, false, 256, false>(w8, refill);
   } else {
     switch (mode) {
       case kFc1Swiglu: kern = gemm_persist_kernel8<kFc1Swiglu, false>; break;
