@@ -587,8 +587,11 @@ def test_block_c2_bf16_full_size(dev, variant):
 
 
 def test_block_many_tokens_per_workgroup(dev):
-    """More tiles per workgroup than the 64-k kernel's tile table holds: the layer
-    has to pick another kernel and still agree with the oracle."""
+    """More tiles per workgroup than the 64-k kernel's tile table holds: the
+    workgroups rewrite their table on the way.  Checked against the oracle on a
+    sample and, for every token, against the same block run on quarters of the
+    batch (tokens are independent and a row's sums do not depend on its tile, so
+    the two must agree bit for bit)."""
     D, E, N = 384, 8, 172032
     p = O.make_block_params(D, E, 2, 4, 2, seed=5, dtype=torch.bfloat16, variant="swiglu")
     x = torch.randn(1, N, D, generator=_gen(5)).bfloat16()
@@ -597,6 +600,27 @@ def test_block_many_tokens_per_workgroup(dev):
     want, _, logits = _subset_oracle(p, x.view(-1, D), sub, torch.bfloat16)
     ties = O.gate_tie_rows(logits, 2).view(-1)
     assert rel_l2(y.view(-1, D)[sub][~ties], want[~ties]) < BF16_TOL
+    xq = x.view(4, N // 4, D).to(dev)
+    parts = torch.cat([blk(xq[i:i + 1]).cpu() for i in range(4)], dim=1)
+    assert torch.equal(parts.view(-1, D), y.view(-1, D))
+
+
+def test_block_xl_width_large_batch_matches_chunks(dev):
+    """73728 tokens at DiT-XL width: groups of ~72 m-tiles (banded tile order) and
+    ~100 turns per workgroup in fc1 (rewritten tile table).  Every token must come
+    out bit-identical to the same block run on 8192-token chunks, which take the
+    plain tile order and a single table; a sample is checked against the oracle."""
+    D, E, N = 1152, 8, 73728
+    p = O.make_block_params(D, E, 2, 4, 2, seed=8, dtype=torch.bfloat16)
+    x = torch.randn(1, N, D, generator=_gen(8)).bfloat16()
+    blk, y = _run_block(dev, p, x, "swiglu", torch.bfloat16)
+    xq = x.view(N // 8192, 8192, D).to(dev)
+    parts = torch.cat([blk(xq[i:i + 1]).cpu() for i in range(N // 8192)], dim=1)
+    assert torch.equal(parts.view(-1, D), y.view(-1, D))
+    sub = torch.randperm(N, generator=_gen(9))[:128]
+    want, _, logits = _subset_oracle(p, x.view(-1, D), sub, torch.bfloat16)
+    ok = ~O.gate_tie_rows(logits, 2).view(-1)
+    assert rel_l2(y.view(-1, D)[sub][ok], want[ok]) < BF16_TOL
 
 
 def test_block_c3_zipf_load(dev):
