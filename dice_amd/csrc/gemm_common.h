@@ -58,13 +58,22 @@ inline int64_t max_tiles(int64_t max_rows, int n_experts, int n, int bm, int bn_
 // the same weight tile across neighbouring m-tiles.
 template <int BM, int BN_OUT>
 __device__ __forceinline__ TileCoord locate_tile(const GemmParams &p) {
+  // Every wave works this out for itself, 64 experts at a time: lane l reads the
+  // row range of expert e0 + l (two loads per lane instead of a scalar loop of
+  // dependent loads over the experts, which costs microseconds before a tile of
+  // a small batch can start).
   TileCoord t;
   t.active = false;
+  const int lane = threadIdx.x & (kWave - 1);
   const int n_tiles = (p.n + BN_OUT - 1) / BN_OUT;
-  int total_mt = 0;
-  for (int e = 0; e < p.n_experts; ++e) {
-    const int cnt = p.offsets[e + 1] - p.offsets[e];
-    total_mt += (cnt + BM - 1) / BM;
+  const bool one_pass = p.n_experts <= kWave;
+  int begin = 0, cnt = 0, mt = 0, total_mt = 0;
+  for (int e0 = 0; e0 < p.n_experts; e0 += kWave) {
+    const int e = e0 + lane;
+    begin = e < p.n_experts ? p.offsets[e] : 0;
+    cnt = e < p.n_experts ? p.offsets[e + 1] - begin : 0;
+    mt = (cnt + BM - 1) / BM;
+    total_mt += wave_sum_i32(mt);
   }
   const int total = total_mt * n_tiles;
   const int per_xcd = (total + kNumXcd - 1) / kNumXcd;
@@ -72,25 +81,39 @@ __device__ __forceinline__ TileCoord locate_tile(const GemmParams &p) {
   const int j = blockIdx.x / kNumXcd;
   const int logical = xcd * per_xcd + j;
   if (j >= per_xcd || logical >= total) return t;
-  int base = 0;
-  for (int e = 0; e < p.n_experts; ++e) {
-    const int begin = p.offsets[e];
-    const int cnt = p.offsets[e + 1] - begin;
-    const int mt = (cnt + BM - 1) / BM;
-    const int span = mt * n_tiles;
-    if (logical < base + span) {
-      const int r = logical - base;
-      const int n_tile = r / mt;
-      const int m_tile = r - n_tile * mt;
-      t.expert = e;
-      t.row_begin = begin + m_tile * BM;
-      const int left = cnt - m_tile * BM;
-      t.rows_valid = left < BM ? left : BM;
-      t.n0 = n_tile * BN_OUT;
+  int base_mt = 0;  // m-tiles of the experts before this chunk
+  for (int e0 = 0; e0 < p.n_experts; e0 += kWave) {
+    if (!one_pass) {  // (a single chunk still holds its row ranges from the first loop)
+      const int e = e0 + lane;
+      begin = e < p.n_experts ? p.offsets[e] : 0;
+      cnt = e < p.n_experts ? p.offsets[e + 1] - begin : 0;
+      mt = (cnt + BM - 1) / BM;
+    }
+    int inc = mt;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+      const int up = __shfl_up(inc, o, kWave);
+      if (lane >= o) inc += up;
+    }
+    inc += base_mt;
+    const int span_begin = (inc - mt) * n_tiles, span_end = inc * n_tiles;
+    const uint64_t hit = __ballot(mt > 0 && logical >= span_begin && logical < span_end);
+    if (hit) {
+      const int g = __builtin_ctzll(hit);
+      const int g_begin = __shfl(begin, g, kWave), g_cnt = __shfl(cnt, g, kWave);
+      const int g_mt = __shfl(mt, g, kWave), g_base = __shfl(span_begin, g, kWave);
+      const int r = logical - g_base;
+      const int n_tile = r / g_mt;
+      const int m_tile = r - n_tile * g_mt;
+      t.expert = __builtin_amdgcn_readfirstlane(e0 + g);
+      t.row_begin = __builtin_amdgcn_readfirstlane(g_begin + m_tile * BM);
+      const int left = g_cnt - m_tile * BM;
+      t.rows_valid = __builtin_amdgcn_readfirstlane(left < BM ? left : BM);
+      t.n0 = __builtin_amdgcn_readfirstlane(n_tile * BN_OUT);
       t.active = true;
       return t;
     }
-    base += span;
+    base_mt = __shfl(inc, kWave - 1, kWave);
   }
   return t;
 }
@@ -145,6 +168,7 @@ struct PersistBatch {
   PersistProblem prob[kMaxPersistProblems];
 };
 bool persist_supported(const PersistBatch &b, int mode);
+int persist_cu_count();  // compute units of the current device
 bool gemm_config_wants_persistent();  // tuning hook state: both stages set to the persistent kernel
 int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s);      // bf16
 int launch_grouped_gemm_persist_f16(const PersistBatch &b, int mode, hipStream_t s);  // fp16

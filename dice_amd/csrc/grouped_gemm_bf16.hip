@@ -74,8 +74,14 @@ __device__ __forceinline__ int lds_off(int row, int chunk) {
   return row * kBK + ((chunk ^ swizzle(row)) * kChunkElems);
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int MODE, bool W_FP8>
+// DEPTH: register stages between global memory and LDS.  The loads of step
+// kt + DEPTH are issued while step kt is multiplied and reach LDS DEPTH - 1
+// steps later; a 64 x 64 tile multiplies a step in 0.2 - 0.4 us, a load takes a
+// microsecond or more, and with few rows there is one wave per SIMD: nothing
+// else hides the difference.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int MODE, bool W_FP8, int DEPTH>
 __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_kernel(GemmParams p) {
+  static_assert(DEPTH == 2 || DEPTH == 4, "an even number of register stages: the LDS stage of a step is its parity");
   constexpr int NT = WAVES_M * WAVES_N * kWave;
   constexpr bool SWIGLU = MODE == kFc1Swiglu;
   constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
@@ -128,30 +134,31 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
     b_src[i] = (uint32_t)wrow * (uint32_t)p.k + b_chunk * (W_FP8 ? 16 : kChunkElems);
   }
 
-  u32x4_t a_reg[A_PASSES], b_reg[B_PASSES];
-  auto load_global = [&](int k0) {
+  u32x4_t a_reg[DEPTH][A_PASSES], b_reg[DEPTH][B_PASSES];
+  // (`r`, the register stage, is a compile-time constant wherever this is called)
+  auto load_global = [&](int k0, int r) {
 #pragma unroll
     for (int i = 0; i < A_PASSES; ++i)
-      a_reg[i] = *reinterpret_cast<const u32x4_t *>(a_base + a_src[i] + k0);
+      a_reg[r][i] = *reinterpret_cast<const u32x4_t *>(a_base + a_src[i] + k0);
     if (W_FP8) {
       const uint8_t *wb = (const uint8_t *)p.w + w_expert;
 #pragma unroll
       for (int i = 0; i < B_PASSES; ++i)
-        b_reg[i] = *reinterpret_cast<const u32x4_t *>(wb + b_src[i] + k0);
+        b_reg[r][i] = *reinterpret_cast<const u32x4_t *>(wb + b_src[i] + k0);
     } else {
       const h16_t *wb = (const h16_t *)p.w + w_expert;
 #pragma unroll
       for (int i = 0; i < B_PASSES; ++i)
-        b_reg[i] = *reinterpret_cast<const u32x4_t *>(wb + b_src[i] + k0);
+        b_reg[r][i] = *reinterpret_cast<const u32x4_t *>(wb + b_src[i] + k0);
     }
   };
-  auto store_lds = [&](int stage) {
+  auto store_lds = [&](int stage, int r) {
     h16_t *as = As + stage * A_STAGE;
     h16_t *bs = Bs + stage * B_STAGE;
 #pragma unroll
     for (int i = 0; i < A_PASSES; ++i) {
       const int rt = a_row0 + i * A_ROWS_PER_PASS;
-      *reinterpret_cast<u32x4_t *>(as + lds_off(rt, a_chunk)) = a_reg[i];
+      *reinterpret_cast<u32x4_t *>(as + lds_off(rt, a_chunk)) = a_reg[r][i];
     }
 #pragma unroll
     for (int i = 0; i < B_PASSES; ++i) {
@@ -162,12 +169,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
         u32x4_t lo, hi;
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
-          auto c0 = DICE_WIDEN_FP8(b_reg[i][q], 1.0f, false);
-          auto c1 = DICE_WIDEN_FP8(b_reg[i][q], 1.0f, true);
+          auto c0 = DICE_WIDEN_FP8(b_reg[r][i][q], 1.0f, false);
+          auto c1 = DICE_WIDEN_FP8(b_reg[r][i][q], 1.0f, true);
           lo[2 * q] = __builtin_bit_cast(uint32_t, c0);
           lo[2 * q + 1] = __builtin_bit_cast(uint32_t, c1);
-          auto d0 = DICE_WIDEN_FP8(b_reg[i][q + 2], 1.0f, false);
-          auto d1 = DICE_WIDEN_FP8(b_reg[i][q + 2], 1.0f, true);
+          auto d0 = DICE_WIDEN_FP8(b_reg[r][i][q + 2], 1.0f, false);
+          auto d1 = DICE_WIDEN_FP8(b_reg[r][i][q + 2], 1.0f, true);
           hi[2 * q] = __builtin_bit_cast(uint32_t, d0);
           hi[2 * q + 1] = __builtin_bit_cast(uint32_t, d1);
         }
@@ -176,7 +183,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
       } else
 #endif
       {
-        *reinterpret_cast<u32x4_t *>(bs + lds_off(rt, b_chunk)) = b_reg[i];
+        *reinterpret_cast<u32x4_t *>(bs + lds_off(rt, b_chunk)) = b_reg[r][i];
       }
     }
   };
@@ -201,12 +208,24 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
   const int frag_row = lane & 31, frag_half = lane >> 5;
   const int kt_count = p.k / kBK;
 
-  load_global(0);
-  store_lds(0);
+  // Step kt sits in register stage kt % DEPTH until it is written to LDS stage
+  // kt % 2.  Loads past the last step re-read the last one (every step issues the
+  // same number of loads, so the wait for a stage's data may leave exactly the
+  // younger stages' loads in flight); their data is never written to LDS.
+  const int k_last = (kt_count - 1) * kBK;
+  auto k_of = [&](int kt) { return kt < kt_count ? kt * kBK : k_last; };
+#pragma unroll
+  for (int r = 0; r < DEPTH; ++r) load_global(k_of(r), r);
+  store_lds(0, 0);
   __syncthreads();
-  for (int kt = 0; kt < kt_count; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < kt_count) load_global((kt + 1) * kBK);
+  for (int kt0 = 0; kt0 < kt_count; kt0 += DEPTH) {
+#pragma unroll
+   for (int r = 0; r < DEPTH; ++r) {
+    const int kt = kt0 + r;
+    if (kt >= kt_count) break;
+    constexpr int kStages = 2;
+    const int cur = r % kStages;
+    load_global(k_of(kt + DEPTH), r);  // stage r went to LDS one step ago
     const h16_t *as = As + cur * A_STAGE;
     const h16_t *bs = Bs + cur * B_STAGE;
 #if DICE_GEMM_F32
@@ -249,8 +268,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
           acc[i][j] = DICE_MFMA_32X32X16(wf[j], af[i], acc[i][j], 0, 0, 0);
     }
 #endif
-    if (kt + 1 < kt_count) store_lds(cur ^ 1);
+    if (kt + 1 < kt_count) store_lds(cur ^ 1, (r + 1) % DEPTH);
     __syncthreads();
+   }
   }
 
   // ---- epilogue: lane holds row (lane&31), columns 8*q + 4*(lane>>5) + {0..3} of each block ----
@@ -295,13 +315,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int MODE, bool W_FP8>
 int launch_cfg(const GemmParams &p, int64_t max_rows, hipStream_t s) {
+  constexpr int DEPTH = BM * BN <= 64 * 128 ? 4 : 2;
   constexpr int BN_OUT = MODE == kFc1Swiglu ? BN / 2 : BN;
   constexpr int NT = WAVES_M * WAVES_N * kWave;
   constexpr size_t lds = 2ull * (BM + BN) * kBK * sizeof(h16_t);
   const int64_t grid = max_tiles(max_rows, p.n_experts, p.n, BM, BN_OUT);
   if (grid <= 0) return DICE_OK;
   if (grid >= (1ll << 31)) return fail(DICE_ERR_UNSUPPORTED, "16-bit expert GEMM: grid too large");
-  auto kern = grouped_gemm_bf16_kernel<BM, BN, WAVES_M, WAVES_N, MODE, W_FP8>;
+  auto kern = grouped_gemm_bf16_kernel<BM, BN, WAVES_M, WAVES_N, MODE, W_FP8, DEPTH>;
   if (lds > 48 * 1024) {
     static thread_local bool configured = false;
     if (!configured) {
@@ -328,11 +349,18 @@ namespace {
 
 template <int MODE, bool W_FP8>
 int launch_mode(const GemmParams &p, int cfg, int64_t max_rows, hipStream_t s) {
+  constexpr bool SWIGLU = MODE == kFc1Swiglu;
+  // Few rows (the reference's DiT-S batches: 1024 tokens): 128-row tiles would
+  // leave most compute units without one and the rest with a long k loop each;
+  // 64-row tiles with 64 output columns make four times as many.
+  if (cfg == 0 && max_tiles(max_rows, p.n_experts, p.n, 128, SWIGLU ? 64 : 128) < 2 * persist_cu_count()) cfg = 3;
   switch (cfg) {
     case 1:
       return launch_cfg<256, 256, 2, 4, MODE, W_FP8>(p, max_rows, s);
     case 2:
       return launch_cfg<256, 128, 2, 2, MODE, W_FP8>(p, max_rows, s);
+    case 3:
+      return launch_cfg<64, SWIGLU ? 128 : 64, 2, 2, MODE, W_FP8>(p, max_rows, s);
     default:
       return launch_cfg<128, 128, 2, 2, MODE, W_FP8>(p, max_rows, s);
   }
@@ -377,8 +405,9 @@ bool gemm_config_wants_persistent() { return g_cfg_fc1 >= kCfgPersistent && g_cf
 }  // namespace dice
 
 // Tuning hook.  For the permutation-addressed kernels of this file it selects
-// the tiling per GEMM (0: 128x128x64 / 4 waves, 1: 256x256x64 / 8 waves,
-// 2: 256x128x64 / 4 waves).  Values >= 20 for both stages make dice_grouped_mlp
+// the tiling per GEMM (0: 128x128 / 4 waves, or 64-row tiles where those would
+// be too few; 1: 256x256 / 8 waves; 2: 256x128 / 4 waves; 3: 64x64 outputs / 4
+// waves; 4: 128x128 whatever the size).  Values >= 20 for both stages make dice_grouped_mlp
 // use the persistent kernels for contiguous rows; 20 also restricts every
 // persistent launch to the 32-k pipeline.  Not part of the drop-in surface;
 // used by the benchmark and the tests to compare kernels.

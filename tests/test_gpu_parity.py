@@ -244,6 +244,11 @@ def _check_mlp(dev, N, D, E, ratio, dtype, variant, counts=None, cfg=(0, 0), tol
 def test_mlp_fp32(dev, variant):
     _check_mlp(dev, 512, 128, 8, 4, torch.float32, variant)
     _check_mlp(dev, 1024, 384, 8, 4, torch.float32, variant)   # DiT-S/2 expert shape
+    # more experts than a wavefront has lanes (the tile search walks them 64 at a
+    # time), some empty, most smaller than a tile
+    counts = [(e * 7) % 33 for e in range(80)]
+    counts[79] += 1280 - sum(counts)
+    _check_mlp(dev, 640, 128, 80, 2, torch.float32, variant, counts=counts)
 
 
 @pytest.mark.parametrize("cfg", [0, 1, 2])
