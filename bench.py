@@ -24,7 +24,7 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 # Bytes one fc1 launch moves past the L2 (Infinity Cache + HBM), from rocprofv3 --pmc FETCH_SIZE (x2.0, the
 # factor a plain 256 MiB copy needs) + WRITE_SIZE (x1.0): profiles/layer_c2_bf16_hbm_traffic.txt.
-FC1_HBM_TRAFFIC_BYTES = 1.149e9
+FC1_HBM_TRAFFIC_BYTES = 0.941e9
 
 N_TOKENS, D, E, TOPK, RATIO = 8192, 1152, 8, 2, 4
 
