@@ -286,6 +286,17 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
   DICE_REQUIRE(n_tokens >= 0 && n_tokens * L->top_k < (1ll << 31), DICE_ERR_BAD_ARG, "%s: n_tokens %lld",
                who, (long long)n_tokens);
   if (n_tokens == 0) return DICE_OK;
+  // Entries are checked before anything is launched.
+  if (work_in)
+    DICE_REQUIRE(work_in->x && work_in->offsets && work_in->perm && work_in->rows && work_in->max_rows >= 0 &&
+                     work_in->max_rows <= n_tokens * L->top_k,
+                 DICE_ERR_BAD_ARG, "%s: the entry to run the experts on lacks a buffer or holds %lld rows (at most %lld)",
+                 who, (long long)work_in->max_rows, (long long)(n_tokens * L->top_k));
+  else if (put)
+    DICE_REQUIRE(put->rows, DICE_ERR_BAD_ARG, "%s: the entry to fill lacks a buffer (its experts run in this call: rows)", who);
+  if (emit_in)
+    DICE_REQUIRE(emit_in->rows && emit_in->inv_perm && emit_in->topk_weight, DICE_ERR_BAD_ARG,
+                 "%s: the entry to combine lacks a buffer", who);
   LayerWorkspace w = carve_layer(L, n_tokens, workspace);
   DICE_REQUIRE(workspace && workspace_bytes >= w.total, DICE_ERR_WORKSPACE, "%s: workspace %zu < %zu bytes",
                who, workspace_bytes, w.total);
