@@ -169,7 +169,7 @@ struct PersistBatch {
 };
 bool persist_supported(const PersistBatch &b, int mode);
 int persist_cu_count();  // compute units of the current device
-bool gemm_config_wants_persistent();  // tuning hook state: both stages set to the persistent kernel
+bool gemm_config_allows_persistent(int mode);  // tuning hook state: no tiling of the permutation-addressed kernels is forced for this stage
 int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s);      // bf16
 int launch_grouped_gemm_persist_f16(const PersistBatch &b, int mode, hipStream_t s);  // fp16
 

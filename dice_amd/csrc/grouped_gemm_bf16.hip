@@ -371,7 +371,8 @@ int launch_mode(const GemmParams &p, int cfg, int64_t max_rows, hipStream_t s) {
 int DICE_GEMM_LAUNCH(const GemmParams &p, int mode, int w_dtype, int64_t max_rows, hipStream_t s) {
   if (p.k % kBK != 0) return fail(DICE_ERR_UNSUPPORTED, "16-bit expert GEMM: k %d %% %d != 0", p.k, kBK);
   if (p.n % 8 != 0) return fail(DICE_ERR_UNSUPPORTED, "16-bit expert GEMM: n %d %% 8 != 0", p.n);
-  const int cfg = mode == kFc2 ? g_cfg_fc2 : g_cfg_fc1;
+  int cfg = mode == kFc2 ? g_cfg_fc2 : g_cfg_fc1;
+  if (cfg >= 20) cfg = 0;  // the hook's persistent-kernel values: this file picks its own tiling
 #if DICE_GEMM_F32
   if (w_dtype != DICE_F32) return fail(DICE_ERR_UNSUPPORTED, "fp32 expert GEMM: w_dtype %d", w_dtype);
   switch (mode) {
@@ -401,16 +402,20 @@ int DICE_GEMM_LAUNCH(const GemmParams &p, int mode, int w_dtype, int64_t max_row
 namespace dice {
 constexpr int kCfgPersistent = 20;
 extern int g_persist_waves;
-bool gemm_config_wants_persistent() { return g_cfg_fc1 >= kCfgPersistent && g_cfg_fc2 >= kCfgPersistent; }
+bool gemm_config_allows_persistent(int mode) {
+  const int cfg = mode == kFc2 ? g_cfg_fc2 : g_cfg_fc1;
+  return cfg == 0 || cfg >= kCfgPersistent;
+}
 }  // namespace dice
 
-// Tuning hook.  For the permutation-addressed kernels of this file it selects
-// the tiling per GEMM (0: 128x128 / 4 waves, or 64-row tiles where those would
-// be too few; 1: 256x256 / 8 waves; 2: 256x128 / 4 waves; 3: 64x64 outputs / 4
-// waves; 4: 128x128 whatever the size).  Values >= 20 for both stages make dice_grouped_mlp
-// use the persistent kernels for contiguous rows; 20 also restricts every
-// persistent launch to the 32-k pipeline.  Not part of the drop-in surface;
-// used by the benchmark and the tests to compare kernels.
+// Tuning hook, per GEMM stage.  0 (default) and values >= 20: dice_grouped_mlp
+// takes the persistent kernels where they apply and otherwise the
+// permutation-addressed kernels of this file with 128x128 tiles / 4 waves, or
+// 64-row tiles where those would be too few; 20 also restricts every persistent
+// launch to the 32-k pipeline.  1 .. 4 name a tiling of this file's kernels for
+// dice_grouped_mlp whatever the shape (1: 256x256 / 8 waves; 2: 256x128 / 4
+// waves; 3: 64x64 outputs / 4 waves; 4: 128x128).  Not part of the drop-in
+// surface; used by the benchmark and the tests to compare kernels.
 extern "C" int dice_set_gemm_config(int fc1_cfg, int fc2_cfg) {
   dice::g_cfg_fc1 = fc1_cfg;
   dice::g_cfg_fc2 = fc2_cfg;

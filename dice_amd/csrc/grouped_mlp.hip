@@ -141,53 +141,64 @@ int grouped_mlp_impl(int stages, const void *x, int act_dtype, const int32_t *pe
   hipStream_t s = (hipStream_t)stream;
   const bool swiglu = act_variant == DICE_ACT_SWIGLU;
 
-  // Contiguous grouped rows + bf16 weights: the persistent kernel applies.
-  if (!perm && is_16bit(act_dtype) && gemm_config_wants_persistent()) {
-    PersistBatch pb1{};
-    pb1.n_problems = 1;
+  // 16-bit activations: each stage takes the persistent kernel where it applies
+  // (fc1 addresses rows through the permutation itself in its SwiGLU form; fc2
+  // writes grouped rows, so a scatter to slot order stays with the
+  // permutation-addressed kernel), unless the tuning hook names a tiling.
+  const int m1 = swiglu ? kFc1Swiglu : kFc1Gelu;
+  PersistBatch pb1{}, pb2{};
+  bool fc1_persist = false, fc2_persist = false;
+  if (is_16bit(act_dtype)) {
+    pb1.n_problems = pb2.n_problems = 1;
     pb1.prob[0] = PersistProblem{x, hidden, offsets, n_experts, w1, swiglu ? 2 * inter : inter, inter,
                                  swiglu ? nullptr : b1, h, inter, inter, hidden, (int)max_rows};
-    PersistBatch pb2{};
-    pb2.n_problems = 1;
+    if (perm) {
+      // This entry point is not told how many rows x has: the row addresses get
+      // the widest range the kernel can address (the permutation-addressed
+      // kernel checks none either); slots beyond it fall back to that kernel.
+      pb1.prob[0].a_rows = perm;
+      pb1.prob[0].a_div = slots_per_token;
+      const int64_t by_slots = ((1ll << 28) - 1) / slots_per_token;
+      const int64_t by_bytes = ((1ll << 31) - 1) / ((int64_t)hidden * 2);
+      pb1.prob[0].a_src_rows = (int)(by_slots < by_bytes ? by_slots : by_bytes);
+    }
     pb2.prob[0] = PersistProblem{h, inter, offsets, n_experts, w2, hidden, 0, swiglu ? nullptr : b2,
                                  out, hidden, hidden, inter, (int)max_rows};
     if (w_dtype == DICE_FP8_E4M3) {
       pb1.prob[0].w_scale = w1_scale;
       pb2.prob[0].w_scale = w2_scale;
     }
-    const int m1 = swiglu ? kFc1Swiglu : kFc1Gelu;
-    if (persist_supported(pb1, m1) && persist_supported(pb2, kFc2)) {
-      if (stages & 1) {
-        rc = launch_persist(pb1, m1, act_dtype, s);
-        if (rc) return rc;
-      }
-      if (stages & 2) return launch_persist(pb2, kFc2, act_dtype, s);
-      return DICE_OK;
-    }
+    fc1_persist = gemm_config_allows_persistent(m1) && persist_supported(pb1, m1);
+    fc2_persist = !scatter_to_slots && gemm_config_allows_persistent(kFc2) && persist_supported(pb2, kFc2);
   }
 
-  GemmParams p1{};
-  p1.a = x;
-  p1.a_perm = perm;
-  p1.a_div = perm ? slots_per_token : 1;
-  p1.lda = hidden;
-  p1.offsets = offsets;
-  p1.n_experts = n_experts;
-  p1.w = w1;
-  p1.w_rows = swiglu ? 2 * inter : inter;
-  p1.up_offset = inter;
-  p1.bias = swiglu ? nullptr : b1;
-  p1.w_scale = w_dtype == DICE_FP8_E4M3 ? w1_scale : nullptr;
-  p1.c = h;
-  p1.ldc = inter;
-  p1.c_perm = nullptr;
-  p1.n = inter;
-  p1.k = hidden;
   if (stages & 1) {
-    rc = run_gemm(p1, swiglu ? kFc1Swiglu : kFc1Gelu, act_dtype, w_dtype, max_rows, s);
+    if (fc1_persist) {
+      rc = launch_persist(pb1, m1, act_dtype, s);
+    } else {
+      GemmParams p1{};
+      p1.a = x;
+      p1.a_perm = perm;
+      p1.a_div = perm ? slots_per_token : 1;
+      p1.lda = hidden;
+      p1.offsets = offsets;
+      p1.n_experts = n_experts;
+      p1.w = w1;
+      p1.w_rows = swiglu ? 2 * inter : inter;
+      p1.up_offset = inter;
+      p1.bias = swiglu ? nullptr : b1;
+      p1.w_scale = w_dtype == DICE_FP8_E4M3 ? w1_scale : nullptr;
+      p1.c = h;
+      p1.ldc = inter;
+      p1.c_perm = nullptr;
+      p1.n = inter;
+      p1.k = hidden;
+      rc = run_gemm(p1, m1, act_dtype, w_dtype, max_rows, s);
+    }
     if (rc) return rc;
   }
   if (!(stages & 2)) return DICE_OK;
+  if (fc2_persist) return launch_persist(pb2, kFc2, act_dtype, s);
 
   GemmParams p2{};
   p2.a = h;

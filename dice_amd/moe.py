@@ -423,9 +423,8 @@ class SparseMoeBlock(nn.Module):
         k = self.num_experts_per_tok
         n = x.shape[0]
         idx = flat_expert_indices.to(torch.int32).contiguous()
-        _, offsets, perm, _ = ops.dispatch(idx, len(self.experts))
-        slot_out = ops.grouped_mlp(x.contiguous(), perm, k, offsets, n * k, p.w1, p.w2, self.variant,
-                                   p.b1, p.b2, p.w1_scale, p.w2_scale, scatter_to_slots=True,
-                                   n_out_rows=n * k)
+        _, offsets, perm, inv_perm = ops.dispatch(idx, len(self.experts))
+        rows = ops.grouped_mlp(x.contiguous(), perm, k, offsets, n * k, p.w1, p.w2, self.variant,
+                               p.b1, p.b2, p.w1_scale, p.w2_scale, scatter_to_slots=False)
         w = flat_expert_weights.reshape(n, k).float().contiguous()
-        return ops.combine(slot_out, w, n, k)
+        return ops.combine(rows, w, n, k, inv_perm=inv_perm)

@@ -234,7 +234,12 @@ def _check_mlp(dev, N, D, E, ratio, dtype, variant, counts=None, cfg=(0, 0), tol
             want[sel] = p.experts[e](xs[sel])
     tol = tol or (FP32_TOL if dtype == torch.float32 else BF16_TOL)
     assert rel_l2(out, want) < tol, f"slot-order output off: {rel_l2(out, want)}"
-    assert torch.equal(out_grouped, out[perm]), "grouped and scattered outputs must be the same rows"
+    if cfg == (0, 0) and dtype != torch.float32:
+        # default selection: the grouped output comes from the persistent fc2 kernel where it applies, the
+        # scattered one from the permutation-addressed kernel (another order of the same fp32 sums)
+        assert rel_l2(out_grouped, out[perm]) < 4e-3
+    else:
+        assert torch.equal(out_grouped, out[perm]), "grouped and scattered outputs must be the same rows"
     # per-row check so that one bad tile cannot hide inside the norm
     err = (out.double() - want.double()).norm(dim=1) / want.double().norm(dim=1).clamp_min(1e-6)
     assert err.max() < 5 * tol, f"worst row {int(err.argmax())} rel err {float(err.max())}"
@@ -251,7 +256,7 @@ def test_mlp_fp32(dev, variant):
     _check_mlp(dev, 640, 128, 80, 2, torch.float32, variant, counts=counts)
 
 
-@pytest.mark.parametrize("cfg", [0, 1, 2])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4])   # 0: default selection; 1-4: tilings of the permutation-addressed kernels
 @pytest.mark.parametrize("variant", ["swiglu", "gelu_tanh"])
 def test_mlp_bf16_tilings(dev, variant, cfg):
     _check_mlp(dev, 1024, 256, 8, 4, torch.bfloat16, variant, cfg=(cfg, cfg))
@@ -318,7 +323,7 @@ def test_mlp_bf16_biased_tiles_across_experts(dev):
 F16_TOL = 4e-3   # 11-bit mantissa: the 2e-2 bar of bf16 would hide a wrong rounding
 
 
-@pytest.mark.parametrize("cfg", [0, 1, 2])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 4])
 @pytest.mark.parametrize("variant", ["swiglu", "gelu_tanh"])
 def test_mlp_f16_tilings(dev, variant, cfg):
     _check_mlp(dev, 1024, 256, 8, 4, torch.float16, variant, cfg=(cfg, cfg), tol=F16_TOL)
@@ -357,7 +362,7 @@ def test_block_f16_full_size(dev, fp8):
     assert not fp8 or err > 1e-3        # the quantised weights are really in use
 
 
-@pytest.mark.parametrize("cfg", [0, 1, 2])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4])
 def test_mlp_bf16_ragged_groups(dev, cfg):
     # empty experts, single-row groups, a group of exactly one tile, one hot expert
     _check_mlp(dev, 512, 256, 8, 2, torch.bfloat16, "swiglu", counts=[0, 1, 128, 0, 257, 3, 635, 0],
@@ -382,7 +387,7 @@ def test_fp8_quantiser_bit_exact(dev):
     assert torch.equal(q.cpu().view(torch.uint8).view(64, 128), wq.view(torch.uint8))
 
 
-@pytest.mark.parametrize("cfg", [0, 1])
+@pytest.mark.parametrize("cfg", [0, 1, 4])
 @pytest.mark.parametrize("variant", ["swiglu", "gelu_tanh"])
 def test_mlp_fp8_weights(dev, variant, cfg):
     from dice_amd import lib, ops
