@@ -633,6 +633,32 @@ def test_block_xl_width_large_batch_matches_chunks(dev):
     assert rel_l2(y.view(-1, D)[sub][ok], want[ok]) < BF16_TOL
 
 
+@pytest.mark.parametrize("variant,dtype,fp8,N", [
+    ("gelu_tanh", torch.bfloat16, False, 344064),   # biased tiles: the bias buffers are staged across a table rewrite
+    ("swiglu", torch.float16, True, 172032),        # fp8 weights: so are the scale buffers
+])
+def test_rewritten_tile_table_other_kernels(dev, variant, dtype, fp8, N):
+    """The other instantiations that rewrite their tile table (more than 64 tiles
+    per workgroup): every token bit-identical to the same block run on chunks
+    that need no rewrite."""
+    D = 384
+    p = O.make_block_params(D, 8, 2, 4, 2, seed=12, dtype=dtype, variant=variant)
+    if variant == "gelu_tanh":
+        g = _gen(13)
+        for e in list(p.experts) + [p.shared]:
+            e.fc1_b = (torch.randn(e.fc1_b.shape, generator=g) * 0.1).to(dtype)
+            e.fc2_b = (torch.randn(e.fc2_b.shape, generator=g) * 0.1).to(dtype)
+    blk = block_from_params(p, D, variant, dtype, dev)
+    if fp8:
+        blk.quantize_fp8()
+    x = torch.randn(1, N, D, generator=torch.Generator(device=dev).manual_seed(14), device=dev).to(dtype)
+    y = blk(x)
+    chunk = N // 8
+    parts = torch.cat([blk(x[:, i:i + chunk]) for i in range(0, N, chunk)], dim=1)
+    assert torch.equal(parts, y)
+    assert torch.isfinite(y.float()).all() and float(y.float().abs().max()) > 0
+
+
 def test_block_c3_zipf_load(dev):
     """16384 tokens, router bias = log Zipf(1.2): heavy imbalance in the grouped GEMM."""
     D, E = 1152, 8
