@@ -281,6 +281,29 @@ def cpu_baseline(variant, budget_s=20.0):
                       f"{sum(times):.1f} s of CPU work"}
 
 
+def time_vendor_gemm(blk, x, dev):
+    """What the vendor's GEMM (torch.matmul -> hipBLASLt) reaches on this board, which is power-limited for
+    bf16 matrix work so that throughput depends on the operand values: the routed fc1 as ONE plain GEMM
+    ([N*k, D] x [2I, D]^T, no activation, no gather, no shared expert) on this run's activations and the first
+    expert's weights, and an 8192^3 GEMM on N(0,1) operands.  A reference for `roofline.achieved`, not a part
+    of the layer."""
+    def run(a, b, reps=20):
+        c = torch.empty(a.shape[0], b.shape[0], dtype=a.dtype, device=dev)
+        for _ in range(3):
+            torch.matmul(a, b.t(), out=c)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            torch.matmul(a, b.t(), out=c)
+        torch.cuda.synchronize()
+        return 2.0 * a.shape[0] * b.shape[0] * a.shape[1] / ((time.perf_counter() - t0) / reps) / 1e12
+    a = x.repeat(TOPK, 1)
+    w1 = blk._packed.w1[0]
+    big = torch.randn(8192, 8192, device=dev).to(x.dtype)
+    return {"routed_fc1_shape_%dx%dx%d" % (a.shape[0], w1.shape[0], a.shape[1]): run(a, w1),
+            "8192x8192x8192_randn": run(big, big)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -294,6 +317,8 @@ def main():
     ap.add_argument("--no-caller", action="store_true", help="skip the fused-caller (LayerNorm/modulate + residual) pass")
     ap.add_argument("--no-staleness", action="store_true", help="skip the 50-step conditional-communication loop")
     ap.add_argument("--no-lagged", action="store_true", help="skip the step-lagged (displaced / interweaved) pass")
+    ap.add_argument("--no-vendor", action="store_true",
+                    help="skip the vendor-GEMM reference (torch.matmul on the routed fc1 shape with the same operands)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a known-size kernel to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
@@ -379,6 +404,8 @@ def main():
         out["step_lag_ms_per_layer_call"] = {
             "displaced": time_lagged(args.variant, dev, x, args.steps, args.warmup, False),
             "interweaved": time_lagged(args.variant, dev, x, args.steps, args.warmup, True)}
+    if not args.no_vendor:
+        out["vendor_gemm_tflops"] = time_vendor_gemm(blk, x, dev)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.variant)
     print(json.dumps(out))
