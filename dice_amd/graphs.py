@@ -69,6 +69,10 @@ class GraphedBlock:
         torch.cuda.synchronize(device)
         with torch.cuda.graph(self.graph, stream=side):
             self._call()
+        # The recorded launches hold raw addresses: the workspace and the packed weights they name stay
+        # alive with this object even if the block later sizes a larger workspace or repacks its weights
+        # (a replay then still computes with what was recorded).
+        self._recorded_buffers = (block._ws, block._packed)
 
     def _call(self):
         cache_in = self.cache if self.mode == MODE_SKIP else None

@@ -45,6 +45,25 @@ def test_graph_replays_match_eager(dev, D, N, dtype, variant):
         first = got.clone() if i == 0 else first
 
 
+def test_graph_survives_a_larger_eager_call(dev):
+    """An eager call on more tokens makes the block size a new workspace; the
+    recorded graph keeps the one it was recorded with."""
+    from dice_amd.graphs import GraphedBlock
+    D, N, dtype = 384, 512, torch.bfloat16
+    p = O.make_block_params(D, 8, 2, 4, 2, seed=25, dtype=dtype)
+    blk = block_from_params(p, D, "swiglu", dtype, dev)
+    graphed = GraphedBlock(blk, N)
+    x = torch.randn(N, D, generator=_gen(70)).to(dtype).to(dev)
+    want = blk.run(x).clone()
+    big = torch.randn(8 * N, D, generator=_gen(71)).to(dtype).to(dev)
+    blk.run(big)                                    # new, larger workspace
+    junk = [torch.full((1 << 20,), 7, dtype=torch.uint8, device=dev) for _ in range(8)]  # reuse freed memory, if any
+    got = graphed(x)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    assert all(int(j.min()) == 7 and int(j.max()) == 7 for j in junk)
+
+
 def test_graph_of_staleness_steps(dev):
     """A full step that fills the skip cache and a skip step that reads it, one
     graph each, alternating as the reference's schedule does."""
