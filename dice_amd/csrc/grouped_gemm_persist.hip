@@ -133,7 +133,7 @@ struct Tile {
   int steps;                 // pipeline steps (k / step extent)
   bool valid;
   const int32_t *a_rows;     // gathered tiles: slot of the tile's first row (else NULL)
-  uint32_t a_magic;          // gathered tiles: source row = mulhi(slot, a_magic) (= slot / a_div)
+  uint32_t a_magic;          // gathered tiles: source row = mulhi(slot, a_magic) (= slot / a_div); 0: a_div == 1
   int rows;                  // rows of the tile that belong to its group
 };
 
@@ -1016,7 +1016,10 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
         uint32_t off = ld_voff_a + (uint32_t)(32 * i) * t.a_pitch;
         if (t.a_rows) {
           const uint32_t slot = (uint32_t)lds_row_slots[r];
-          off = r < t.rows ? __umulhi(slot, W8 ? w8_magic : t.a_magic) * t.a_pitch + cp_chunk * 16 : kOutOfRange;
+          // (one slot per source row: 2^32 / 1 does not fit the multiplier, which then reads 0)
+          const uint32_t magic = W8 ? w8_magic : t.a_magic;
+          const uint32_t src_row = magic ? __umulhi(slot, magic) : slot;
+          off = r < t.rows ? src_row * t.a_pitch + cp_chunk * 16 : kOutOfRange;
         }
         ld_voff_rows[i] = off;
         asm volatile("" : "+v"(ld_voff_rows[i]));

@@ -547,6 +547,8 @@ def test_block_c1_fp32(dev, variant):
     (1000, 1024, 16, 2, torch.bfloat16),   # DiT-L width
     (333, 1408, 16, 2, torch.bfloat16),    # DiT-G width (11 x 128)
     (130, 384, 8, 1, torch.float32),       # top-1
+    (300, 768, 8, 1, torch.bfloat16),      # top-1 on the kernels that address rows through the permutation
+    (300, 512, 4, 4, torch.float16),       # top-4 likewise
     (130, 384, 8, 4, torch.float32),       # top-4
     (64, 384, 64, 2, torch.float32),       # as many experts as the layer call takes
 ])
