@@ -230,3 +230,16 @@ def test_forced_sync_schedule():
     assert not diep.ep_forced_sync(47, 50, ep_async_warm_up=2)
     assert diep.ep_forced_sync(40, 50, strided_sync=10)
     assert diep.ep_forced_sync(2, 50, strided_sync=100, ep_async_cool_down=3)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asked for more (or started under a multi-rank
+    launcher) it says so and exits before touching a device."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for argv, env in ((["--gpus", "2"], {}), ([], {"WORLD_SIZE": "2"})):
+        r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), *argv], capture_output=True, text=True,
+                           env={**os.environ, **env}, timeout=300)
+        assert r.returncode == 2
+        assert "one GPU" in r.stderr and r.stdout.strip() == ""
