@@ -243,3 +243,40 @@ def test_bench_refuses_more_than_one_gpu():
                            env={**os.environ, **env}, timeout=300)
         assert r.returncode == 2
         assert "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_header_is_plain_c_and_links(tmp_path):
+    """include/dice_moe.h compiles as strict C99 and a C program links against
+    the library: the boundary is usable from any language with a C FFI.  The
+    program only makes calls that are answered before a device is touched."""
+    import shutil
+    import subprocess
+    from dice_amd import lib
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = tmp_path / "abi.c"
+    src.write_text(r'''
+#include "dice_moe.h"
+#include <stdio.h>
+int main(void) {
+  dice_moe_layer_t layer = {0};
+  dice_moe_lag_entry_t entry = {0};
+  dice_moe_caller_t caller = {0};
+  (void)entry; (void)caller;
+  if (dice_abi_version() < 1) return 10;
+  if (dice_moe_workspace_bytes(&layer, 8) == 0) return 11;
+  if (dice_gate_topk(0, DICE_BF16, 0, DICE_BF16, 0, 8, 64, 8, 2, 0, 0, 0, 0, 0, 0) != DICE_ERR_BAD_ARG) return 12;
+  printf("%s\n", dice_last_error());
+  return 0;
+}
+''')
+    exe = tmp_path / "abi"
+    libdir = os.path.dirname(lib.LIB_PATH)
+    cc = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(root, "include"),
+                         str(src), "-o", str(exe), "-L", libdir, "-ldice_moe", f"-Wl,-rpath,{libdir}"],
+                        capture_output=True, text=True)
+    assert cc.returncode == 0, cc.stderr
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0, (run.returncode, run.stderr)
+    assert "null pointer" in run.stdout
