@@ -374,10 +374,14 @@ def main():
     # fused), timed inside the timed region above.
     dom_flops = flops["fc1"] + flops["shared_fc1"]
     ach = dom_flops / (fc1_ms * 1e-3) / 1e12
+    swiglu = args.variant == "swiglu"
     out["roofline"] = {"bound": "mfma",
-                       "kernel": "gemm_persist_kernel4<fc1 SwiGLU> (routed + shared expert fc1, activation fused)",
+                       "kernel": "gemm_persist_kernel4<fc1 %s> (routed + shared expert fc1, activation fused)"
+                                 % ("SwiGLU" if swiglu else "GELU-tanh, biased"),
                        "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                       "frac": ach / PEAK_BF16_TFLOPS, "traffic": FC1_HBM_TRAFFIC_BYTES,
+                       "frac": ach / PEAK_BF16_TFLOPS,
+                       # counters were collected for the reference (SwiGLU) expert only
+                       "traffic": FC1_HBM_TRAFFIC_BYTES if swiglu else None,
                        "flop_per_launch": dom_flops, "ms_per_launch": fc1_ms}
     if not args.no_stages:
         # every launch of the layer, in a second pass of back-to-back calls
