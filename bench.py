@@ -410,6 +410,16 @@ def main():
             "interweaved": time_lagged(args.variant, dev, x, args.steps, args.warmup, True)}
     if not args.no_vendor:
         out["vendor_gemm_tflops"] = time_vendor_gemm(blk, x, dev)
+        # The same launches with every expert weight zero (same instructions, addresses and traffic): how far the
+        # board's power limit, which depends on the operand values, sets the time of the dominant kernel.
+        zero = make_block(args.variant, dev)
+        zero.pack_weights()
+        for t in (zero._packed.w1, zero._packed.w2, zero._packed.sw1, zero._packed.sw2):
+            if t is not None:
+                t.zero_()
+        _, zero_fc1_ms = time_layer(zero, x, args.steps, args.warmup)
+        out["roofline"]["ms_per_launch_zero_weights"] = zero_fc1_ms
+        del zero
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.variant)
     print(json.dumps(out))
