@@ -12,6 +12,8 @@
 // group is therefore (span, round, lane) = ascending slot index: stable and
 // independent of any atomic's timing.  Integer/byte work, HBM traffic is
 // 4 B read + 8 B written per slot.
+#include <mutex>
+
 #include "common.h"
 
 namespace dice {
@@ -456,6 +458,69 @@ extern "C" int dice_dispatch(const int32_t *flat_idx, const uint8_t *skip_mask, 
                              void *stream) {
   return dice::dispatch_impl(flat_idx, skip_mask, n_slots, n_experts, counts, offsets, perm, inv_perm,
                              workspace, workspace_bytes, nullptr, 0, stream);
+}
+
+// dice_dispatch for callers that cannot allocate: the per-span histogram table
+// lives in a file-scope device array instead of a caller-provided workspace.
+// Every GPU the library runs on holds its own copy of the array at its own
+// address; the array's name is only a host-side handle, so the device address
+// is looked up once per device and that pointer is what the kernels get.
+namespace dice {
+namespace {
+constexpr size_t kStaticScratchBytes = DICE_DISPATCH_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_lock;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (NULL + error text on failure).
+void *static_scratch(int *rc) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    *rc = fail(DICE_ERR_LAUNCH, "dice_dispatch_static: hipGetDevice: %s (device %d)",
+               hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  if (!g_scratch_ptr[dev]) {
+    void *ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      *rc = fail(DICE_ERR_LAUNCH, "dice_dispatch_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  *rc = DICE_OK;
+  return g_scratch_ptr[dev];
+}
+}  // namespace
+}  // namespace dice
+
+extern "C" size_t dice_dispatch_static_scratch_bytes(void) { return dice::kStaticScratchBytes; }
+
+extern "C" int dice_dispatch_static(const int32_t *flat_idx, const uint8_t *skip_mask, int64_t n_slots,
+                                    int n_experts, int32_t *counts, int32_t *offsets, int32_t *perm,
+                                    int32_t *inv_perm, void *stream) {
+  using namespace dice;
+  DICE_REQUIRE(n_experts >= 1 && n_experts <= kMaxExperts, DICE_ERR_UNSUPPORTED,
+               "dice_dispatch_static: n_experts %d outside [1, %d]", n_experts, kMaxExperts);
+  DICE_REQUIRE(n_slots >= 0 && n_slots < (1ll << 31), DICE_ERR_BAD_ARG,
+               "dice_dispatch_static: n_slots %lld outside [0, 2^31)", (long long)n_slots);
+  const size_t need = dice_dispatch_workspace_bytes(n_slots, n_experts);
+  DICE_REQUIRE(need <= kStaticScratchBytes, DICE_ERR_WORKSPACE,
+               "dice_dispatch_static: %lld slots x %d experts need %zu bytes of scratch, the static array "
+               "holds %zu (use dice_dispatch with a workspace)",
+               (long long)n_slots, n_experts, need, kStaticScratchBytes);
+  int rc = DICE_OK;
+  void *ptr = static_scratch(&rc);
+  if (!ptr) return rc;
+  // Every table entry a launch reads was written by the same call's count
+  // kernel, so nothing has to be cleared between calls.
+  return dispatch_impl(flat_idx, skip_mask, n_slots, n_experts, counts, offsets, perm, inv_perm, ptr,
+                       kStaticScratchBytes, nullptr, 0, stream);
 }
 
 namespace dice {

@@ -32,6 +32,8 @@ EXPORTS = [
     "dice_gate_topk",
     "dice_dispatch_workspace_bytes",
     "dice_dispatch",
+    "dice_dispatch_static_scratch_bytes",
+    "dice_dispatch_static",
     "dice_gather_rows",
     "dice_grouped_mlp",
     "dice_grouped_mlp_stage",
@@ -109,6 +111,11 @@ def load() -> ctypes.CDLL:
     lib.dice_dispatch.restype = c_int
     lib.dice_dispatch.argtypes = [c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_size_t, c_void_p]
+    lib.dice_dispatch_static_scratch_bytes.restype = c_size_t
+    lib.dice_dispatch_static_scratch_bytes.argtypes = []
+    lib.dice_dispatch_static.restype = c_int
+    lib.dice_dispatch_static.argtypes = [c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p,
+                                         c_void_p, c_void_p]
     lib.dice_gather_rows.restype = c_int
     lib.dice_gather_rows.argtypes = [c_void_p, c_int, c_void_p, c_int, c_int64, c_int, c_void_p, c_void_p]
     lib.dice_grouped_mlp.restype = c_int

@@ -89,6 +89,27 @@ int dice_dispatch(const int32_t *flat_idx, const uint8_t *skip_mask,
                   void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * dice_dispatch without a workspace argument and without any allocation.  It
+ * has no counterpart in the reference; it is for callers that cannot allocate
+ * device memory around the call: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  The per-span histogram table that
+ * dice_dispatch keeps in `workspace` lives in a file-scope device array of
+ * DICE_DISPATCH_STATIC_SCRATCH_BYTES instead (one copy per GPU, held until the
+ * process ends; its device address is looked up once per device on the first
+ * call there).  Same outputs as dice_dispatch, bit for bit.  Sizes whose table
+ * exceeds the array (dice_dispatch_workspace_bytes(n_slots, n_experts) >
+ * DICE_DISPATCH_STATIC_SCRATCH_BYTES) are refused with DICE_ERR_WORKSPACE.
+ * All calls on one GPU share that GPU's array: calls that overlap in time on
+ * one GPU (different streams) race; calls on one stream are ordered.
+ */
+#define DICE_DISPATCH_STATIC_SCRATCH_BYTES (1u << 20)
+size_t dice_dispatch_static_scratch_bytes(void);
+int dice_dispatch_static(const int32_t *flat_idx, const uint8_t *skip_mask,
+                         int64_t n_slots, int n_experts, int32_t *counts,
+                         int32_t *offsets, int32_t *perm, int32_t *inv_perm,
+                         void *stream);
+
+/*
  * Row gather.  Replaces _local_dispatch (expertpara/ep_fwd.py:345-347) and
  * x[exp_token_idx] (models.py:373): out[r] = x[perm[r] / slots_per_token] for
  * r < n_rows with perm[r] >= 0.  The fused expert path below reads x through
