@@ -49,10 +49,29 @@ def find_model(model_name: str) -> Mapping[str, torch.Tensor]:
     checkpoint file to host memory and unwraps it.  Tensors only: the file is
     read with ``weights_only=True``.  The reference's download of the dense DiT
     weights (download.py:36-47) has no counterpart."""
+    import argparse
     import os
+    import pickle
     if not os.path.isfile(model_name):
         raise DiceError(f"Could not find DiT checkpoint at {model_name}")
-    checkpoint = torch.load(model_name, map_location="cpu", weights_only=True)
+    # The reference's training script stores its command-line arguments beside
+    # the weights ({"model", "ema", "opt", "args": argparse.Namespace},
+    # train.py:258-266).  A Namespace is a plain attribute bag whose
+    # reconstruction runs no code of the file's choosing, so it is the one class
+    # allowed on top of the tensors-only unpickler; anything else in a file is
+    # refused, with the name of what was refused.
+    try:
+        with torch.serialization.safe_globals([argparse.Namespace]):
+            checkpoint = torch.load(model_name, map_location="cpu", weights_only=True)
+    except pickle.UnpicklingError as e:
+        text = str(e)
+        m = re.search(r"Unsupported global: GLOBAL (\S+)", text) or re.search(r"Unsupported class (\S+)", text)
+        what = m.group(1) if m else text.splitlines()[0][:200]
+        raise DiceError(f"{model_name}: not a tensors-only checkpoint ({what}); this loader executes nothing "
+                        "from a checkpoint file and accepts tensors, containers, numbers, strings and "
+                        "argparse.Namespace only") from None
+    if not isinstance(checkpoint, Mapping):
+        raise DiceError(f"{model_name}: expected a state dict or a dict wrapping one, got {type(checkpoint).__name__}")
     return unwrap_checkpoint(checkpoint)
 
 

@@ -63,12 +63,15 @@ __global__ __launch_bounds__(256) void combine_kernel(
     const int64_t s = t * top_k + j;
     const float w = topk_weight[s];
     const bool skipped = skip_mask && skip_mask[s];
-    Pack<T> row;
+    Pack<T> row{};
     if (skipped && cache_in) {
       row = cache_in[t * vec_per_row + c];
     } else {
+      // A slot the dispatch left out (masked, or an expert id outside the
+      // table: inv_perm = -1) contributes a zero row, as the zero-initialised
+      // buffer of the reference's _local_combine does (ep_fwd.py:350-354).
       const int64_t src = inv_perm ? (int64_t)inv_perm[s] : s;
-      row = slot_out[src * vec_per_row + c];
+      if (src >= 0) row = slot_out[src * vec_per_row + c];
       if (skipped && cache_out) cache_out[t * vec_per_row + c] = row;
     }
 #pragma unroll

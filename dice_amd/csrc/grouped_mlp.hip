@@ -336,7 +336,6 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
   int32_t *idx = topk_idx_out ? topk_idx_out : w.topk_idx;
   float *wt = own.topk_weight;
 
-  g_timers.recorded = false;
   stamp(0, s);
   // With the caller's prologue the layer input is LN(x) modulated, written
   // straight into the entry that outlives the call when there is one; x itself

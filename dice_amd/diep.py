@@ -28,7 +28,8 @@ _noskip_interval = 1
 _enable_skip = False
 _skip_mode: Optional[str] = None
 _rand_mask: Optional[torch.Tensor] = None
-_mask_cache = {}
+_mask_cache = {}      # (mode, length) -> CPU bool mask
+_device_masks = {}    # (id of the CPU mask, device) -> (CPU mask, its uint8 device copy)
 
 
 class EPSkipCache:
@@ -73,7 +74,8 @@ class LagEntry:
     the skipped slot of every token, ``owner`` is the block whose experts the
     entry needs."""
 
-    __slots__ = ("x", "offsets", "perm", "inv_perm", "topk_weight", "rows", "max_rows", "dropped", "owner")
+    __slots__ = ("x", "offsets", "perm", "inv_perm", "topk_weight", "rows", "max_rows", "dropped", "owner",
+                 "_rows_buf")
 
     def __init__(self, x, n_experts: int, top_k: int, dropped: bool, owner=None, copy_x: bool = True):
         n = x.shape[0]
@@ -84,6 +86,7 @@ class LagEntry:
         self.inv_perm = torch.empty(n * top_k, dtype=torch.int32, device=dev)
         self.topk_weight = torch.empty(n * top_k, dtype=torch.float32, device=dev)
         self.rows = None
+        self._rows_buf = None
         self.max_rows = n * (top_k - 1) if dropped else n * top_k
         self.dropped = dropped
         self.owner = owner
@@ -96,15 +99,31 @@ class LagEntry:
         n = x.shape[0]
         e.x, e.offsets, e.perm, e.inv_perm, e.topk_weight = x, offsets, perm, inv_perm, topk_weight
         e.rows = None
+        e._rows_buf = None
         e.max_rows = n * (top_k - 1) if dropped else n * top_k
         e.dropped = dropped
         e.owner = owner
         return e
 
+    def recycle(self, top_k: int, dropped: bool, owner=None):
+        """Makes a retired entry ready for a new call.  The buffers stay;
+        ``rows`` reads as None again until the entry has been through the
+        experts, its memory is kept aside for ``ensure_rows``."""
+        n = self.x.shape[0]
+        self.max_rows = n * (top_k - 1) if dropped else n * top_k
+        self.dropped = dropped
+        self.owner = owner
+        if self.rows is not None:
+            self._rows_buf, self.rows = self.rows, None
+
     def ensure_rows(self):
         if self.rows is None:
-            self.rows = torch.empty((max(self.max_rows, 1), self.x.shape[-1]), dtype=self.x.dtype,
-                                    device=self.x.device)
+            buf, self._rows_buf = self._rows_buf, None
+            if buf is not None and buf.shape[0] >= max(self.max_rows, 1):
+                self.rows = buf
+            else:
+                self.rows = torch.empty((max(self.max_rows, 1), self.x.shape[-1]), dtype=self.x.dtype,
+                                        device=self.x.device)
         return self.rows
 
     def desc(self):
@@ -169,6 +188,7 @@ def ep_cache_init(cache_capacity, auto_gc=False, noskip_step=1, skip_mode=None,
     _diep_cache_combine = All2AllCache(cache_capacity)
     _diep_cache_skip = EPSkipCache(capacity=cache_capacity if _enable_skip else 0)
     _mask_cache.clear()
+    _device_masks.clear()
 
 
 def use_latest_expert_weights(val):
@@ -219,18 +239,30 @@ def layer_is_async(ep_async_mode, layer_idx, total_layers) -> bool:
     raise ValueError(f"Invalid ep_async_mode: {ep_async_mode}")
 
 
+# Per selective-async strategy: (distance to the previous lagged layer, number
+# of layers the lagged range wraps over as a fraction of all layers, first
+# layer of the range as a fraction of all layers).
+_LAG_RANGES = {
+    "all": (1, 1.0, 0.0),
+    "shallow": (1, 0.5, 0.0),
+    "deep": (1, 0.5, 0.5),
+    "interleaved": (2, 1.0, 0.0),
+}
+
+
 def _past_layer_key(key):
-    """Reference diep.py:184-194: the lagged layer that ran before ``key``."""
-    total_layers = _diep_cache_dispatch.capacity
-    if _selective_async_strategy == "all":
-        return (key - 1) % total_layers
-    if _selective_async_strategy == "shallow":
-        return (key - 1) % (total_layers // 2)
-    if _selective_async_strategy == "deep":
-        return (key - 1) % (total_layers // 2) + total_layers // 2
-    if _selective_async_strategy == "interleaved":
-        return (key - 2) % total_layers
-    raise ValueError(f"Unknown selective async strategy: {_selective_async_strategy}")
+    """The lagged layer that ran before layer ``key`` (reference
+    diep.py:184-194), wrapping from the first lagged layer to the last one of
+    the previous step."""
+    try:
+        back, span_frac, first_frac = _LAG_RANGES[_selective_async_strategy]
+    except KeyError:
+        raise ValueError(f"Unknown selective async strategy: {_selective_async_strategy}") from None
+    layers = _diep_cache_dispatch.capacity
+    half = layers // 2
+    span = layers if span_frac == 1.0 else half
+    first = half if first_frac else 0
+    return (key - back) % span + first
 
 
 def lag_roles(cache_key: int, new_entry: LagEntry):
@@ -264,6 +296,11 @@ def lag_roles(cache_key: int, new_entry: LagEntry):
     return work, emit
 
 
+def lag_entry_cached(entry) -> bool:
+    """Whether ``entry`` still sits in the dispatch or the combine cache."""
+    return any(e is entry for cache in (_diep_cache_dispatch, _diep_cache_combine) for e in cache.cache)
+
+
 def ep_get_max_mem():
     return max_mem
 
@@ -284,36 +321,64 @@ def ep_skip_now(idx):
     return _step % _noskip_interval != 0
 
 
+def _draw_rand_mask(length):
+    """One masked slot per token pair, drawn with the CPU generator exactly as
+    the reference draws it (one ``randint(0, 2, (pairs,))`` call, diep.py:80-88),
+    so a seeded process gets the reference's mask."""
+    pick = torch.randint(0, 2, (length // 2,))
+    return torch.stack((pick == 0, pick == 1), dim=1).reshape(-1)
+
+
 def ep_skip_mask(length):
     """Bool mask over flat slots, one True per token pair (reference
     diep.py:72-90): 'high' = slot 0, 'low' = slot 1, 'rand' = one random slot
-    per pair drawn once per process and reused."""
+    per pair drawn once per process and reused.  A 'rand' mask drawn for
+    another length is an error here (the reference fails later, on the shape
+    of the indexing it does with it)."""
     global _rand_mask
     if _skip_mode in ("high", "low"):
         key = (_skip_mode, length)
-        if key not in _mask_cache:
+        mask = _mask_cache.get(key)
+        if mask is None:
             mask = torch.zeros(length, dtype=torch.bool)
-            if _skip_mode == "high":
-                mask[::2] = True
-            else:
-                mask[1::2] = True
+            mask[(0 if _skip_mode == "high" else 1)::2] = True
             _mask_cache[key] = mask
-        return _mask_cache[key]
+        return mask
     if _skip_mode == "rand":
         if _rand_mask is None:
-            n = length // 2
-            bool_tensor = torch.zeros((n, 2), dtype=torch.bool)
-            random_indices = torch.randint(0, 2, (n,))
-            bool_tensor[torch.arange(n), random_indices] = True
-            _rand_mask = bool_tensor.view(-1)
+            _rand_mask = _draw_rand_mask(length)
+        if _rand_mask.numel() != length:
+            from .lib import DiceError
+            raise DiceError(f"the 'rand' skip mask was drawn for {_rand_mask.numel()} slots, this call has {length}: "
+                            "the batch changed; install a new mask with ep_set_rand_mask(None)")
         return _rand_mask
     raise ValueError(f"Unknown skip mode: {_skip_mode}")
+
+
+def mask_on_device(mask, device):
+    """``mask`` (a CPU bool tensor from ``ep_skip_mask``) as a uint8 tensor on
+    ``device``.  The host policy hands out the same mask object for every layer
+    and step, so the copy is made once per (mask, device) and not per layer call."""
+    key = (id(mask), str(device))
+    hit = _device_masks.get(key)
+    if hit is None or hit[0] is not mask:
+        if len(_device_masks) > 16:
+            _device_masks.clear()
+        hit = (mask, mask.to(device).view(torch.uint8))
+        _device_masks[key] = hit
+    return hit[1]
+
+
+def ep_skip_mask_on(length, device):
+    """``ep_skip_mask(length)`` as a uint8 tensor on ``device``."""
+    return mask_on_device(ep_skip_mask(length), device)
 
 
 def ep_set_rand_mask(mask: Optional[torch.Tensor]):
     """Extension: installs (or clears) the 'rand' mask so runs are reproducible."""
     global _rand_mask
     _rand_mask = mask
+    _device_masks.clear()
 
 
 def ep_cache_clear():

@@ -61,8 +61,11 @@ def moe_infer_ep(inp, experts, flat_expert_indices, flat_expert_weights, num_exp
     idx = flat_expert_indices.to(torch.int32).contiguous()
     mask = None
     if partial_skip:
-        mask = skip_mask.to(x.device)
-        mask = mask.view(torch.uint8) if mask.dtype == torch.bool else mask
+        if skip_mask.numel() != n * k:
+            raise DiceError(f"moe_infer_ep: skip mask of {skip_mask.numel()} entries for {n} tokens x {k}")
+        if skip_mask.device != x.device:        # the reference's mask is a CPU tensor (diep.py:72-90)
+            skip_mask = diep.mask_on_device(skip_mask, x.device)
+        mask = skip_mask.view(torch.uint8) if skip_mask.dtype == torch.bool else skip_mask
     _, offsets, perm, inv_perm = ops.dispatch(idx, n_experts, mask if skip_now else None)
     weights = flat_expert_weights.reshape(-1).float().contiguous()
     new = diep.LagEntry.from_tables(x.clone() if async_op else x, offsets, perm, inv_perm, weights, k,
@@ -91,6 +94,9 @@ def moe_infer_ep(inp, experts, flat_expert_indices, flat_expert_weights, num_exp
             cache_in = diep.ep_skip_get(cache_key)
             if cache_in is None:
                 raise DiceError("moe_infer_ep: the skip cache holds nothing for the dropped slots")
+            if cache_in.shape != x.shape or cache_in.dtype != x.dtype or cache_in.device != x.device:
+                raise DiceError(f"moe_infer_ep: the skip cache holds {tuple(cache_in.shape)} {cache_in.dtype}, this call "
+                                f"has {tuple(x.shape)} {x.dtype}: clear the caches when the batch changes")
         else:                                                # :186-188
             cache_out = torch.empty_like(x)
     scale = weights if (diep.latest_expert_weights() or emit is new) else emit.topk_weight

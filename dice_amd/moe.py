@@ -93,15 +93,48 @@ class MoeMLP(nn.Module):
         self.up_proj = nn.Linear(hidden_size, intermediate_size, bias=False)
         self.down_proj = nn.Linear(intermediate_size, hidden_size, bias=False)
         self.pretraining_tp = pretraining_tp
+        self._w1 = self._w2 = None      # [1, 2I, D] / [1, D, I] storage the three parameters are views of
+        self._row_range = {}            # (rows, device) -> int32 [0, rows] on the device
+
+    def _apply(self, fn, *args, **kwargs):
+        self._w1 = self._w2 = None
+        self._row_range = {}
+        return super()._apply(fn, *args, **kwargs)
+
+    def adopt_packed(self, w1, w2):
+        """Re-points the three parameters at ``w1 [1, 2I, D]`` = rows
+        ``[gate_proj; up_proj]`` and ``w2 [1, D, I]`` (slices of a block's
+        packed storage, or this expert's own), so the weights exist once and
+        ``forward`` needs no concatenation."""
+        inter = self.intermediate_size
+        self.gate_proj.weight.data = w1[0, :inter]
+        self.up_proj.weight.data = w1[0, inter:]
+        self.down_proj.weight.data = w2[0]
+        self._w1, self._w2 = w1, w2
+
+    def _packed_views(self):
+        w = self.gate_proj.weight
+        ok = (self._w1 is not None and self._w1.data_ptr() == w.data_ptr() and self._w1.dtype == w.dtype
+              and self._w2.data_ptr() == self.down_proj.weight.data_ptr()
+              and self.up_proj.weight.data_ptr() == w.data_ptr() + w.numel() * w.element_size())
+        if not ok:
+            w1 = torch.cat([self.gate_proj.weight, self.up_proj.weight], 0).unsqueeze(0).contiguous()
+            w2 = self.down_proj.weight.detach().unsqueeze(0).contiguous()
+            self.adopt_packed(w1, w2)
+        return self._w1, self._w2
 
     @torch.no_grad()
     def forward(self, x):
         shape = x.shape
         x2 = x.reshape(-1, shape[-1]).contiguous()
         n = x2.shape[0]
-        w1 = torch.cat([self.gate_proj.weight, self.up_proj.weight], 0).unsqueeze(0).contiguous()
-        w2 = self.down_proj.weight.unsqueeze(0).contiguous()
-        offsets = torch.tensor([0, n], dtype=torch.int32, device=x.device)
+        w1, w2 = self._packed_views()
+        key = (n, str(x.device))
+        offsets = self._row_range.get(key)
+        if offsets is None:
+            if len(self._row_range) > 64:
+                self._row_range.clear()
+            offsets = self._row_range[key] = torch.tensor([0, n], dtype=torch.int32, device=x.device)
         out = ops.grouped_mlp(x2, None, 1, offsets, n, w1, w2, "swiglu")
         return out.view(shape)
 
@@ -165,6 +198,8 @@ class SparseMoeBlock(nn.Module):
         self._fp8 = False
         self._desc = None
         self._ws = None
+        self._spare_cache = None     # a skip-cache tensor a skip step has consumed: the next full step writes into it
+        self._spare_entries = []     # step-lag entries that have left both caches, for re-use
 
     # ------------------------------------------------------------------ #
     # weight packing
@@ -173,6 +208,8 @@ class SparseMoeBlock(nn.Module):
         self._packed = None
         self._desc = None
         self._ws = None
+        self._spare_cache = None
+        self._spare_entries = []
         return super()._apply(fn, *args, **kwargs)
 
     def load_state_dict(self, *args, **kwargs):
@@ -192,19 +229,13 @@ class SparseMoeBlock(nn.Module):
         if self.variant == "swiglu":
             p.w1 = torch.stack([torch.cat([e.gate_proj.weight, e.up_proj.weight], 0) for e in ex]).contiguous()
             p.w2 = torch.stack([e.down_proj.weight for e in ex]).contiguous()
-            inter = self.inter
             for i, e in enumerate(ex):
-                e.gate_proj.weight.data = p.w1[i, :inter]
-                e.up_proj.weight.data = p.w1[i, inter:]
-                e.down_proj.weight.data = p.w2[i]
+                e.adopt_packed(p.w1[i:i + 1], p.w2[i:i + 1])
             if self.n_shared_experts is not None:
                 s = self.shared_experts
                 p.sw1 = torch.cat([s.gate_proj.weight, s.up_proj.weight], 0).unsqueeze(0).contiguous()
                 p.sw2 = s.down_proj.weight.data.unsqueeze(0).contiguous()
-                si = s.intermediate_size
-                s.gate_proj.weight.data = p.sw1[0, :si]
-                s.up_proj.weight.data = p.sw1[0, si:]
-                s.down_proj.weight.data = p.sw2[0]
+                s.adopt_packed(p.sw1, p.sw2)
         else:
             p.w1 = torch.stack([e.fc1.weight for e in ex]).contiguous()
             p.w2 = torch.stack([e.fc2.weight for e in ex]).contiguous()
@@ -326,7 +357,7 @@ class SparseMoeBlock(nn.Module):
             self.para_mode.ep_async_mode, self.layer_idx, self.total_layers)
         mask, skip_now = None, None
         if diep.ep_skip_enabled():
-            mask = diep.ep_skip_mask(x.shape[0] * self.num_experts_per_tok).to(x.device)
+            mask = diep.ep_skip_mask_on(x.shape[0] * self.num_experts_per_tok, x.device)
             skip_now = diep.ep_skip_now(self.layer_idx)
         if async_op:
             return self._run_lagged(x, mask, skip_now, caller=caller, y=y).view(*orig_shape)
@@ -336,12 +367,40 @@ class SparseMoeBlock(nn.Module):
             if skip_now:
                 mode, cache_in = MODE_SKIP, diep.ep_skip_get(self.layer_idx)
             else:
-                mode = MODE_PUT
-                cache_out = torch.empty_like(x)
+                mode, cache_out = MODE_PUT, self._cache_buffer(x)
         y = self.run(x, mode, mask, cache_in, cache_out, y=y, caller=caller)
         if mode == MODE_PUT:
             diep.ep_skip_put(self.layer_idx, cache_out)
+        elif mode == MODE_SKIP:
+            self._spare_cache = cache_in      # consumed (the cache entry is empty now): the next full step refills it
         return y.view(*orig_shape)
+
+    def _cache_buffer(self, x):
+        """Where a full step writes the skip cache: the tensor the last skip
+        step consumed when it still fits, else a new one.  Everything runs on
+        one stream, so the skip step's read is over before the refill starts."""
+        spare, self._spare_cache = self._spare_cache, None
+        if spare is not None and spare.shape == x.shape and spare.dtype == x.dtype and spare.device == x.device:
+            return spare
+        return torch.empty_like(x)
+
+    def _check_skip_args(self, x, mode, skip_mask, cache_in, cache_out):
+        """The kernels index the mask by slot and the cache by token row of THIS
+        call; a mask or cache of another batch would be read out of bounds."""
+        n, k = x.shape[0], self.num_experts_per_tok
+        if mode != MODE_PLAIN and skip_mask is None:
+            raise DiceError("a put or skip step needs the skip mask")
+        if skip_mask is not None and (skip_mask.numel() != n * k or skip_mask.device != x.device
+                                      or skip_mask.dtype not in (torch.uint8, torch.bool)):
+            raise DiceError(f"skip mask: {skip_mask.numel()} entries of {skip_mask.dtype} on {skip_mask.device}, "
+                            f"this call needs {n * k} bool / uint8 entries on {x.device}")
+        for name, c, wanted in (("cache_in", cache_in, mode == MODE_SKIP), ("cache_out", cache_out, mode == MODE_PUT)):
+            if wanted and c is None:
+                raise DiceError(f"layer {self.layer_idx}: this step needs {name}")
+            if c is not None and (c.shape != x.shape or c.dtype != x.dtype or c.device != x.device):
+                raise DiceError(f"layer {self.layer_idx}: {name} is {tuple(c.shape)} {c.dtype} on {c.device}, the "
+                                f"layer input {tuple(x.shape)} {x.dtype} on {x.device}: the batch changed since the "
+                                "cache was filled; call ep_cache_clear() and run a full step")
 
     @torch.no_grad()
     def _run_lagged(self, x, mask, skip_now, topk_idx_out=None, topk_weight_out=None, caller=None, y=None):
@@ -354,7 +413,7 @@ class SparseMoeBlock(nn.Module):
         desc = self._ensure(x)
         n = x.shape[0]
         ws = self._workspace(desc, n, x.device)
-        new = diep.LagEntry(x, len(self.experts), self.num_experts_per_tok, bool(skip_now), owner=self)
+        new = self._take_entry(x, bool(skip_now))
         work, emit = diep.lag_roles(self.layer_idx, new)
         for entry in (work, emit):
             if entry.x.shape != x.shape or entry.x.dtype != x.dtype or entry.x.device != x.device:
@@ -372,9 +431,10 @@ class SparseMoeBlock(nn.Module):
                     raise DiceError(f"layer {self.layer_idx}: a step dispatched without its skipped slots "
                                     "came back but the skip cache is empty")
             else:
-                mode, cache_out = MODE_PUT, torch.empty_like(x)
+                mode, cache_out = MODE_PUT, self._cache_buffer(x)
             if mask.dtype == torch.bool:
                 mask = mask.view(torch.uint8)
+        self._check_skip_args(x, mode, mask, cache_in, cache_out)
         owner = work.owner if work.owner is not None else self
         experts_of = owner._ensure(x)
         put_d, work_d, emit_d = new.desc(), work.desc(), emit.desc()
@@ -388,7 +448,27 @@ class SparseMoeBlock(nn.Module):
             ptr(topk_idx_out), ptr(topk_weight_out), ptr(ws), ws.numel(), stream_ptr()))
         if mode == MODE_PUT:
             diep.ep_skip_put(self.layer_idx, cache_out)
+        elif mode == MODE_SKIP:
+            self._spare_cache = cache_in
+        if emit is not work and emit is not new and not diep.lag_entry_cached(emit):
+            # The returned entry has left both caches: its buffers serve a later call of the
+            # block that made it (work queued on the one stream is ordered before any re-use).
+            home = emit.owner if emit.owner is not None else self
+            if len(home._spare_entries) < 2:
+                home._spare_entries.append(emit)
         return y
+
+    def _take_entry(self, x, dropped: bool):
+        """A step-lag entry for this call: a retired one of the same shape when
+        there is one (its seven buffers are re-used), else a new one."""
+        k = self.num_experts_per_tok
+        while self._spare_entries:
+            e = self._spare_entries.pop()
+            if (e.x.shape == x.shape and e.x.dtype == x.dtype and e.x.device == x.device
+                    and e.perm.numel() == x.shape[0] * k and e.offsets.numel() == len(self.experts) + 1):
+                e.recycle(k, dropped, self)
+                return e
+        return diep.LagEntry(x, len(self.experts), k, dropped, owner=self)
 
     @torch.no_grad()
     def run(self, x, mode=MODE_PLAIN, skip_mask=None, cache_in=None, cache_out=None,
@@ -398,6 +478,7 @@ class SparseMoeBlock(nn.Module):
         along: ``x`` is then the residual stream)."""
         desc = self._ensure(x)
         n = x.shape[0]
+        self._check_skip_args(x, mode, skip_mask, cache_in, cache_out)
         ws = self._workspace(desc, n, x.device)
         if y is None:
             y = torch.empty_like(x)
@@ -422,7 +503,10 @@ class SparseMoeBlock(nn.Module):
         p = self._packed
         k = self.num_experts_per_tok
         n = x.shape[0]
-        idx = flat_expert_indices.to(torch.int32).contiguous()
+        if flat_expert_indices.numel() != n * k or flat_expert_weights.numel() != n * k:
+            raise DiceError(f"moe_infer: {flat_expert_indices.numel()} indices and {flat_expert_weights.numel()} "
+                            f"weights for {n} tokens x {k}")
+        idx = flat_expert_indices.reshape(-1).to(torch.int32).contiguous()
         _, offsets, perm, inv_perm = ops.dispatch(idx, len(self.experts))
         rows = ops.grouped_mlp(x.contiguous(), perm, k, offsets, n * k, p.w1, p.w2, self.variant,
                                p.b1, p.b2, p.w1_scale, p.w2_scale, scatter_to_slots=False)

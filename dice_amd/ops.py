@@ -38,23 +38,40 @@ def gate_topk(x: torch.Tensor, weight: torch.Tensor, top_k: int, norm_topk_prob:
     return idx, wt, logits, idx64
 
 
-def dispatch(flat_idx: torch.Tensor, n_experts: int, skip_mask: Optional[torch.Tensor] = None):
+def dispatch(flat_idx: torch.Tensor, n_experts: int, skip_mask: Optional[torch.Tensor] = None,
+             out=None, static_scratch: bool = False):
     """Dispatch tables (reference models.py:365-367, ep_fwd.py:57-76,100-106).
 
     ``flat_idx`` int32 [S]; ``skip_mask`` uint8/bool [S] marks dropped slots.
-    Returns ``(counts [E], offsets [E+1], perm [S], inv_perm [S])`` int32."""
+    Returns ``(counts [E], offsets [E+1], perm [S], inv_perm [S])`` int32;
+    ``out`` may bring these four tensors along.  ``static_scratch`` takes the
+    entry point that keeps its histogram table in the library's own device
+    array and allocates nothing (given ``out``, neither does this wrapper)."""
     if flat_idx.dtype != torch.int32:
         raise _l.DiceError("dispatch needs int32 expert indices")
     s = flat_idx.numel()
     dev = flat_idx.device
-    counts = torch.empty(n_experts, dtype=torch.int32, device=dev)
-    offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=dev)
-    perm = torch.empty(s, dtype=torch.int32, device=dev)
-    inv_perm = torch.empty(s, dtype=torch.int32, device=dev)
+    if out is None:
+        counts = torch.empty(n_experts, dtype=torch.int32, device=dev)
+        offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=dev)
+        perm = torch.empty(s, dtype=torch.int32, device=dev)
+        inv_perm = torch.empty(s, dtype=torch.int32, device=dev)
+    else:
+        counts, offsets, perm, inv_perm = out
+        for t, n in ((counts, n_experts), (offsets, n_experts + 1), (perm, s), (inv_perm, s)):
+            if t.dtype != torch.int32 or t.numel() < n or t.device != dev:
+                raise _l.DiceError("dispatch: an output table is too small, not int32 or on another device")
+    if skip_mask is not None:
+        if skip_mask.numel() != s or skip_mask.device != dev:
+            raise _l.DiceError(f"dispatch: skip mask of {skip_mask.numel()} entries on {skip_mask.device} "
+                               f"for {s} slots on {dev}")
+        skip_mask = skip_mask.view(torch.uint8) if skip_mask.dtype == torch.bool else skip_mask
+    if static_scratch:
+        check(load().dice_dispatch_static(ptr(flat_idx), ptr(skip_mask), s, n_experts, ptr(counts),
+                                          ptr(offsets), ptr(perm), ptr(inv_perm), stream_ptr()))
+        return counts, offsets, perm, inv_perm
     ws_bytes = load().dice_dispatch_workspace_bytes(s, n_experts)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-    if skip_mask is not None:
-        skip_mask = skip_mask.view(torch.uint8) if skip_mask.dtype == torch.bool else skip_mask
     check(load().dice_dispatch(ptr(flat_idx), ptr(skip_mask), s, n_experts, ptr(counts), ptr(offsets),
                                ptr(perm), ptr(inv_perm), ptr(ws), ws_bytes, stream_ptr()))
     return counts, offsets, perm, inv_perm
@@ -117,9 +134,18 @@ def ln_modulate(x: torch.Tensor, shift: torch.Tensor, scale: torch.Tensor, eps: 
     parameters (reference models.py:75-76,497,519).  ``x [B, T, D]``, ``shift``
     and ``scale`` ``[B, D]``."""
     b, t, d = x.shape
+    if shift.shape != (b, d) or scale.shape != (b, d):
+        raise _l.DiceError(f"ln_modulate: x {tuple(x.shape)} needs shift and scale [{b}, {d}], "
+                           f"got {tuple(shift.shape)} and {tuple(scale.shape)}")
+    if shift.dtype != x.dtype or scale.dtype != x.dtype:
+        raise _l.DiceError("ln_modulate: shift and scale must have x's dtype")
     x = x.contiguous()
+    # Contiguous copies of strided views (chunks of the adaLN output) must stay
+    # alive until the launch is enqueued: a temporary dies as soon as its
+    # address has been taken and the allocator may hand its block to the next.
+    shift_c, scale_c = shift.contiguous(), scale.contiguous()
     out = torch.empty_like(x)
-    check(load().dice_ln_modulate(ptr(x), ptr(shift.contiguous()), ptr(scale.contiguous()), ptr(out),
+    check(load().dice_ln_modulate(ptr(x), ptr(shift_c), ptr(scale_c), ptr(out),
                                   dtype_code(x.dtype), b * t, d, t, eps, stream_ptr()))
     return out
 

@@ -222,6 +222,25 @@ def test_skip_policy_matches_oracle():
     assert not diep.ep_skip_enabled() and not diep.ep_skip_now(0)
 
 
+def test_skip_mask_slot_literals():
+    """Which slot each strategy masks, written out (reference diep.py:74-79:
+    'high' -> mask[::2], the slot with the higher router score; 'low' ->
+    mask[1::2]).  Exchanging the two in both the oracle and the product would
+    pass every symmetry test; it fails here."""
+    from dice_amd import diep
+    from oracle import dice_oracle as O
+    T, F = True, False
+    assert O.skip_mask(8, "high").tolist() == [T, F, T, F, T, F, T, F]
+    assert O.skip_mask(8, "low").tolist() == [F, T, F, T, F, T, F, T]
+    try:
+        diep.ep_cache_init(cache_capacity=1, noskip_step=2, skip_mode="high")
+        assert diep.ep_skip_mask(8).tolist() == [T, F, T, F, T, F, T, F]
+        diep.ep_cache_init(cache_capacity=1, noskip_step=2, skip_mode="low")
+        assert diep.ep_skip_mask(8).tolist() == [F, T, F, T, F, T, F, T]
+    finally:
+        diep.ep_cache_init(cache_capacity=1, noskip_step=1)
+
+
 def test_forced_sync_schedule():
     from dice_amd import diep
     assert diep.ep_forced_sync(50, 50)

@@ -102,6 +102,41 @@ def test_build_blocks_from_file_on_cpu(tmp_path):
         C.find_model(os.path.join(tmp_path, "absent.pt"))
 
 
+def test_train_script_checkpoint_opens_weights_only(tmp_path):
+    """The file the reference's train.py writes (train.py:258-266): model, ema,
+    optimizer state and ``"args": argparse.Namespace``.  It must open through
+    the tensors-only loader (ema wins), and a file holding any other class must
+    be refused by name instead of being unpickled."""
+    import argparse
+    import collections
+    from dice_amd import checkpoint as C
+    from dice_amd.lib import DiceError
+    D, E = 64, 4
+    model = _reference_style_state_dict([O.make_block_params(D, E, 2, 4, 2, seed=7)], D)
+    ema = collections.OrderedDict((k, v + 1) for k, v in model.items())
+    opt = {"state": {0: {"step": torch.tensor(3.0), "exp_avg": torch.zeros(4), "exp_avg_sq": torch.zeros(4)}},
+           "param_groups": [{"lr": 1e-4, "betas": (0.9, 0.999), "eps": 1e-8, "weight_decay": 0, "amsgrad": False,
+                             "params": [0]}]}
+    args = argparse.Namespace(model="DiT-S/2", image_size=256, num_experts=8, num_experts_per_tok=2,
+                              ckpt_every=50000, resume=None, results_dir="results", vae="ema")
+    path = os.path.join(tmp_path, "0050000.pt")
+    torch.save({"model": model, "ema": ema, "opt": opt, "args": args}, path)
+    sd = C.find_model(path)
+    assert set(sd) == set(ema) and all(torch.equal(sd[k], ema[k]) for k in ema)
+    blocks = C.build_moe_blocks(sd)
+    assert list(blocks) == [0]
+
+    import fractions
+    bad = os.path.join(tmp_path, "bad.pt")
+    torch.save({"model": model, "extra": fractions.Fraction(1, 3)}, bad)   # not a tensor, not a Namespace
+    with pytest.raises(DiceError, match="Fraction"):
+        C.find_model(bad)
+    lst = os.path.join(tmp_path, "list.pt")
+    torch.save([torch.zeros(2)], lst)
+    with pytest.raises(DiceError, match="state dict"):
+        C.find_model(lst)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("fp8", [False, True])
 def test_blocks_from_checkpoint_match_oracle_on_gpu(tmp_path, fp8):

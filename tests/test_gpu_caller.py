@@ -222,3 +222,100 @@ def test_half_model_under_autocast_with_fp32_stream(dev):
     want = x + gate.unsqueeze(1) * wy.float()
     ok2 = ~O.gate_tie_rows(logits2, 2, tol=1e-3).view(B, T)
     assert rel_l2(out.cpu()[ok2], want[ok2]) < 4e-3
+
+
+def test_strided_adaln_chunks(dev):
+    """shift / scale / gate as the reference hands them over: chunks of ONE
+    adaLN output tensor (``self.adaLN_modulation(c).chunk(6, dim=1)``,
+    models.py:515), i.e. strided views.  Every wrapper must keep its contiguous
+    copies alive until the launch; a copy freed early is overwritten by the
+    next one (shift and scale would then read the same memory)."""
+    from dice_amd import ops
+    B, T, D = 3, 64, 384
+    g = _gen(23)
+    x = (torch.randn(B, T, D, generator=g) * 2 + 0.5)
+    c = torch.randn(B, 6 * D, generator=g) * 0.3
+    cd = c.to(dev)
+    shift_msa, scale_msa, gate_msa, shift, scale, gate = cd.chunk(6, dim=1)
+    assert not shift.is_contiguous() and not scale.is_contiguous()
+    w_shift, w_scale, w_gate = c.chunk(6, dim=1)[3:]
+    want = O.norm_modulate(x, w_shift, w_scale, single_rounding=True)
+    got = ops.ln_modulate(x.to(dev), shift, scale).cpu()
+    assert torch.allclose(got, want, atol=2e-5, rtol=1e-5)
+    # the whole line, same-dtype branch (fused prologue / epilogue)
+    p = O.make_block_params(D, 8, 2, 4, 2, seed=5, gate_std=0.1)
+    blk = block_from_params(p, D, "swiglu", torch.float32, dev)
+    want_line, _, _, _, logits = O.dit_block_moe_half(p, x, w_shift, w_scale, w_gate, single_rounding=True)
+    ok = ~O.gate_tie_rows(logits, 2, tol=1e-4).view(B, T)
+    out = blk.forward_modulated(x.to(dev), shift, scale, gate).cpu()
+    assert rel_l2(out[ok], want_line[ok]) < FP32_TOL
+    # mixed-precision branch: fp16 block under autocast, fp32 stream and fp32 strided chunks
+    p16 = O.make_block_params(D, 8, 2, 4, 2, seed=5, gate_std=0.1, dtype=torch.float16)
+    blk16 = block_from_params(p16, D, "swiglu", torch.float16, dev)
+    with torch.autocast(device_type="cuda", dtype=torch.float16):
+        out16 = blk16.forward_modulated(x.to(dev), shift, scale, gate).cpu()
+    h = O.norm_modulate(x, w_shift, w_scale)
+    wy, _, _, logits2 = O.sparse_moe_block_forward(p16, h.half())
+    want16 = x + w_gate.unsqueeze(1) * wy.float()
+    ok2 = ~O.gate_tie_rows(logits2, 2, tol=1e-3).view(B, T)
+    assert rel_l2(out16[ok2], want16[ok2]) < 4e-3
+    with pytest.raises(Exception, match="shift and scale"):
+        ops.ln_modulate(x.to(dev), shift[:, :-8], scale)
+
+
+def test_stale_mask_or_cache_is_refused_before_launch(dev):
+    """A skip mask or cache tensor left over from another batch size would be
+    indexed out of bounds by the kernels; the host side raises instead (the
+    reference fails with a shape error in the same situation).  Nothing is
+    launched on the refused calls."""
+    from dice_amd import DiceError, diep, ops
+    from dice_amd.lib import MODE_PUT, MODE_SKIP
+    D, E, N = 256, 8, 256
+    p = O.make_block_params(D, E, 2, 4, 2, seed=6)
+    blk = block_from_params(p, D, "swiglu", torch.float32, dev, ep=True, layer_idx=0)
+    x = torch.randn(N, D, generator=_gen(6)).to(dev)
+    mask = O.skip_mask(2 * N, "high").to(dev)
+    cache = torch.empty_like(x)
+    blk.run(x, MODE_PUT, mask, None, cache)
+    with pytest.raises(DiceError, match="skip mask"):
+        blk.run(x, MODE_SKIP, mask[:-2], cache, None)
+    with pytest.raises(DiceError, match="skip mask"):
+        blk.run(x, MODE_SKIP, mask.cpu(), cache, None)
+    with pytest.raises(DiceError, match="cache_in"):
+        blk.run(x, MODE_SKIP, mask, cache[: N // 2], None)
+    with pytest.raises(DiceError, match="cache_in"):
+        blk.run(x, MODE_SKIP, mask, cache.half(), None)
+    with pytest.raises(DiceError, match="cache_out"):
+        blk.run(x, MODE_PUT, mask, None, torch.empty(N, D // 2, device=dev))
+    with pytest.raises(DiceError, match="needs cache_in"):
+        blk.run(x, MODE_SKIP, mask, None, None)
+    # through the module: the batch grows between a full step and the skip step that follows
+    diep.ep_cache_init(cache_capacity=1, noskip_step=2, skip_mode="rand")
+    diep.ep_set_rand_mask(None)
+    try:
+        diep.ep_set_step(8)
+        diep.ep_cache_clear()
+        blk(x.view(1, N, D))
+        diep.ep_set_step(7)
+        assert diep.ep_skip_now(0)
+        with pytest.raises(DiceError, match="rand"):
+            blk(torch.cat([x, x]).view(1, 2 * N, D))      # the 'rand' mask was drawn for N tokens
+        diep.ep_cache_init(cache_capacity=1, noskip_step=2, skip_mode="high")
+        diep.ep_set_step(8)
+        blk(x.view(1, N, D))
+        diep.ep_set_step(7)
+        with pytest.raises(DiceError, match="cache_in"):
+            blk(torch.cat([x, x]).view(1, 2 * N, D))      # cached rows of N tokens, 2N arrive
+    finally:
+        diep.ep_cache_init(cache_capacity=1, noskip_step=1)
+    # caller-supplied routing with an expert id outside the table: the slot is dropped and adds nothing
+    idx = torch.randint(0, E, (2 * N,), generator=_gen(7))
+    w = torch.rand(2 * N, 1, generator=_gen(8))
+    bad = idx.clone()
+    bad[5], bad[100] = E, -1
+    y_bad = blk.moe_infer(x, bad.to(dev), w.to(dev)).cpu()
+    w0 = w.clone()
+    w0[5], w0[100] = 0, 0
+    y_ref = blk.moe_infer(x, idx.to(dev), w0.to(dev)).cpu()
+    assert torch.allclose(y_bad, y_ref, atol=1e-6)
+    torch.cuda.synchronize()
