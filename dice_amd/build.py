@@ -29,6 +29,7 @@ SOURCES = [
     "grouped_gemm_f16.hip",
     "grouped_gemm_persist.hip",
     "grouped_gemm_persist_f16.hip",
+    "grouped_gemm_persist_f8.hip",
     "grouped_mlp.hip",
 ]
 

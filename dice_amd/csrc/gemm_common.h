@@ -161,6 +161,8 @@ struct PersistProblem {
   int a_div;               // slots per source row (top-k)
   int a_src_rows;          // rows of the source matrix (range check of the gather)
   const float *w_scale;    // [n_experts, w_rows] per-output-channel scales: the weights are fp8 (e4m3) bytes; NULL: bf16
+  const float *a_scale;    // [max_rows] per-row scales in grouped order: the activations too are fp8 (e4m3) bytes
+                           // (lda then counts bytes) and the products run on the fp8 matrix pipe; NULL: 16-bit rows
 };
 constexpr int kMaxPersistProblems = 3;
 struct PersistBatch {
@@ -172,6 +174,9 @@ int persist_cu_count();  // compute units of the current device
 bool gemm_config_allows_persistent(int mode);  // tuning hook state: no tiling of the permutation-addressed kernels is forced for this stage
 int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s);      // bf16
 int launch_grouped_gemm_persist_f16(const PersistBatch &b, int mode, hipStream_t s);  // fp16
+// fp8 activations (a_scale) and weights (w_scale) on the fp8 matrix pipe, bf16 output
+bool persist_f8_supported(const PersistBatch &b, int mode);
+int launch_grouped_gemm_persist_f8(const PersistBatch &b, int mode, hipStream_t s);
 
 // LayerNorm + adaLN modulation in front of the layer, and the combine with the
 // caller's residual / gate epilogue behind it (modulate.hip, combine.hip).
@@ -188,6 +193,11 @@ int dispatch_impl(const int32_t *flat_idx, const uint8_t *skip_mask, int64_t n_s
 int gather_rows_impl(const void *x, int dtype, const int32_t *perm, int slots_per_token,
                      int64_t n_rows, int hidden, void *out, int32_t *range_out, int32_t range_n,
                      void *stream);
+
+// Rows of x (row perm[r] / slots_per_token when perm is given) -> e4m3 rows and one scale per row (quant.hip).
+int quantize_act_impl(const void *x, int in_dtype, const int32_t *perm, int slots_per_token,
+                      const int32_t *n_rows_dev, int64_t max_rows, int cols, uint8_t *q, float *scale,
+                      void *stream);
 
 int launch_grouped_gemm_bf16(const GemmParams &p, int mode, int w_dtype, int64_t max_rows,
                              hipStream_t s);

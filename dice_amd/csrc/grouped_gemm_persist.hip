@@ -46,6 +46,12 @@
 #ifndef DICE_PERSIST_F16
 #define DICE_PERSIST_F16 0
 #endif
+// A third compilation (grouped_gemm_persist_f8.hip, DICE_PERSIST_F8) holds the
+// kernel whose activations are fp8 as well; it shares the tile order, the tile
+// table and the epilogue with the others and writes bf16.
+#ifndef DICE_PERSIST_F8
+#define DICE_PERSIST_F8 0
+#endif
 
 namespace dice {
 namespace {
@@ -258,8 +264,11 @@ struct TileWalker {
   // turn0 + r - and leaves them in LDS, kTileWords dwords per turn in PackedTile order, so
   // that a tile switch inside the kernel is a single LDS read.  Turns past the
   // XCD's run give descriptions that cover no bytes.  Called by one wave.
+  // a8: the activations are fp8 bytes (one byte per element; no row table) and
+  // words 20/21 carry the address of the tile's per-row scales instead.
   __device__ __forceinline__ void build_table(const PersistBatch &batch, int lane, int bk,
-                                              uint32_t *table, bool w8 = false, int turn0 = 0) const {
+                                              uint32_t *table, bool w8 = false, int turn0 = 0,
+                                              bool a8 = false) const {
     const int turn = turn0 + lane;  // entry `lane` of the table describes this turn
     const int w = (turn & 1) ? wgs_per_xcd - 1 - wg_in_xcd : wg_in_xcd;
     const int id = run_begin + turn * wgs_per_xcd + w;
@@ -276,7 +285,7 @@ struct TileWalker {
     const int row0 = __shfl(g_row0, grp, kWave), cnt = __shfl(g_cnt, grp, kWave);
     const int mt = __shfl(g_mt, grp, kWave), base = __shfl(g_base, grp, kWave);
     // this lane's problem (a handful of selects instead of a divergent struct index)
-    uint64_t pa = 0, pw = 0, pc = 0, pbias = 0, prows = 0;
+    uint64_t pa = 0, pw = 0, pc = 0, pbias = 0, prows = 0, pascale = 0;
     int lda = 0, ldc = 0, w_rows = 0, up_offset = 0, n = 0, k = 0, a_div = 1, a_src_rows = 0;
     for (int q = 0; q < batch.n_problems; ++q) {
       const PersistProblem &pr = batch.prob[q];
@@ -284,6 +293,7 @@ struct TileWalker {
         pa = (uint64_t)pr.a; pw = (uint64_t)pr.w; pc = (uint64_t)pr.c; pbias = (uint64_t)pr.bias;
         lda = pr.lda; ldc = pr.ldc; w_rows = pr.w_rows; up_offset = pr.up_offset; n = pr.n; k = pr.k;
         prows = (uint64_t)pr.a_rows; a_div = pr.a_div; a_src_rows = pr.a_src_rows;
+        pascale = (uint64_t)pr.a_scale;
       }
     }
     const int r = idc - base;
@@ -297,7 +307,7 @@ struct TileWalker {
     // (fp8 weights: one byte per element, and word 22 carries the row of the
     // per-output-channel scale table instead of the gather's reciprocal, which a
     // single-problem launch takes from its arguments)
-    const uint32_t a_pitch = (uint32_t)lda * 2, b_pitch = (uint32_t)k * (w8 ? 1 : 2), c_pitch = (uint32_t)ldc * 2;
+    const uint32_t a_pitch = (uint32_t)lda * (a8 ? 1 : 2), b_pitch = (uint32_t)k * (w8 ? 1 : 2), c_pitch = (uint32_t)ldc * 2;
     const uint64_t wexp = pw + (uint64_t)expert * w_rows * b_pitch;
     // Gathered rows are addressed from the start of the source matrix.
     const uint64_t ptrs[5] = {prows ? pa : pa + (uint64_t)(row0 + m_tile * kPBM) * a_pitch, wexp + (uint64_t)n0 * b_pitch,
@@ -316,7 +326,8 @@ struct TileWalker {
     }
 #pragma unroll
     for (int i = 0; i < 10; ++i) entry[10 + i] = words[i];
-    const uint64_t tile_rows = prows ? prows + (uint64_t)(row0 + m_tile * kPBM) * sizeof(int32_t) : 0;
+    const uint64_t tile_rows = a8 ? pascale + (uint64_t)(row0 + m_tile * kPBM) * sizeof(float)
+                                  : (prows ? prows + (uint64_t)(row0 + m_tile * kPBM) * sizeof(int32_t) : 0);
     entry[20] = (uint32_t)tile_rows;
     entry[21] = (uint32_t)(tile_rows >> 32);
     entry[22] = w8 ? (uint32_t)(expert * w_rows + n0)
@@ -423,10 +434,14 @@ __device__ __forceinline__ f32x16_t acc_block(const f32x16_t &a) {
 // offset no descriptor covers.
 // HAS_SCALE: the weights were fp8; column c of the product is multiplied by
 // scale_lds[c - n0] (SwiGLU: gate columns first, the up columns 128 floats on).
-template <int MODE, bool HAS_BIAS, int WAVES, int TM, int TN, bool HAS_SCALE = false, int RESERVE = 0>
+// HAS_ROW: the activations were fp8 with one scale per row; row m of the tile is
+// multiplied by rowscale_lds[m] as well.
+template <int MODE, bool HAS_BIAS, int WAVES, int TM, int TN, bool HAS_SCALE = false, int RESERVE = 0,
+          bool HAS_ROW = false>
 __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM][TN], unsigned char *stage,
                                               int wave_row0, int wave_col0, int lane,
-                                              const float *scale_lds = nullptr) {
+                                              const float *scale_lds = nullptr,
+                                              const float *rowscale_lds = nullptr) {
   using G = EpiGeom<MODE, WAVES, TM, TN, RESERVE>;
   constexpr bool SWIGLU = G::SWIGLU;
   constexpr int OUT_BLOCKS = G::OUT_BLOCKS, PITCH = G::PITCH, BAND = G::BAND;
@@ -458,6 +473,10 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
     const float *sp = scale_lds + wave_col0 + (j) * 32 + frag_half * 4 + (q) * 8;                       \
     sg = *reinterpret_cast<const f32x4_t *>(sp);                                                      \
     if (SWIGLU) su = *reinterpret_cast<const f32x4_t *>(sp + 128);                                    \
+    if (HAS_ROW) {                                                                                    \
+      sg *= row_scale;                                                                                \
+      if (SWIGLU) su *= row_scale;                                                                    \
+    }                                                                                                 \
   }
 #define DICE_EPI_VALUE(v, j, q, r)                          \
   do {                                                      \
@@ -491,6 +510,8 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
   } while (0)
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
+    float row_scale = 1.0f;
+    if (HAS_ROW) row_scale = rowscale_lds[wave_row0 + i * 32 + frag_row];
     if constexpr (BAND == 32) {
 #pragma unroll
       for (int j = 0; j < OUT_BLOCKS; ++j) {
@@ -1277,6 +1298,442 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   }
 }
 
+#if DICE_PERSIST_F8
+// ---------------------------------------------------------------------------
+// fp8 x fp8 pipeline, four waves: e4m3 activations (one fp32 scale per row) times
+// e4m3 weights (one fp32 scale per output channel) on v_mfma_f32_32x32x64_f8f6f4,
+// which multiplies at twice the rate of the bf16 instruction.
+//
+// In bytes this is the 64-k pipeline above: rows of 128 bytes per step (now 128
+// k), two 64 KB LDS slots, operands staged through two register stages four
+// steps ahead, the same 256x256 tile, wave tile, epilogue and tile table - so
+// the bytes moved per matrix-pipe cycle are those of the bf16 kernel while every
+// byte carries twice the arithmetic.  What differs:
+//
+//   * A fragment of the fp8 instruction is 32 bytes per lane (two 16-byte LDS
+//     reads).  The hardware lets lanes 0-31 and 32-63 each hold 32 k of a row;
+//     any assignment of k to (lane half, byte) works as long as both operands
+//     use the same one, here: half h of k-block kb takes the row's 16-byte
+//     chunks 4 kb + 2 h and 4 kb + 2 h + 1.
+//   * Fragments twice the size do not fit twice in the register file, so they
+//     are not double-buffered.  A step is two halves of 16 MFMAs (one per 64-k
+//     block), taken row block by row block; during a half the next half's
+//     fragments are read into the registers of operands as they die: row block
+//     i behind the four MFMAs that use it, the weight blocks one by one during
+//     the last row block, and what the half's last MFMA still holds (the last
+//     weight block and the last row block) right behind it.  Eight fragments =
+//     64 registers, as many as the bf16 kernel's double-buffered set.
+//   * The workgroup barrier sits four MFMAs into the second half: by then
+//     every wave has read the step's slot for the last time (the trailing reads
+//     of the first half have had four MFMAs to land) and has finished writing
+//     the other slot; behind it the second half starts to refill this slot and
+//     to read the next step's fragments from the other one.  Each half writes
+//     two quarters of a step into LDS and issues the loads that refill those
+//     register stages.
+//   * The epilogue multiplies the fp32 sums by the row's and the column's scale
+//     (both staged in LDS a tile ahead); a bias enters the accumulators divided
+//     by both.
+//
+// Rows are contiguous (the quantiser writes the activations in grouped order),
+// the reduction length is a multiple of 256 (an even number of steps), weight
+// tiles are 256 rows (SwiGLU: 128 gate + 128 up), single-problem launches.
+typedef int i32x8_t __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ f32x16_t mfma_f8_32x32x64(i32x8_t a, i32x8_t b, f32x16_t c) {
+  // cbsz = blgp = 0: both operands e4m3; zero scale operands select the unscaled instruction
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+
+// Instruction order of one half.  MFMA m (row block m / 4) is followed by the
+// fragment reads whose registers have just come free: row block 0 behind MFMAs 4
+// and 5, row block 1 behind 8 and 9, row block 2 and three weight blocks in pairs
+// behind 12..15, the last weight block and row block 3 behind the half; and by
+// the LDS writes of a register stage alternating with the global loads that
+// refill it, from MFMA FIRST on (the second half of a step starts them behind its
+// barrier: 16 of them over 12 MFMAs).
+template <int M, int FIRST>
+__device__ __forceinline__ void f8_sched_half() {
+  if constexpr (M < 16) {
+    if constexpr (M >= FIRST) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      constexpr int reads = (M == 4 || M == 5 || M == 8 || M == 9) ? 1 : (M >= 12 ? 2 : 0);
+      if constexpr (reads > 0) __builtin_amdgcn_sched_group_barrier(0x100, reads, 0);
+      if constexpr (FIRST > 0 && M < 2 * FIRST) {
+        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      } else if constexpr (M % 2 == 0) {
+        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+      } else {
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
+    }
+    f8_sched_half<M + 1, FIRST>();
+  } else {
+    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+  }
+}
+
+template <int MODE, bool HAS_BIAS, bool REFILL>
+__device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) {
+  constexpr bool SWIGLU = MODE == kFc1Swiglu;
+  static_assert(!(SWIGLU && HAS_BIAS), "the SwiGLU expert has no bias");
+  constexpr int BN_OUT = SWIGLU ? kPBN / 2 : kPBN;
+  constexpr int WTM = 128, TM = 4, TN = 4;
+  constexpr int kFBK = 128;                         // k per step (one byte per element)
+  constexpr int kCopiesA = kPBM / 8 / kQWaves;      // 16-byte loads per lane and step: 8 + 8
+  constexpr int kFCopies = 2 * kCopiesA;
+  constexpr int kScaleBufFloats = 256, kBiasBufFloats = 256;
+  constexpr int kTableBytes = kTableTurns * kTileWords * 4;
+  // three buffers each for the column and the row scales: the epilogue of a tile
+  // reads them while the first wave, a little ahead, may already stage those of
+  // the tile after the next; the bias (read at the tile switch) needs two
+  constexpr int kColScaleBytes = 3 * kScaleBufFloats * 4, kRowScaleBytes = 3 * kPBM * 4;
+  constexpr int kBiasBytes = HAS_BIAS ? 2 * kBiasBufFloats * 4 : 0;
+  constexpr int kEpiReserve = kTableBytes + kColScaleBytes + kRowScaleBytes + kBiasBytes;
+  using Epi = EpiGeom<MODE, kQWaves, TM, TN, kEpiReserve>;
+  static_assert(kQWaves * Epi::WAVE_BYTES + kEpiReserve <= kPStageArea, "no room beside the epilogue's staging rows");
+  const template_int<0> c0; const template_int<1> c1; const template_int<2> c2; const template_int<3> c3;
+
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_slot0[kQSlotBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_slot1[kQSlotBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_stage[kPStageArea];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+
+  uint32_t *const tile_table = reinterpret_cast<uint32_t *>(lds_stage + kPStageArea - kTableBytes);
+  float *const lds_colscale = reinterpret_cast<float *>(lds_stage + kPStageArea - kTableBytes - kColScaleBytes);
+  float *const lds_rowscale =
+      reinterpret_cast<float *>(lds_stage + kPStageArea - kTableBytes - kColScaleBytes - kRowScaleBytes);
+  float *const lds_bias = reinterpret_cast<float *>(lds_stage + kPStageArea - kEpiReserve);
+  if (wave == 0) {
+    TileWalker<BN_OUT> walk(batch, lane);
+    walk.build_table(batch, lane, kFBK, tile_table, true, 0, true);
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  phase_barrier();
+  auto fetch_tile = [&](int turn) {
+    if constexpr (REFILL) {
+      if (turn != 0 && (turn & (kTableTurns - 1)) == 0) {
+        phase_barrier();
+        if (wave == 0) {
+          TileWalker<BN_OUT> walk(batch, lane);
+          walk.build_table(batch, lane, kFBK, tile_table, true, turn, true);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        phase_barrier();
+      }
+    }
+    return PackedTile{tile_table[(turn & (kTableTurns - 1)) * kTileWords + (lane < kTileWords ? lane : 0)]};
+  };
+
+  // ---- what the first wave stages in LDS a tile ahead (one global->LDS
+  // instruction each): column scales, row scales, bias ----
+  auto copy_colscale = [&](const PackedTile &pk, int buf) {
+    const uint32_t row = (uint32_t)__builtin_amdgcn_readlane(pk.words, 22);
+    const int n0 = __builtin_amdgcn_readlane(pk.words, 16), n = __builtin_amdgcn_readlane(pk.words, 17);
+    if (wave == 0) {
+      const float *base = batch.prob[0].w_scale + row;
+      // SwiGLU: 128 gate scales, then the 128 up scales up_offset rows further on;
+      // otherwise the tile's columns, those past the matrix reading as 0
+      const uint32_t bytes = SWIGLU ? (uint32_t)(batch.prob[0].up_offset + 128) * 4 : (uint32_t)(n - n0) * 4;
+      const uint32_t voff = SWIGLU && lane >= 32 ? (uint32_t)batch.prob[0].up_offset * 4 + (lane - 32) * 16 : lane * 16;
+      const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, bytes, kRsrcFlags);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rs, (__attribute__((address_space(3))) void *)(lds_colscale + buf * kScaleBufFloats), 16, voff, 0, 0, 0);
+    }
+  };
+  auto copy_rowscale = [&](const PackedTile &pk, int buf) {
+    const uint64_t ptr = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane(pk.words, 21) << 32) |
+                         (uint32_t)__builtin_amdgcn_readlane(pk.words, 20);
+    const int rows = __builtin_amdgcn_readlane(pk.words, 23);
+    if (wave == 0 && ptr != 0) {
+      // rows past the group's end read as 0 (their products are never stored)
+      const __amdgpu_buffer_rsrc_t rs =
+          __builtin_amdgcn_make_buffer_rsrc((void *)ptr, 0, (uint32_t)rows * 4, kRsrcFlags);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rs, (__attribute__((address_space(3))) void *)(lds_rowscale + buf * kPBM), 16, lane * 16, 0, 0, 0);
+    }
+  };
+  auto copy_bias = [&](const PackedTile &pk, int buf) {
+    if constexpr (HAS_BIAS) {
+      const uint64_t ptr = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane(pk.words, 9) << 32) |
+                           (uint32_t)__builtin_amdgcn_readlane(pk.words, 8);
+      const int n0 = __builtin_amdgcn_readlane(pk.words, 16), n = __builtin_amdgcn_readlane(pk.words, 17);
+      if (wave == 0 && ptr != 0) {
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(ptr + (uint64_t)n0 * 4), 0, (uint32_t)(n - n0) * 4, kRsrcFlags);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rs, (__attribute__((address_space(3))) void *)(lds_bias + buf * kBiasBufFloats), 16, lane * 16, 0, 0, 0);
+      }
+    }
+  };
+
+  // ---- global loads: one instruction fetches 8 rows x 128 bytes (8 lanes per
+  // row, whole lines); load l of a wave covers rows wave * 8 + 32 (l % 8) .. + 8
+  // of the activation tile (l < 8) or of the weight tile ----
+  const int cp_row0 = wave * 8 + (lane >> 3);
+  const int cp_chunk = lane & 7;
+  uint32_t wr_off = qring_off(cp_row0, cp_chunk);
+  asm volatile("" : "+v"(wr_off));
+  uint32_t ld_voff_a = 0, ld_voff_b = 0;
+  auto set_copy_offsets = [&](const Tile &t) {
+    ld_voff_a = (uint32_t)cp_row0 * t.a_pitch + cp_chunk * 16;
+    ld_voff_b = (uint32_t)cp_row0 * t.b_pitch + cp_chunk * 16;
+    asm volatile("" : "+v"(ld_voff_a), "+v"(ld_voff_b));
+  };
+  u32x4_t stage_regs[2][kFCopies];
+
+  // ---- fragment reads: lane part per (k-block, 16-byte half); 32-row blocks and
+  // the slot add compile-time constants ----
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  const int b_row0 = SWIGLU ? wn * 64 : wn * 128;
+  uint32_t rd_a[4], rd_b[4];   // [2 kb + t]: chunk 4 kb + 2 h + t of the lane's row
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      rd_a[kb * 2 + t] = qring_off(wm * WTM + frag_row, kb * 4 + frag_half * 2 + t);
+      rd_b[kb * 2 + t] = kPBM * 128 + qring_off(b_row0 + frag_row, kb * 4 + frag_half * 2 + t);
+      asm volatile("" : "+v"(rd_a[kb * 2 + t]), "+v"(rd_b[kb * 2 + t]));
+    }
+  auto read32 = [&](const unsigned char *slot, uint32_t off_lo, uint32_t off_hi) {
+    const u32x4_t lo = *reinterpret_cast<const u32x4_any_t *>(slot + off_lo);
+    const u32x4_t hi = *reinterpret_cast<const u32x4_any_t *>(slot + off_hi);
+    i32x8_t f;
+    f[0] = (int)lo[0]; f[1] = (int)lo[1]; f[2] = (int)lo[2]; f[3] = (int)lo[3];
+    f[4] = (int)hi[0]; f[5] = (int)hi[1]; f[6] = (int)hi[2]; f[7] = (int)hi[3];
+    return f;
+  };
+  // activation rows 32 i .. of the wave's 128, k-block KB of slot SLOT
+  auto read_a = [&](auto slot_c, auto kb_c, int i) {
+    constexpr int SLOT = decltype(slot_c)::value, KB = decltype(kb_c)::value;
+    const unsigned char *base = (SLOT == 0 ? lds_slot0 : lds_slot1) + i * 32 * 128;
+    return read32(base, rd_a[KB * 2], rd_a[KB * 2 + 1]);
+  };
+  // weight block j of the wave's four (SwiGLU: two of gate rows, two of up rows)
+  auto read_w = [&](auto slot_c, auto kb_c, int j) {
+    constexpr int SLOT = decltype(slot_c)::value, KB = decltype(kb_c)::value;
+    const int jrow = (SWIGLU && j >= 2) ? kPBN / 2 + (j - 2) * 32 : j * 32;
+    const unsigned char *base = (SLOT == 0 ? lds_slot0 : lds_slot1) + jrow * 128;
+    return read32(base, rd_b[KB * 2], rd_b[KB * 2 + 1]);
+  };
+
+  const int wave_col0 = SWIGLU ? wn * 64 : wn * 128;
+  f32x16_t acc[TM][TN];
+  // Biased tiles start their accumulators from bias / (column scale * row scale):
+  // the epilogue multiplies the sums by both.
+  auto init_acc = [&](const Tile &t, int bbuf, int sbuf) {
+    if constexpr (HAS_BIAS) {
+      if (uni((int)(t.bias != nullptr))) {
+        float rinv[TM];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const float rs = lds_rowscale[sbuf * kPBM + wm * WTM + i * 32 + frag_row];
+          rinv[i] = rs > 0.f ? 1.0f / rs : 0.f;
+        }
+        const float *src = lds_bias + bbuf * kBiasBufFloats + wave_col0 + frag_half * 4;
+        const float *scl = lds_colscale + sbuf * kScaleBufFloats + wave_col0 + frag_half * 4;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          f32x16_t b;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const f32x4_t v = *reinterpret_cast<const f32x4_t *>(src + j * 32 + q * 8);
+            const f32x4_t sc = *reinterpret_cast<const f32x4_t *>(scl + j * 32 + q * 8);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) b[q * 4 + r] = sc[r] != 0.f ? v[r] / sc[r] : 0.f;
+          }
+#pragma unroll
+          for (int i = 0; i < TM; ++i) acc[i][j] = b * rinv[i];
+        }
+        return;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+  };
+
+  // ---- pipeline state (as in the 64-k pipeline) ----
+  int next_turn = 0;
+  PackedTile nxt = fetch_tile(next_turn++);
+  Tile ld = unpack_tile(nxt);                     // tile being loaded
+  if (!ld.valid) return;
+  int bias_buf = 0, scale_buf = 0;
+  copy_colscale(nxt, 0);
+  copy_rowscale(nxt, 0);
+  copy_bias(nxt, 0);
+  pwait_vmcnt<0>();
+  phase_barrier();
+  Tile cp = ld;                                   // tile being multiplied
+  int ld_kt = 0;
+  set_copy_offsets(ld);
+  nxt = fetch_tile(next_turn++);                  // the one the load side opens next
+  copy_colscale(nxt, 1);
+  copy_rowscale(nxt, 1);
+  copy_bias(nxt, 1);
+  auto advance_copy = [&]() {
+    if (++ld_kt == ld.steps) {
+      ld = unpack_tile(nxt);
+      set_copy_offsets(ld);
+      ld_kt = 0;
+    }
+  };
+  // A step's loads in four quarters of four: the two halves of the activation
+  // rows, then the two halves of the weight rows.
+  auto load_quarter = [&](auto stage_c, auto q_c) {
+    constexpr int P = decltype(stage_c)::value, Q = decltype(q_c)::value;
+#pragma unroll
+    for (int l = 4 * Q; l < 4 * Q + 4; ++l) {
+      // The row block of a load is folded into its descriptor (base moved on, extent
+      // cut by as much: scalar arithmetic only), not into the scalar offset, which
+      // the range check ignores: rows past the tile's end must read as zero, never
+      // from beyond the matrix.
+      if (l < kCopiesA) {
+        const uint32_t skip = (uint32_t)(32 * l) * uni(ld.a_pitch);
+        const uint32_t extent = uni(ld.a_bytes);
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(uni(ld.a) + skip), 0, extent > skip ? extent - skip : 0u, kRsrcFlags);
+        stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(rs, ld_voff_a, uni(ld_kt * kFBK), 0);
+      } else {
+        const int i = l - kCopiesA;
+        const bool up_half = SWIGLU && 32 * i >= kPBN / 2;
+        const int row = up_half ? 32 * i - kPBN / 2 : 32 * i;
+        const uint32_t skip = (uint32_t)row * uni(ld.b_pitch);
+        const uint32_t extent = uni(ld.b_bytes);
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(uni(up_half ? ld.b1 : ld.b0) + skip), 0, extent > skip ? extent - skip : 0u, kRsrcFlags);
+        stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(rs, ld_voff_b, uni(ld_kt * kFBK), 0);
+      }
+    }
+  };
+  auto write_quarter = [&](auto stage_c, auto q_c) {
+    constexpr int P = decltype(stage_c)::value, Q = decltype(q_c)::value;
+#pragma unroll
+    for (int l = 4 * Q; l < 4 * Q + 4; ++l) {
+      const int i = l < kCopiesA ? l : l - kCopiesA;
+      unsigned char *dst = (P == 0 ? lds_slot0 : lds_slot1) + (l < kCopiesA ? 0 : kPBM * 128) + i * 32 * 128 + wr_off;
+      *reinterpret_cast<u32x4_any_t *>(dst) = stage_regs[P][l];
+    }
+  };
+  auto load_step = [&](auto stage_c) {
+    load_quarter(stage_c, c0); load_quarter(stage_c, c1); load_quarter(stage_c, c2); load_quarter(stage_c, c3);
+    advance_copy();
+  };
+
+  i32x8_t W[TN], A[TM];   // the 64-k block being multiplied: weight blocks, row blocks
+  auto read_first_frags = [&]() {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) W[j] = read_w(c0, c0, j);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) A[i] = read_a(c0, c0, i);
+  };
+
+  // Prologue: steps 0 and 1 through the stages into the slots (of step 1 only
+  // the first two quarters: the rest follows during the first half of step 0, as
+  // in the steady state), step 2 and the first half of step 3 into the stages.
+  load_step(c0);           // step 0
+  load_step(c1);           // step 1
+  write_quarter(c0, c0); write_quarter(c0, c1); write_quarter(c0, c2); write_quarter(c0, c3);
+  load_step(c0);           // step 2
+  write_quarter(c1, c0);
+  write_quarter(c1, c1);
+  load_quarter(c1, c0);    // first half of step 3; the stage keeps quarters 2, 3 of step 1
+  load_quarter(c1, c1);
+  init_acc(cp, 0, 0);
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  phase_barrier();
+  read_first_frags();
+  __builtin_amdgcn_sched_barrier(0);
+
+  unsigned char *const stage_rows = lds_stage + wave * Epi::WAVE_BYTES;
+
+  // One half of a step: the 16 MFMAs of the 64-k block whose fragments sit in W
+  // and A, while the fragments of block RKB of slot RSLOT replace them, quarters
+  // WQ and WQ + 1 of register stage WSLOT go to LDS slot WSLOT and are loaded
+  // again for the step after next.  BARRIER: the workgroup barrier of the step
+  // sits behind the first row block; everything but MFMAs follows it.
+  auto half = [&](auto rslot_c, auto rkb_c, auto wslot_c, auto wq_c, auto barrier_c) {
+    constexpr int WQ = decltype(wq_c)::value;
+    constexpr bool BARRIER = decltype(barrier_c)::value != 0;
+    if constexpr (BARRIER) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[0][j] = mfma_f8_32x32x64(W[j], A[0], acc[0][j]);
+      // This wave has read the step's slot for the last time and has finished
+      // writing the other slot; after the barrier both hold for every wave.
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      phase_barrier();
+    }
+    // (program order = the order in which the registers come free)
+    const i32x8_t na0 = read_a(rslot_c, rkb_c, 0);
+    const i32x8_t na1 = read_a(rslot_c, rkb_c, 1);
+    const i32x8_t na2 = read_a(rslot_c, rkb_c, 2);
+    i32x8_t nw[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) nw[j] = read_w(rslot_c, rkb_c, j);
+    const i32x8_t na3 = read_a(rslot_c, rkb_c, 3);
+    write_quarter(wslot_c, template_int<WQ>{});
+    load_quarter(wslot_c, template_int<WQ>{});
+    write_quarter(wslot_c, template_int<WQ + 1>{});
+    load_quarter(wslot_c, template_int<WQ + 1>{});
+#pragma unroll
+    for (int i = BARRIER ? 1 : 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = mfma_f8_32x32x64(W[j], A[i], acc[i][j]);
+    f8_sched_half<0, BARRIER ? 4 : 0>();
+    __builtin_amdgcn_sched_barrier(0);
+    A[0] = na0;
+    A[1] = na1;
+    A[2] = na2;
+    A[3] = na3;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) W[j] = nw[j];
+  };
+
+  while (true) {  // one tile per iteration
+    // Every tile has an even number of steps, so a tile always starts in slot 0.
+    auto step = [&](auto slot_c) {
+      constexpr int S = decltype(slot_c)::value;
+      const template_int<S ^ 1> other_c;
+      // first k-block; the other slot receives the second half of the next step
+      half(slot_c, c1, other_c, c2, c0);
+      advance_copy();
+      // second k-block; behind its barrier this slot receives the first half of
+      // the step after next and the next step's first fragments are read
+      half(other_c, c0, slot_c, c0, c1);
+    };
+    for (int s = 0; s < cp.steps; s += 2) {
+      step(c0);
+      step(c1);
+    }
+    tile_epilogue<MODE, false, kQWaves, TM, TN, true, kEpiReserve, true>(
+        cp, acc, stage_rows, wm * WTM, wave_col0, lane, lds_colscale + scale_buf * kScaleBufFloats,
+        lds_rowscale + scale_buf * kPBM);
+    // The load side is within the next tile here (every tile has at least
+    // kQMinSteps steps).
+    cp = ld;
+    if (!cp.valid) break;
+    nxt = fetch_tile(next_turn++);
+    // (buffers written here were last read a whole tile ago; the copies are older
+    // than every load of the coming steps, whose waits therefore cover them)
+    copy_bias(nxt, bias_buf);
+    bias_buf ^= 1;
+    scale_buf = scale_buf == 2 ? 0 : scale_buf + 1;          // the tile multiplied next
+    copy_colscale(nxt, scale_buf == 2 ? 0 : scale_buf + 1);  // the one after it
+    copy_rowscale(nxt, scale_buf == 2 ? 0 : scale_buf + 1);
+    init_acc(cp, bias_buf, scale_buf);
+    // The last half above already fetched these fragments; reading them again
+    // here keeps their registers free during the epilogue.
+    read_first_frags();
+  }
+}
+
+#endif  // DICE_PERSIST_F8
+
 // The kernels are thin wrappers: builtins and inline assembly that only exist
 // for the device must not appear in a __global__ template's own body, or the
 // host pass silently drops its definition.
@@ -1290,8 +1747,57 @@ __global__ __launch_bounds__(4 * kWave, 1) void gemm_persist_kernel4(PersistBatc
   gemm_persist64_body<MODE, HAS_BIAS, BN, GATHER, W8, REFILL>(batch);
 }
 
+#if DICE_PERSIST_F8
+// fp8 activations and weights (see gemm_persist_f8_body).
+template <int MODE, bool HAS_BIAS, bool REFILL>
+__global__ __launch_bounds__(4 * kWave, 1) void gemm_persist_kernel_f8(PersistBatch batch) {
+  gemm_persist_f8_body<MODE, HAS_BIAS, REFILL>(batch);
+}
+#endif
+
 }  // namespace
 
+#if DICE_PERSIST_F8
+int persist_cu_count();
+bool persist_fits_table(const PersistBatch &b, int mode);
+
+// fp8 activations: single-problem launches of contiguous rows, an even number
+// of 128-k steps, both scale tables, bf16 output.
+bool persist_f8_supported(const PersistBatch &b, int mode) {
+  if (b.n_problems != 1 || persist_cu_count() < kNumXcd) return false;
+  const PersistProblem &p = b.prob[0];
+  if (!p.a_scale || !p.w_scale || p.a_rows) return false;
+  if (p.n_experts < 1 || p.n_experts > kWave) return false;
+  if (p.k % 256 != 0 || p.k < 128 * kQMinSteps) return false;
+  if (p.n % 8 != 0 || p.lda % 16 != 0 || p.ldc % 8 != 0) return false;  // 16-byte loads and stores
+  if (mode == kFc1Swiglu && p.n % (kPBN / 2) != 0) return false;        // gate/up halves share one range check
+  if ((size_t)kPBM * p.lda >= (1ull << 31) || (size_t)kPBN * p.k >= (1ull << 31)) return false;
+  return true;
+}
+
+int launch_grouped_gemm_persist_f8(const PersistBatch &b, int mode, hipStream_t s) {
+  if (!persist_f8_supported(b, mode))
+    return fail(DICE_ERR_UNSUPPORTED, "fp8 expert GEMM: unsupported shape");
+  const int grid = persist_cu_count() / kNumXcd * kNumXcd;
+  const bool has_bias = mode != kFc1Swiglu && b.prob[0].bias != nullptr;
+  const bool refill = !persist_fits_table(b, mode);
+  void (*kern)(PersistBatch) = nullptr;
+  if (mode == kFc1Swiglu)
+    kern = refill ? gemm_persist_kernel_f8<kFc1Swiglu, false, true> : gemm_persist_kernel_f8<kFc1Swiglu, false, false>;
+  else if (mode == kFc1Gelu && has_bias)
+    kern = refill ? gemm_persist_kernel_f8<kFc1Gelu, true, true> : gemm_persist_kernel_f8<kFc1Gelu, true, false>;
+  else if (mode == kFc1Gelu)
+    kern = refill ? gemm_persist_kernel_f8<kFc1Gelu, false, true> : gemm_persist_kernel_f8<kFc1Gelu, false, false>;
+  else if (has_bias)
+    kern = refill ? gemm_persist_kernel_f8<kFc2, true, true> : gemm_persist_kernel_f8<kFc2, true, false>;
+  else
+    kern = refill ? gemm_persist_kernel_f8<kFc2, false, true> : gemm_persist_kernel_f8<kFc2, false, false>;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kQWaves * kWave), 0, s, b);
+  return launch_status("grouped_gemm_persist_f8");
+}
+
+}  // namespace dice
+#else  // !DICE_PERSIST_F8
 #if DICE_PERSIST_F16
 extern int g_persist_waves;
 int persist_variant(const PersistBatch &b, int mode);
@@ -1356,6 +1862,7 @@ bool persist64_fits_table(const PersistBatch &b, int mode) {
 bool persist64_ok(const PersistBatch &b, int mode) {
   for (int i = 0; i < b.n_problems; ++i) {
     const PersistProblem &p = b.prob[i];
+    if (p.a_scale) return false;  // fp8 activations: the kernel of the fp8 compilation unit
     if (p.k < kQBK * kQMinSteps) return false;
     if (p.w_scale && b.n_problems != 1) return false;  // fp8 weights: single-problem launches
     if (p.a_rows) {  // gathered activation rows: SwiGLU instantiation only (the GELU one would
@@ -1377,7 +1884,7 @@ int persist_variant(const PersistBatch &b, int mode) {
   if (!persist_common_ok(b, mode)) return 0;
   if (g_persist_waves == 4 && persist64_ok(b, mode)) return 4;
   for (int i = 0; i < b.n_problems; ++i)
-    if (b.prob[i].a_rows || b.prob[i].w_scale) return 0;  // the 32-k kernel wants contiguous rows and bf16 weights
+    if (b.prob[i].a_rows || b.prob[i].w_scale || b.prob[i].a_scale) return 0;  // the 32-k kernel wants contiguous rows and bf16 operands
   return 8;
 }
 
@@ -1449,3 +1956,4 @@ int DICE_PERSIST_LAUNCH(const PersistBatch &b, int mode, hipStream_t s) {
 }
 
 }  // namespace dice
+#endif  // !DICE_PERSIST_F8

@@ -37,6 +37,8 @@ struct LayerWorkspace {
   size_t dispatch_ws_bytes;
   void *h, *slot_out, *shared_h, *shared_out, *modulated;
   int32_t *shared_offsets;
+  uint8_t *q_rows;   // (act_quant) fp8 rows of the GEMM about to run: [slots, max(hidden, inter)]
+  float *q_scale;    // ... and their scales [slots]
   size_t total;
 };
 
@@ -63,6 +65,12 @@ LayerWorkspace carve_layer(const dice_moe_layer_t *L, int64_t n_tokens, void *ws
     w.shared_h = w.shared_out = nullptr;
   }
   w.modulated = c.take_bytes((size_t)n_tokens * L->hidden * es);  // layer input when the caller's prologue runs here
+  w.q_rows = nullptr;
+  w.q_scale = nullptr;
+  if (L->act_quant) {
+    w.q_rows = c.take<uint8_t>(slots * (size_t)(L->inter > L->hidden ? L->inter : L->hidden));
+    w.q_scale = c.take<float>(slots);
+  }
   w.total = c.used;
   return w;
 }
@@ -116,6 +124,87 @@ int check_mlp_shape(const char *who, int act_dtype, int w_dtype, int act_variant
 
 }  // namespace
 }  // namespace dice
+
+namespace dice {
+namespace {
+// The two fp8 x fp8 problems of an expert MLP whose activations are quantised
+// per row on the way in: fc1 reads q_rows as [rows, hidden] bytes, fc2 as
+// [rows, inter] bytes (the buffer is re-used between the stages).
+void a8_problems(const int32_t *offsets, int n_experts, int64_t max_rows, int hidden, int inter, const void *w1,
+                 const float *b1, const void *w2, const float *b2, const float *w1_scale, const float *w2_scale,
+                 bool swiglu, void *h, void *out, const uint8_t *q_rows, const float *q_scale, PersistBatch *f1,
+                 PersistBatch *f2) {
+  *f1 = PersistBatch{};
+  *f2 = PersistBatch{};
+  f1->n_problems = f2->n_problems = 1;
+  f1->prob[0] = PersistProblem{q_rows, hidden, offsets, n_experts, w1, swiglu ? 2 * inter : inter, inter,
+                               swiglu ? nullptr : b1, h, inter, inter, hidden, (int)max_rows};
+  f2->prob[0] = PersistProblem{q_rows, inter, offsets, n_experts, w2, hidden, 0, swiglu ? nullptr : b2,
+                               out, hidden, hidden, inter, (int)max_rows};
+  f1->prob[0].w_scale = w1_scale;
+  f2->prob[0].w_scale = w2_scale;
+  f1->prob[0].a_scale = f2->prob[0].a_scale = q_scale;
+}
+
+// Stage 1: quantise the (gathered) input rows, fc1 + activation -> h (bf16).
+// Stage 2: quantise h, fc2 -> out.  `after_fc1` runs between the stages (the
+// layer call puts the shared expert's launches and its timer stamps there).
+template <typename Between>
+int mlp_a8_run(int stages, const void *x, const int32_t *perm, int slots_per_token, const int32_t *offsets,
+               int n_experts, int64_t max_rows, int hidden, int inter, const PersistBatch &f1, const PersistBatch &f2,
+               bool swiglu, void *h, uint8_t *q_rows, float *q_scale, hipStream_t s, Between between) {
+  const int m1 = swiglu ? kFc1Swiglu : kFc1Gelu;
+  int rc = DICE_OK;
+  if (stages & 1) {
+    rc = quantize_act_impl(x, DICE_BF16, perm, slots_per_token, offsets + n_experts, max_rows, hidden, q_rows,
+                           q_scale, s);
+    if (rc) return rc;
+    rc = launch_grouped_gemm_persist_f8(f1, m1, s);
+    if (rc) return rc;
+  }
+  rc = between();
+  if (rc) return rc;
+  if (stages & 2) {
+    rc = quantize_act_impl(h, DICE_BF16, nullptr, 1, offsets + n_experts, max_rows, inter, q_rows, q_scale, s);
+    if (rc) return rc;
+    rc = launch_grouped_gemm_persist_f8(f2, kFc2, s);
+  }
+  return rc;
+}
+}  // namespace
+}  // namespace dice
+
+extern "C" int dice_grouped_mlp_a8(int stages, const void *x, int act_dtype, const int32_t *perm,
+                                   int slots_per_token, const int32_t *offsets, int n_experts,
+                                   int64_t max_rows, int hidden, int inter, const void *w1, const float *b1,
+                                   const void *w2, const float *b2, const float *w1_scale,
+                                   const float *w2_scale, int act_variant, void *h, void *out,
+                                   uint8_t *q_rows, float *q_scale, void *stream) {
+  using namespace dice;
+  DICE_REQUIRE(x && offsets && w1 && w2 && h && out && q_rows && q_scale && w1_scale && w2_scale, DICE_ERR_BAD_ARG,
+               "dice_grouped_mlp_a8: null pointer");
+  DICE_REQUIRE(stages >= 1 && stages <= 3, DICE_ERR_BAD_ARG, "dice_grouped_mlp_a8: stages %d (1 = fc1, 2 = fc2, 3 = both)",
+               stages);
+  DICE_REQUIRE(act_dtype == DICE_BF16, DICE_ERR_UNSUPPORTED, "dice_grouped_mlp_a8: act_dtype %d (BF16)", act_dtype);
+  int rc = check_mlp_shape("dice_grouped_mlp_a8", act_dtype, DICE_FP8_E4M3, act_variant, hidden, inter, n_experts);
+  if (rc) return rc;
+  DICE_REQUIRE(max_rows >= 0 && max_rows < (1ll << 31) &&
+                   max_rows * (int64_t)(inter > hidden ? inter : hidden) < (1ll << 31),
+               DICE_ERR_BAD_ARG, "dice_grouped_mlp_a8: max_rows %lld", (long long)max_rows);
+  DICE_REQUIRE(!perm || slots_per_token >= 1, DICE_ERR_BAD_ARG, "dice_grouped_mlp_a8: slots_per_token %d",
+               slots_per_token);
+  if (max_rows == 0) return DICE_OK;
+  const bool swiglu = act_variant == DICE_ACT_SWIGLU;
+  PersistBatch f1, f2;
+  a8_problems(offsets, n_experts, max_rows, hidden, inter, w1, b1, w2, b2, w1_scale, w2_scale, swiglu, h, out,
+              q_rows, q_scale, &f1, &f2);
+  DICE_REQUIRE(persist_f8_supported(f1, swiglu ? kFc1Swiglu : kFc1Gelu) && persist_f8_supported(f2, kFc2),
+               DICE_ERR_UNSUPPORTED,
+               "dice_grouped_mlp_a8: hidden %d and inter %d must be multiples of 256 (at least 768), n_experts %d at most 64",
+               hidden, inter, n_experts);
+  return mlp_a8_run(stages, x, perm, slots_per_token, offsets, n_experts, max_rows, hidden, inter, f1, f2, swiglu, h,
+                    q_rows, q_scale, (hipStream_t)stream, [] { return (int)DICE_OK; });
+}
 
 namespace dice {
 namespace {
@@ -286,6 +375,11 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
     DICE_REQUIRE(L->shared_w1 && L->shared_w2 && L->shared_inter % 64 == 0, DICE_ERR_BAD_ARG,
                  "%s: shared expert weights / shared_inter %d", who, L->shared_inter);
   }
+  if (L->act_quant || LE->act_quant)
+    DICE_REQUIRE(L->act_quant == 1 && LE->act_quant == 1 && L->act_dtype == DICE_BF16 &&
+                     LE->w_dtype == DICE_FP8_E4M3 && LE->w1_scale && LE->w2_scale,
+                 DICE_ERR_UNSUPPORTED,
+                 "%s: act_quant (0 or 1) needs bf16 activations and fp8 expert weights with scales, in both layers", who);
   if (combine_mode == 1)
     DICE_REQUIRE(skip_mask && cache_out, DICE_ERR_BAD_ARG, "%s: a put step needs skip_mask and cache_out", who);
   if (combine_mode == 2)
@@ -384,7 +478,47 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
   // (bf16) gets launches of its own.
   bool done = false;
   const bool w8 = LE->w_dtype == DICE_FP8_E4M3;
-  if (is_16bit(L->act_dtype) && (LE->w_dtype == L->act_dtype || (w8 && LE->w1_scale && LE->w2_scale))) {
+  if (LE->act_quant) {
+    // fp8 activations too: the routed experts run on the fp8 matrix pipe, each
+    // GEMM behind a quantiser of its input rows; the shared expert (bf16)
+    // keeps its own two launches.
+    const bool swiglu = L->act_variant == DICE_ACT_SWIGLU;
+    const int m1 = swiglu ? kFc1Swiglu : kFc1Gelu;
+    PersistBatch f1, f2, s1{}, s2{};
+    a8_problems(work.offsets, L->n_experts, max_rows, L->hidden, L->inter, LE->w1, LE->b1, LE->w2, LE->b2,
+                LE->w1_scale, LE->w2_scale, swiglu, w.h, work.rows, w.q_rows, w.q_scale, &f1, &f2);
+    DICE_REQUIRE(persist_f8_supported(f1, m1) && persist_f8_supported(f2, kFc2), DICE_ERR_UNSUPPORTED,
+                 "%s: act_quant needs hidden %d and inter %d to be multiples of 256 (at least 768)", who,
+                 L->hidden, L->inter);
+    if (L->shared_inter > 0) {
+      const int si = L->shared_inter;
+      s1.prob[0] = PersistProblem{x, L->hidden, w.shared_offsets, 1, L->shared_w1, swiglu ? 2 * si : si, si,
+                                  swiglu ? nullptr : L->shared_b1, w.shared_h, si, si, L->hidden, (int)n_tokens};
+      s2.prob[0] = PersistProblem{w.shared_h, si, w.shared_offsets, 1, L->shared_w2, L->hidden, 0,
+                                  swiglu ? nullptr : L->shared_b2, w.shared_out, L->hidden, L->hidden, si, (int)n_tokens};
+      s1.n_problems = s2.n_problems = 1;
+    }
+    const bool shared_persist = s1.n_problems && persist_supported(s1, m1) && persist_supported(s2, kFc2);
+    stamp(3, s);
+    rc = mlp_a8_run(3, work.x, work.perm, L->top_k, work.offsets, L->n_experts, max_rows, L->hidden, L->inter, f1,
+                    f2, swiglu, w.h, w.q_rows, w.q_scale, s, [&]() -> int {
+                      int r = DICE_OK;
+                      if (shared_persist) r = launch_persist(s1, m1, L->act_dtype, s);
+                      stamp(4, s);
+                      return r;
+                    });
+    if (rc) return rc;
+    if (shared_persist) {
+      rc = launch_persist(s2, kFc2, L->act_dtype, s);
+    } else if (L->shared_inter > 0) {
+      rc = dice_grouped_mlp(x, L->act_dtype, nullptr, 1, w.shared_offsets, 1, n_tokens, L->hidden,
+                            L->shared_inter, L->shared_w1, L->shared_b1, L->shared_w2, L->shared_b2, nullptr,
+                            nullptr, L->act_dtype, L->act_variant, w.shared_h, w.shared_out, 0, stream);
+    }
+    if (rc) return rc;
+    stamp(5, s);
+    done = true;
+  } else if (is_16bit(L->act_dtype) && (LE->w_dtype == L->act_dtype || (w8 && LE->w1_scale && LE->w2_scale))) {
     const bool swiglu = L->act_variant == DICE_ACT_SWIGLU;
     const int m1 = swiglu ? kFc1Swiglu : kFc1Gelu;
     PersistBatch f1{}, f2{};

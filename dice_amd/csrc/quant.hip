@@ -1,4 +1,5 @@
-// Per-output-channel fp8 (OCP e4m3fn) quantiser for expert weights.
+// fp8 (OCP e4m3fn) quantisers: per output channel for expert weights, per row
+// (token) for the activations of the fp8 expert GEMMs.
 //
 // The reference has no fp8 path; the scheme is defined here:
 //   scale[r] = amax(|w[r,:]|) / 448   (1 when the row is all zero)
@@ -39,8 +40,112 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const T *__restrict_
   }
 }
 
+// Activation rows -> e4m3 with one scale per row, for the expert GEMMs that
+// multiply on the fp8 matrix pipe (build-defined, like the weight quantiser):
+//   amax = max |x[r,:]|;  scale[r] = amax / 448 (1 when the row is all zero)
+//   q[r,c] = e4m3fn(rne(x[r,c] * (448 / amax)))
+// (a multiplication by the reciprocal, not a division: one rounding of the
+// reciprocal, one of the product, both reproducible in fp32 anywhere).
+// One wavefront per output row; the row stays in registers between the max and
+// the conversion (CHUNKS 16-byte pieces per lane), so x is read once.  With a
+// row table the source row of output row r is perm[r] / slots_per_token: the
+// gather of the dispatch fused into the quantiser, output in grouped order.
+// Rows at and beyond *n_rows_dev (the device-side row count) are left alone.
+template <typename T, int CHUNKS>
+__global__ __launch_bounds__(256) void quantize_act_rows_kernel(const T *__restrict__ x, const int32_t *__restrict__ perm,
+                                                                int slots_per_token, const int32_t *__restrict__ n_rows_dev,
+                                                                int64_t max_rows, int cols, uint8_t *__restrict__ q,
+                                                                float *__restrict__ scale) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t r = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (r >= max_rows) return;
+  if (n_rows_dev && r >= *n_rows_dev) return;
+  int64_t src = r;
+  if (perm) {
+    const int slot = perm[r];
+    if (slot < 0) return;
+    src = slot / slots_per_token;
+  }
+  const u32x4_t *row = reinterpret_cast<const u32x4_t *>(x + src * cols);
+  const int n_chunks = cols / 8;  // 16-byte pieces of a row
+  u32x4_t v[CHUNKS];
+  float m = 0.f;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int i = c * kWave + lane;
+    v[c] = u32x4_t{0, 0, 0, 0};
+    if (i < n_chunks) v[c] = row[i];
+    const T *e = reinterpret_cast<const T *>(&v[c]);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(to_f32(e[j])));
+  }
+  m = wave_max(m);
+  const float inv = m > 0.f ? 448.0f / m : 1.0f;
+  if (lane == 0) scale[r] = m > 0.f ? m / 448.0f : 1.0f;
+  u32x2_t *qrow = reinterpret_cast<u32x2_t *>(q + r * cols);
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int i = c * kWave + lane;
+    const T *e = reinterpret_cast<const T *>(&v[c]);
+    float f[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f[j] = fminf(fmaxf(to_f32(e[j]) * inv, -448.f), 448.f);
+    u32x2_t o;
+    int w = 0;
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], w, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], w, true);
+    o[0] = (uint32_t)w;
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], w, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], w, true);
+    o[1] = (uint32_t)w;
+    if (i < n_chunks) qrow[i] = o;
+  }
+}
+
+template <typename T>
+int launch_quantize_act(const void *x, const int32_t *perm, int slots_per_token, const int32_t *n_rows_dev,
+                        int64_t max_rows, int cols, uint8_t *q, float *scale, hipStream_t s) {
+  const unsigned grid = (unsigned)((max_rows + 3) / 4);
+  const int per_lane = (cols / 8 + kWave - 1) / kWave;
+#define DICE_QA(C)                                                                                        \
+  hipLaunchKernelGGL((quantize_act_rows_kernel<T, C>), dim3(grid), dim3(256), 0, s, (const T *)x, perm, \
+                     slots_per_token, n_rows_dev, max_rows, cols, q, scale)
+  if (per_lane <= 2) DICE_QA(2);
+  else if (per_lane <= 4) DICE_QA(4);
+  else if (per_lane <= 8) DICE_QA(8);
+  else DICE_QA(16);
+#undef DICE_QA
+  return launch_status("dice_quantize_fp8_act");
+}
+
 }  // namespace
+
+int quantize_act_impl(const void *x, int in_dtype, const int32_t *perm, int slots_per_token,
+                      const int32_t *n_rows_dev, int64_t max_rows, int cols, uint8_t *q, float *scale,
+                      void *stream) {
+  DICE_REQUIRE(x && q && scale, DICE_ERR_BAD_ARG, "dice_quantize_fp8_act: null pointer");
+  DICE_REQUIRE(max_rows >= 0 && max_rows < (1ll << 31), DICE_ERR_BAD_ARG, "dice_quantize_fp8_act: max_rows %lld",
+               (long long)max_rows);
+  DICE_REQUIRE(cols > 0 && cols % 8 == 0 && cols <= 16 * 8 * kWave, DICE_ERR_UNSUPPORTED,
+               "dice_quantize_fp8_act: cols %d must be a positive multiple of 8, at most %d", cols, 16 * 8 * kWave);
+  DICE_REQUIRE(!perm || slots_per_token >= 1, DICE_ERR_BAD_ARG, "dice_quantize_fp8_act: slots_per_token %d",
+               slots_per_token);
+  if (max_rows == 0) return DICE_OK;
+  hipStream_t s = (hipStream_t)stream;
+  if (in_dtype == DICE_BF16)
+    return launch_quantize_act<bf16_t>(x, perm, slots_per_token, n_rows_dev, max_rows, cols, q, scale, s);
+  if (in_dtype == DICE_F16)
+    return launch_quantize_act<f16_t>(x, perm, slots_per_token, n_rows_dev, max_rows, cols, q, scale, s);
+  return fail(DICE_ERR_UNSUPPORTED, "dice_quantize_fp8_act: in_dtype %d (BF16 or F16)", in_dtype);
+}
+
 }  // namespace dice
+
+extern "C" int dice_quantize_fp8_act(const void *x, int in_dtype, const int32_t *perm, int slots_per_token,
+                                     const int32_t *n_rows_dev, int64_t max_rows, int cols, uint8_t *q,
+                                     float *scale, void *stream) {
+  return dice::quantize_act_impl(x, in_dtype, perm, slots_per_token, n_rows_dev, max_rows, cols, q, scale, stream);
+}
 
 extern "C" int dice_quantize_fp8_rowwise(const void *w, int in_dtype, int64_t rows, int64_t cols,
                                          uint8_t *q, float *scale, void *stream) {

@@ -44,6 +44,8 @@ EXPORTS = [
     "dice_profile_read",
     "dice_combine",
     "dice_quantize_fp8_rowwise",
+    "dice_quantize_fp8_act",
+    "dice_grouped_mlp_a8",
     "dice_moe_workspace_bytes",
     "dice_moe_forward",
     "dice_moe_forward_lagged",
@@ -69,6 +71,7 @@ class MoeLayerDesc(Structure):
         ("b1", c_void_p), ("b2", c_void_p), ("w1_scale", c_void_p), ("w2_scale", c_void_p),
         ("shared_w1", c_void_p), ("shared_w2", c_void_p),
         ("shared_b1", c_void_p), ("shared_b2", c_void_p),
+        ("act_quant", c_int32),
     ]
 
 
@@ -129,6 +132,13 @@ def load() -> ctypes.CDLL:
                                  c_void_p, c_int, c_int64, c_int, c_int, c_void_p]
     lib.dice_quantize_fp8_rowwise.restype = c_int
     lib.dice_quantize_fp8_rowwise.argtypes = [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p]
+    lib.dice_quantize_fp8_act.restype = c_int
+    lib.dice_quantize_fp8_act.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int64, c_int, c_void_p,
+                                          c_void_p, c_void_p]
+    lib.dice_grouped_mlp_a8.restype = c_int
+    lib.dice_grouped_mlp_a8.argtypes = [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int64, c_int,
+                                        c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
     lib.dice_moe_workspace_bytes.restype = c_size_t
     lib.dice_moe_workspace_bytes.argtypes = [POINTER(MoeLayerDesc), c_int64]
     lib.dice_moe_forward.restype = c_int
@@ -160,8 +170,8 @@ def load() -> ctypes.CDLL:
     lib.dice_profile_read.argtypes = [POINTER(c_float), c_int]
     lib.dice_set_gemm_config.restype = c_int
     lib.dice_set_gemm_config.argtypes = [c_int, c_int]
-    if lib.dice_abi_version() != 1:
-        raise DiceError(f"ABI version {lib.dice_abi_version()} != 1")
+    if lib.dice_abi_version() != 2:
+        raise DiceError(f"ABI version {lib.dice_abi_version()} != 2")
     _lib = lib
     return lib
 

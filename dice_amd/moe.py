@@ -196,6 +196,7 @@ class SparseMoeBlock(nn.Module):
         self.inter = inter
         self._packed: Optional[_Packed] = None
         self._fp8 = False
+        self._act_quant = False      # fp8 experts: activations quantised per row too (fp8 matrix pipe)
         self._desc = None
         self._ws = None
         self._spare_cache = None     # a skip-cache tensor a skip step has consumed: the next full step writes into it
@@ -260,9 +261,14 @@ class SparseMoeBlock(nn.Module):
         self._desc = None
         return p
 
-    def quantize_fp8(self):
-        """Switches the routed experts to e4m3 weights (build-defined path)."""
+    def quantize_fp8(self, activations: bool = False):
+        """Switches the routed experts to e4m3 weights (build-defined path).
+        ``activations=True`` also quantises the routed experts' input rows (per
+        token, dynamically, in front of each GEMM), so that the products run on
+        the fp8 matrix pipe; bf16 blocks whose widths are multiples of 256."""
         self.pack_weights(fp8=True)
+        self._act_quant = bool(activations)
+        self._desc = None
         return self
 
     def _ensure(self, x: torch.Tensor):
@@ -286,6 +292,7 @@ class SparseMoeBlock(nn.Module):
             d.w1_scale, d.w2_scale = ptr(p.w1_scale), ptr(p.w2_scale)
             d.shared_w1, d.shared_w2 = ptr(p.sw1), ptr(p.sw2)
             d.shared_b1, d.shared_b2 = ptr(p.sb1), ptr(p.sb2)
+            d.act_quant = int(self._act_quant and self._fp8)
             self._desc = d
         return self._desc
 

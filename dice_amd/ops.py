@@ -160,3 +160,42 @@ def quantize_fp8_rowwise(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     check(load().dice_quantize_fp8_rowwise(ptr(w), dtype_code(w.dtype), rows, cols, ptr(q), ptr(scale),
                                            stream_ptr()))
     return q.view(torch.float8_e4m3fn), scale
+
+
+def quantize_fp8_act(x: torch.Tensor, perm: Optional[torch.Tensor] = None, slots_per_token: int = 1,
+                     n_rows: Optional[torch.Tensor] = None, max_rows: Optional[int] = None
+                     ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-row e4m3fn quantisation of activation rows ``x [*, cols]`` (bf16 /
+    fp16), optionally gathered: output row r comes from row
+    ``perm[r] // slots_per_token``.  ``n_rows``: int32 device scalar, rows at and
+    beyond it are left untouched.  Returns ``(q float8_e4m3fn [max_rows, cols],
+    scale fp32 [max_rows])``; untouched rows read as zero bytes / scale 0."""
+    cols = x.shape[-1]
+    if max_rows is None:
+        max_rows = perm.numel() if perm is not None else x.shape[0]
+    q = torch.zeros((max_rows, cols), dtype=torch.uint8, device=x.device)
+    scale = torch.zeros((max_rows,), dtype=torch.float32, device=x.device)
+    check(load().dice_quantize_fp8_act(ptr(x), dtype_code(x.dtype), ptr(perm), slots_per_token, ptr(n_rows),
+                                       max_rows, cols, ptr(q), ptr(scale), stream_ptr()))
+    return q.view(torch.float8_e4m3fn), scale
+
+
+def grouped_mlp_a8(x: torch.Tensor, perm: Optional[torch.Tensor], slots_per_token: int,
+                   offsets: torch.Tensor, max_rows: int, w1: torch.Tensor, w2: torch.Tensor,
+                   w1_scale: torch.Tensor, w2_scale: torch.Tensor, variant: str = "swiglu", b1=None, b2=None,
+                   stages: int = 3, h: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None):
+    """Grouped expert MLP with e4m3 weights AND per-row e4m3 activations on the
+    fp8 matrix pipe (``dice_grouped_mlp_a8``).  Returns ``(out [max_rows, D]
+    grouped, h [max_rows, I])`` in bf16."""
+    e, d, inter = w2.shape
+    if h is None:
+        h = torch.empty((max(max_rows, 1), inter), dtype=x.dtype, device=x.device)
+    if out is None:
+        out = torch.zeros((max_rows, d), dtype=x.dtype, device=x.device)
+    q_rows = torch.empty((max(max_rows, 1), max(d, inter)), dtype=torch.uint8, device=x.device)
+    q_scale = torch.empty((max(max_rows, 1),), dtype=torch.float32, device=x.device)
+    check(load().dice_grouped_mlp_a8(
+        stages, ptr(x), dtype_code(x.dtype), ptr(perm), slots_per_token, ptr(offsets), e, max_rows, d, inter,
+        ptr(w1), ptr(b1), ptr(w2), ptr(b2), ptr(w1_scale), ptr(w2_scale), VARIANTS[variant], ptr(h), ptr(out),
+        ptr(q_rows), ptr(q_scale), stream_ptr()))
+    return out, h

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define DICE_MOE_ABI_VERSION 1
+#define DICE_MOE_ABI_VERSION 2
 
 /* element types */
 #define DICE_F32 0
@@ -202,6 +202,43 @@ int dice_quantize_fp8_rowwise(const void *w, int in_dtype, int64_t rows,
                               void *stream);
 
 /*
+ * Per-row fp8 quantiser for activations (build-defined, the reference has no
+ * fp8 path), with the dispatch gather fused in: for output row r < max_rows
+ *   src = perm ? perm[r] / slots_per_token : r     (rows with perm[r] < 0 and
+ *         rows >= *n_rows_dev, when that device pointer is given, are skipped)
+ *   amax = max |x[src,:]|;  scale[r] = amax/448 (1 if the row is all zero)
+ *   q[r,c] = e4m3fn(rne(x[src,c] * (448/amax)))
+ *   x [*, cols] in_dtype in {BF16, F16};  q [max_rows, cols] uint8;  scale [max_rows]
+ * cols % 8 == 0, cols <= 8192.
+ */
+int dice_quantize_fp8_act(const void *x, int in_dtype, const int32_t *perm,
+                          int slots_per_token, const int32_t *n_rows_dev,
+                          int64_t max_rows, int cols, uint8_t *q, float *scale,
+                          void *stream);
+
+/*
+ * dice_grouped_mlp with fp8 weights AND fp8 activations, on the fp8 matrix
+ * pipe (v_mfma_f32_32x32x64_f8f6f4): each GEMM is preceded by
+ * dice_quantize_fp8_act of its input rows (fc1: rows of x gathered through
+ * perm; fc2: rows of h), the fp32 sums are multiplied by the row's and the
+ * output channel's scale in the epilogue; h and out are BF16.  Same reference
+ * lines as dice_grouped_mlp (models.py:252-273, 368-377); the quantisation is
+ * build-defined.
+ *   stages   1 = fc1 (writes h), 2 = fc2 (reads h), 3 = both
+ *   q_rows   [max_rows, max(hidden, inter)] bytes of scratch (the fp8 rows)
+ *   q_scale  [max_rows] floats of scratch (their scales)
+ * Output rows are in grouped order.  Limits: act_dtype BF16, hidden and inter
+ * multiples of 256 and at least 768, n_experts <= 64.
+ */
+int dice_grouped_mlp_a8(int stages, const void *x, int act_dtype,
+                        const int32_t *perm, int slots_per_token,
+                        const int32_t *offsets, int n_experts, int64_t max_rows,
+                        int hidden, int inter, const void *w1, const float *b1,
+                        const void *w2, const float *b2, const float *w1_scale,
+                        const float *w2_scale, int act_variant, void *h,
+                        void *out, uint8_t *q_rows, float *q_scale, void *stream);
+
+/*
  * Whole layer.  Replaces SparseMoeBlock.forward, inference branch
  * (models.py:302-312,321-358) with moe_infer / moe_infer_ep as above:
  * gate -> dispatch -> grouped MLP (+ shared expert MLP) -> combine, enqueued
@@ -222,6 +259,13 @@ typedef struct dice_moe_layer {
   const float *b1, *b2, *w1_scale, *w2_scale;
   const void *shared_w1, *shared_w2; /* one expert, act_dtype */
   const float *shared_b1, *shared_b2;
+  int32_t act_quant;      /* 0: 16-bit activations (fp8 weights are widened and
+                           * multiplied on the 16-bit matrix pipe); 1: the routed
+                           * experts' activations are quantised per row to e4m3
+                           * on the way into each GEMM (dice_quantize_fp8_act)
+                           * and multiplied on the fp8 matrix pipe: needs
+                           * act_dtype BF16, w_dtype FP8_E4M3, hidden and inter
+                           * multiples of 256 */
 } dice_moe_layer_t;
 
 /* mode: 0 = plain step; 1 = full step that also writes cache_out ("put");

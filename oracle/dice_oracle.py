@@ -51,6 +51,12 @@ Pinning status (what independently fixes each function's result):
 * bf16 / fp8 variants   - no reference code or vector exists for them
                           ("parity unpinned" by the reference); they are the
                           same functions evaluated in that dtype.
+* ``quantize_fp8_act`` / - build-defined (the reference has no fp8 code): pinned
+  ``Fp8ActExpert``        by a brute-force nearest-code search over all 256
+                          e4m3 codes in numpy (ties to the even code), by
+                          amax -> +-448, zero rows, power-of-two scale
+                          invariance and idempotence; the expert by the float64
+                          product of the dequantised operands.
 """
 from __future__ import annotations
 
@@ -769,3 +775,63 @@ def quantize_fp8_rowwise(w: torch.Tensor):
 
 def dequantize_fp8_rowwise(q: torch.Tensor, scale: torch.Tensor, dtype=torch.float32):
     return (q.float() * scale[:, None]).to(dtype)
+
+
+def quantize_fp8_act(x: torch.Tensor):
+    """Per-row (per-token) dynamic quantisation of activations to OCP e4m3fn,
+    as the fp8 expert GEMMs take them: ``amax = max|row|``,
+    ``q = rne(row * (448 / amax))``, ``scale = amax / 448`` (1.0 and zeros for
+    an all-zero row).  The quotient ``448 / amax`` and the product are each
+    rounded once in fp32 (IEEE division, not reciprocal times 448).  Returns (q float8_e4m3fn [rows, cols], scale fp32 [rows])."""
+    xf = x.float()
+    amax = xf.abs().amax(dim=-1)
+    nz = amax > 0
+    one = torch.ones_like(amax)
+    # a true fp32 quotient: torch evaluates ``448.0 / amax`` (python scalar over
+    # tensor) as reciprocal times scalar, which rounds twice
+    inv = torch.where(nz, torch.full_like(amax, E4M3_MAX) / amax, one)
+    scale = torch.where(nz, amax / E4M3_MAX, one)
+    q = (xf * inv[:, None]).clamp(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn)
+    return q, scale
+
+
+class Fp8ActExpert:
+    """An expert whose two GEMMs take e4m3 weights (``quantize_fp8_rowwise``
+    of the master weights) AND e4m3 activations (``quantize_fp8_act`` of the
+    rows in front of each GEMM).  Products and sums in fp32, the row's and the
+    output channel's scale applied to the sums, the activation function in fp32,
+    one rounding to the activation dtype for ``h`` and for the output - the
+    arithmetic of the fp8 kernels.  Wraps a ``SwiGLUExpert`` or ``GeluExpert``."""
+
+    def __init__(self, master):
+        self.swiglu = isinstance(master, SwiGLUExpert)
+        if self.swiglu:
+            w1 = torch.cat([master.gate_proj, master.up_proj], 0)
+            w2 = master.down_proj
+            self.b1 = self.b2 = None
+        else:
+            w1, w2 = master.fc1_w, master.fc2_w
+            self.b1 = None if master.fc1_b is None else master.fc1_b.float()
+            self.b2 = None if master.fc2_b is None else master.fc2_b.float()
+        self.q1, self.s1 = quantize_fp8_rowwise(w1)
+        self.q2, self.s2 = quantize_fp8_rowwise(w2)
+
+    def hidden_act(self, x: torch.Tensor) -> torch.Tensor:
+        qx, sx = quantize_fp8_act(x)
+        a = (qx.float() @ self.q1.float().t()) * (sx[:, None] * self.s1[None, :])
+        if self.swiglu:
+            inter = a.shape[1] // 2
+            h = F.silu(a[:, :inter]) * a[:, inter:]
+        else:
+            if self.b1 is not None:
+                a = a + self.b1
+            h = F.gelu(a, approximate="tanh")
+        return h.to(x.dtype)
+
+    def __call__(self, x: torch.Tensor) -> torch.Tensor:
+        h = self.hidden_act(x)
+        qh, sh = quantize_fp8_act(h)
+        o = (qh.float() @ self.q2.float().t()) * (sh[:, None] * self.s2[None, :])
+        if self.b2 is not None:
+            o = o + self.b2
+        return o.to(x.dtype)

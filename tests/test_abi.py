@@ -24,14 +24,15 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(cdll, n), f"{n} declared in include/dice_moe.h but not exported"
     for n in lib.EXPORTS:
         assert n in names, f"{n} bound in python but not declared in the header"
-    assert cdll.dice_abi_version() == 1
+    assert cdll.dice_abi_version() == 2
 
 
 def test_layer_struct_matches_header_layout():
     from dice_amd.lib import MoeLayerDesc
-    # 10 int32 fields then 12 pointers, naturally aligned.
+    # 10 int32 fields, 12 pointers, one more int32 (+ padding), naturally aligned.
     assert MoeLayerDesc.gate_w.offset == 40
-    assert ctypes.sizeof(MoeLayerDesc) == 40 + 12 * 8
+    assert MoeLayerDesc.act_quant.offset == 40 + 12 * 8
+    assert ctypes.sizeof(MoeLayerDesc) == 40 + 12 * 8 + 8
 
 
 def test_lag_entry_and_caller_structs_match_header_layout():

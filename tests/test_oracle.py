@@ -231,6 +231,111 @@ def test_fp8_rowwise_quantiser_properties():
     assert ((deq - w).abs()[big] <= w.abs()[big] * 2 ** -4 + 1e-9).all()
 
 
+def _e4m3_codes():
+    """The 127 non-negative finite e4m3fn values by their bit pattern (float64)."""
+    c = np.arange(127)
+    e, m = c >> 3, c & 7
+    return np.where(e == 0, m * 2.0 ** -9, (1 + m / 8.0) * 2.0 ** (e.astype(np.float64) - 7))
+
+
+def _nearest_e4m3(p):
+    """Nearest code of every element of p (float64 magnitudes within 448), ties
+    to the even bit pattern: brute force over all codes."""
+    vals = _e4m3_codes()
+    d = np.abs(np.abs(p)[..., None] - vals)
+    best = d.argmin(-1)                               # first minimum = the lower code
+    nxt = np.minimum(best + 1, 126)
+    tie = (np.take_along_axis(d, nxt[..., None], -1)[..., 0] == d.min(-1)) & (nxt != best)
+    best = np.where(tie & (best % 2 == 1), nxt, best)
+    return (best | np.where(np.signbit(p), 128, 0)).astype(np.uint8)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fp8_act_quantiser_against_bruteforce(dtype):
+    """Bytes of ``quantize_fp8_act`` against a search over all e4m3 codes in
+    numpy (float32 quotient 448 / amax by IEEE division, float32 product, then
+    the nearest code, ties to even).  16-bit inputs are often simple fractions of
+    the row maximum, which puts products within an ulp of a tie: there a quotient
+    rounded twice (reciprocal times 448) picks the other code, and the last
+    assertion checks that these rows hold such elements."""
+    g = torch.Generator().manual_seed(384)
+    x = (torch.randn(67, 384, generator=g) * torch.logspace(-3, 2, 67)[:, None]).to(dtype)
+    x[3] = 0
+    q, s = O.quantize_fp8_act(x)
+    xn = x.float().numpy()
+    amax = np.abs(xn).max(1)
+    inv = np.where(amax > 0, np.float32(448.0) / np.where(amax > 0, amax, np.float32(1)), np.float32(1))
+    prod = (xn * inv[:, None].astype(np.float32)).astype(np.float32)
+    want = _nearest_e4m3(np.clip(prod.astype(np.float64), -448, 448))
+    got = q.view(torch.uint8).numpy()
+    zero = prod == 0                                  # the sign of a zero byte is not part of the contract
+    assert np.array_equal(got[~zero], want[~zero]) and not (got[zero] & 0x7f).any()
+    assert np.array_equal(s.numpy(), np.where(amax > 0, amax / np.float32(448.0), np.float32(1)).astype(np.float32))
+    inv2 = (np.float32(1) / np.where(amax > 0, amax, np.float32(1))).astype(np.float32) * np.float32(448.0)
+    prod2 = (xn * inv2[:, None].astype(np.float32)).astype(np.float32)
+    twice = _nearest_e4m3(np.clip(prod2.astype(np.float64), -448, 448))
+    assert (twice != want).any(), "no element near a tie: the data no longer tells the two quotients apart"
+
+
+def test_fp8_act_quantiser_properties():
+    g = torch.Generator().manual_seed(22)
+    x = torch.randn(33, 128, generator=g).bfloat16()
+    x[4] = 0
+    q, s = O.quantize_fp8_act(x)
+    assert q.dtype == torch.float8_e4m3fn and s.dtype == torch.float32 and s.shape == (33,)
+    assert s[4] == 1.0 and (q[4].float() == 0).all()
+    nz = torch.arange(33) != 4
+    assert (q.float().abs().amax(1)[nz] == 448).all()                 # the row maximum maps to +-448
+    # a power-of-two factor changes the scale by that factor and no byte
+    q2, s2 = O.quantize_fp8_act((x.float() * 8).bfloat16())
+    assert torch.equal(q2.view(torch.uint8), q.view(torch.uint8)) and torch.equal(s2[nz], s[nz] * 8)
+    # idempotence: codes times a power-of-two scale re-quantise to the same codes
+    y = (q.float() * 2.0 ** -5).bfloat16()                            # e4m3 values are exact in bf16
+    q3, s3 = O.quantize_fp8_act(y)
+    assert torch.equal(q3.view(torch.uint8)[nz], q.view(torch.uint8)[nz]) and (s3[nz] == 2.0 ** -5).all()
+    deq = q.float() * s[:, None]
+    assert ((deq - x.float()).abs() <= x.float().abs().amax(1, keepdim=True) * 2 ** -4).all()
+
+
+@pytest.mark.parametrize("variant", ["swiglu", "gelu_tanh"])
+def test_fp8_act_expert_is_the_product_of_dequantised_operands(variant):
+    """``Fp8ActExpert`` against float64 numpy on the dequantised operands: the
+    products of e4m3 codes are exact in float64, so only the rounding of ``h`` to
+    bf16 (re-done here from the float64 value) and of the output differ."""
+    D, I = 64, 128
+    p = O.make_block_params(D, 2, 1, I // D, n_shared=0, seed=5, dtype=torch.bfloat16, variant=variant)
+    ex = p.experts[0]
+    if variant == "gelu_tanh":
+        g = torch.Generator().manual_seed(6)
+        ex.fc1_b = (torch.randn(I, generator=g) * 0.1).bfloat16()
+        ex.fc2_b = (torch.randn(D, generator=g) * 0.1).bfloat16()
+    x = torch.randn(48, D, generator=torch.Generator().manual_seed(7)).bfloat16()
+    got_h = O.Fp8ActExpert(ex).hidden_act(x).float().numpy()
+    got = O.Fp8ActExpert(ex)(x).float().numpy()
+
+    def deq(t):
+        q, s = O.quantize_fp8_act(t)
+        return q.float().double().numpy() * s.double().numpy()[:, None]
+
+    def wdeq(w):
+        q, s = O.quantize_fp8_rowwise(w)
+        return q.float().double().numpy() * s.double().numpy()[:, None]
+
+    if variant == "swiglu":
+        a = deq(x) @ wdeq(torch.cat([ex.gate_proj, ex.up_proj], 0)).T
+        gate, up = a[:, :I], a[:, I:]
+        h = gate / (1 + np.exp(-gate)) * up
+        w2, b2 = ex.down_proj, 0.0
+    else:
+        a = deq(x) @ wdeq(ex.fc1_w).T + ex.fc1_b.double().numpy()
+        h = 0.5 * a * (1 + np.tanh(np.sqrt(2 / np.pi) * (a + 0.044715 * a ** 3)))
+        w2, b2 = ex.fc2_w, ex.fc2_b.double().numpy()
+    assert np.abs(got_h - h).max() <= np.abs(h).max() * 2 ** -8
+    # fc2 on the oracle's own h (its bf16 rounding is then shared)
+    out = deq(torch.from_numpy(got_h).bfloat16()) @ wdeq(w2).T + b2
+    assert np.abs(got - out).max() <= np.abs(out).max() * 2 ** -8
+
+
 # --------------------------------------------------------------------------- #
 # step-lagged expert parallelism (displaced / interweaved) on one worker
 # --------------------------------------------------------------------------- #
