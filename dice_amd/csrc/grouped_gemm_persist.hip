@@ -436,12 +436,17 @@ __device__ __forceinline__ f32x16_t acc_block(const f32x16_t &a) {
 // scale_lds[c - n0] (SwiGLU: gate columns first, the up columns 128 floats on).
 // HAS_ROW: the activations were fp8 with one scale per row; row m of the tile is
 // multiplied by rowscale_lds[m] as well.
+// BIAS_LDS: the bias of the tile's columns sits in LDS (bias_lds[c - n0]) and is
+// read four values at a time where it is added, instead of being held in
+// registers for the whole epilogue (HAS_BIAS) or folded into the accumulators.
 template <int MODE, bool HAS_BIAS, int WAVES, int TM, int TN, bool HAS_SCALE = false, int RESERVE = 0,
-          bool HAS_ROW = false>
+          bool HAS_ROW = false, bool BIAS_LDS = false>
 __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM][TN], unsigned char *stage,
                                               int wave_row0, int wave_col0, int lane,
                                               const float *scale_lds = nullptr,
-                                              const float *rowscale_lds = nullptr) {
+                                              const float *rowscale_lds = nullptr,
+                                              const float *bias_lds = nullptr) {
+  static_assert(!(HAS_BIAS && BIAS_LDS), "one source of the bias");
   using G = EpiGeom<MODE, WAVES, TM, TN, RESERVE>;
   constexpr bool SWIGLU = G::SWIGLU;
   constexpr int OUT_BLOCKS = G::OUT_BLOCKS, PITCH = G::PITCH, BAND = G::BAND;
@@ -477,7 +482,9 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
       sg *= row_scale;                                                                                \
       if (SWIGLU) su *= row_scale;                                                                    \
     }                                                                                                 \
-  }
+  }                                                                                                   \
+  f32x4_t sb;                                                                                         \
+  if (BIAS_LDS) sb = *reinterpret_cast<const f32x4_t *>(bias_lds + wave_col0 + (j) * 32 + frag_half * 4 + (q) * 8);
 #define DICE_EPI_VALUE(v, j, q, r)                          \
   do {                                                      \
     if (HAS_SCALE) v *= sg[r];                              \
@@ -487,6 +494,7 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
       v = silu_fast(v) * u;                                 \
     } else {                                                \
       if (HAS_BIAS) v += bias_v[j][(q) * 4 + (r)];          \
+      if (BIAS_LDS) v += sb[r];                             \
       if (MODE == kFc1Gelu) v = gelu_tanh_fast(v);          \
     }                                                       \
   } while (0)
@@ -1331,8 +1339,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
 //     two quarters of a step into LDS and issues the loads that refill those
 //     register stages.
 //   * The epilogue multiplies the fp32 sums by the row's and the column's scale
-//     (both staged in LDS a tile ahead); a bias enters the accumulators divided
-//     by both.
+//     and adds the bias (all three staged in LDS a tile ahead).
 //
 // Rows are contiguous (the quantiser writes the activations in grouped order),
 // the reduction length is a multiple of 256 (an even number of steps), weight
@@ -1383,11 +1390,11 @@ __device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) 
   constexpr int kFCopies = 2 * kCopiesA;
   constexpr int kScaleBufFloats = 256, kBiasBufFloats = 256;
   constexpr int kTableBytes = kTableTurns * kTileWords * 4;
-  // three buffers each for the column and the row scales: the epilogue of a tile
-  // reads them while the first wave, a little ahead, may already stage those of
-  // the tile after the next; the bias (read at the tile switch) needs two
+  // three buffers each for the column scales, the row scales and the bias: the
+  // epilogue of a tile reads them while the first wave, a little ahead, may
+  // already stage those of the tile after the next
   constexpr int kColScaleBytes = 3 * kScaleBufFloats * 4, kRowScaleBytes = 3 * kPBM * 4;
-  constexpr int kBiasBytes = HAS_BIAS ? 2 * kBiasBufFloats * 4 : 0;
+  constexpr int kBiasBytes = HAS_BIAS ? 3 * kBiasBufFloats * 4 : 0;
   constexpr int kEpiReserve = kTableBytes + kColScaleBytes + kRowScaleBytes + kBiasBytes;
   using Epi = EpiGeom<MODE, kQWaves, TM, TN, kEpiReserve>;
   static_assert(kQWaves * Epi::WAVE_BYTES + kEpiReserve <= kPStageArea, "no room beside the epilogue's staging rows");
@@ -1520,35 +1527,8 @@ __device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) 
 
   const int wave_col0 = SWIGLU ? wn * 64 : wn * 128;
   f32x16_t acc[TM][TN];
-  // Biased tiles start their accumulators from bias / (column scale * row scale):
-  // the epilogue multiplies the sums by both.
-  auto init_acc = [&](const Tile &t, int bbuf, int sbuf) {
-    if constexpr (HAS_BIAS) {
-      if (uni((int)(t.bias != nullptr))) {
-        float rinv[TM];
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          const float rs = lds_rowscale[sbuf * kPBM + wm * WTM + i * 32 + frag_row];
-          rinv[i] = rs > 0.f ? 1.0f / rs : 0.f;
-        }
-        const float *src = lds_bias + bbuf * kBiasBufFloats + wave_col0 + frag_half * 4;
-        const float *scl = lds_colscale + sbuf * kScaleBufFloats + wave_col0 + frag_half * 4;
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          f32x16_t b;
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const f32x4_t v = *reinterpret_cast<const f32x4_t *>(src + j * 32 + q * 8);
-            const f32x4_t sc = *reinterpret_cast<const f32x4_t *>(scl + j * 32 + q * 8);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) b[q * 4 + r] = sc[r] != 0.f ? v[r] / sc[r] : 0.f;
-          }
-#pragma unroll
-          for (int i = 0; i < TM; ++i) acc[i][j] = b * rinv[i];
-        }
-        return;
-      }
-    }
+  // (a bias is added in the epilogue, from LDS, behind the two scales)
+  auto init_acc = [&]() {
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -1562,7 +1542,7 @@ __device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) 
   PackedTile nxt = fetch_tile(next_turn++);
   Tile ld = unpack_tile(nxt);                     // tile being loaded
   if (!ld.valid) return;
-  int bias_buf = 0, scale_buf = 0;
+  int scale_buf = 0;                              // buffer of the scales and the bias of the tile being multiplied
   copy_colscale(nxt, 0);
   copy_rowscale(nxt, 0);
   copy_bias(nxt, 0);
@@ -1594,18 +1574,20 @@ __device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) 
       // from beyond the matrix.
       if (l < kCopiesA) {
         const uint32_t skip = (uint32_t)(32 * l) * uni(ld.a_pitch);
-        const uint32_t extent = uni(ld.a_bytes);
+        // (signed, both below 2^31: a scalar subtract and max; the unsigned form
+        // becomes a saturating vector subtract and the descriptor a per-lane value)
+        const int left = (int)uni(ld.a_bytes) - (int)skip;
         const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)(uni(ld.a) + skip), 0, extent > skip ? extent - skip : 0u, kRsrcFlags);
+            (void *)(uni(ld.a) + skip), 0, uni((uint32_t)(left > 0 ? left : 0)), kRsrcFlags);
         stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(rs, ld_voff_a, uni(ld_kt * kFBK), 0);
       } else {
         const int i = l - kCopiesA;
         const bool up_half = SWIGLU && 32 * i >= kPBN / 2;
         const int row = up_half ? 32 * i - kPBN / 2 : 32 * i;
         const uint32_t skip = (uint32_t)row * uni(ld.b_pitch);
-        const uint32_t extent = uni(ld.b_bytes);
+        const int left = (int)uni(ld.b_bytes) - (int)skip;
         const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)(uni(up_half ? ld.b1 : ld.b0) + skip), 0, extent > skip ? extent - skip : 0u, kRsrcFlags);
+            (void *)(uni(up_half ? ld.b1 : ld.b0) + skip), 0, uni((uint32_t)(left > 0 ? left : 0)), kRsrcFlags);
         stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(rs, ld_voff_b, uni(ld_kt * kFBK), 0);
       }
     }
@@ -1643,7 +1625,7 @@ __device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) 
   write_quarter(c1, c1);
   load_quarter(c1, c0);    // first half of step 3; the stage keeps quarters 2, 3 of step 1
   load_quarter(c1, c1);
-  init_acc(cp, 0, 0);
+  init_acc();
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   phase_barrier();
   read_first_frags();
@@ -1710,9 +1692,9 @@ __device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) 
       step(c0);
       step(c1);
     }
-    tile_epilogue<MODE, false, kQWaves, TM, TN, true, kEpiReserve, true>(
+    tile_epilogue<MODE, false, kQWaves, TM, TN, true, kEpiReserve, true, HAS_BIAS>(
         cp, acc, stage_rows, wm * WTM, wave_col0, lane, lds_colscale + scale_buf * kScaleBufFloats,
-        lds_rowscale + scale_buf * kPBM);
+        lds_rowscale + scale_buf * kPBM, lds_bias + scale_buf * kBiasBufFloats);
     // The load side is within the next tile here (every tile has at least
     // kQMinSteps steps).
     cp = ld;
@@ -1720,12 +1702,11 @@ __device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) 
     nxt = fetch_tile(next_turn++);
     // (buffers written here were last read a whole tile ago; the copies are older
     // than every load of the coming steps, whose waits therefore cover them)
-    copy_bias(nxt, bias_buf);
-    bias_buf ^= 1;
     scale_buf = scale_buf == 2 ? 0 : scale_buf + 1;          // the tile multiplied next
     copy_colscale(nxt, scale_buf == 2 ? 0 : scale_buf + 1);  // the one after it
     copy_rowscale(nxt, scale_buf == 2 ? 0 : scale_buf + 1);
-    init_acc(cp, bias_buf, scale_buf);
+    copy_bias(nxt, scale_buf == 2 ? 0 : scale_buf + 1);
+    init_acc();
     // The last half above already fetched these fragments; reading them again
     // here keeps their registers free during the epilogue.
     read_first_frags();

@@ -80,9 +80,14 @@ LayerWorkspace carve_layer(const dice_moe_layer_t *L, int64_t n_tokens, void *ws
 // "moe.gate" / "moe.mlp" / "moe.mlp_shared" (models.py:305,356,375;
 // cudaprof/prof.py:19-60).  Off by default; events are host objects created on
 // first use.
-constexpr int kStages = 6;
+// "moe.gather" is the gathered copy of the rows, or (fp8 activations) the
+// quantiser of the fc1 input, which gathers; "moe.quant_h" the quantiser of the
+// fc2 input.  The shared expert's stages are empty where its problems ride in
+// the routed experts' launches.
+constexpr int kStages = 9;
 const char *const kStageNames[kStages] = {"moe.gate", "moe.dispatch", "moe.gather", "moe.mlp.fc1",
-                                          "moe.mlp.fc2", "moe.combine"};
+                                          "moe.mlp.shared_fc1", "moe.quant_h", "moe.mlp.fc2",
+                                          "moe.mlp.shared_fc2", "moe.combine"};
 // A ring of event sets, one per timed call, so that a run of back-to-back calls
 // can be timed without a host synchronisation between them.
 constexpr int kTimerRing = 64;
@@ -147,26 +152,33 @@ void a8_problems(const int32_t *offsets, int n_experts, int64_t max_rows, int hi
 }
 
 // Stage 1: quantise the (gathered) input rows, fc1 + activation -> h (bf16).
-// Stage 2: quantise h, fc2 -> out.  `after_fc1` runs between the stages (the
-// layer call puts the shared expert's launches and its timer stamps there).
-template <typename Between>
+// Stage 2: quantise h, fc2 -> out.  `mark(i)` is called in front of launch i
+// (0 quantiser, 1 fc1, 2 what the caller runs between the stages, 3 quantiser,
+// 4 fc2) and `between` runs between the stages: the layer call puts the shared
+// expert's first launch and its timer stamps there.
+template <typename Between, typename Mark>
 int mlp_a8_run(int stages, const void *x, const int32_t *perm, int slots_per_token, const int32_t *offsets,
                int n_experts, int64_t max_rows, int hidden, int inter, const PersistBatch &f1, const PersistBatch &f2,
-               bool swiglu, void *h, uint8_t *q_rows, float *q_scale, hipStream_t s, Between between) {
+               bool swiglu, void *h, uint8_t *q_rows, float *q_scale, hipStream_t s, Between between, Mark mark) {
   const int m1 = swiglu ? kFc1Swiglu : kFc1Gelu;
   int rc = DICE_OK;
   if (stages & 1) {
+    mark(0);
     rc = quantize_act_impl(x, DICE_BF16, perm, slots_per_token, offsets + n_experts, max_rows, hidden, q_rows,
                            q_scale, s);
     if (rc) return rc;
+    mark(1);
     rc = launch_grouped_gemm_persist_f8(f1, m1, s);
     if (rc) return rc;
   }
+  mark(2);
   rc = between();
   if (rc) return rc;
   if (stages & 2) {
+    mark(3);
     rc = quantize_act_impl(h, DICE_BF16, nullptr, 1, offsets + n_experts, max_rows, inter, q_rows, q_scale, s);
     if (rc) return rc;
+    mark(4);
     rc = launch_grouped_gemm_persist_f8(f2, kFc2, s);
   }
   return rc;
@@ -203,7 +215,7 @@ extern "C" int dice_grouped_mlp_a8(int stages, const void *x, int act_dtype, con
                "dice_grouped_mlp_a8: hidden %d and inter %d must be multiples of 256 (at least 768), n_experts %d at most 64",
                hidden, inter, n_experts);
   return mlp_a8_run(stages, x, perm, slots_per_token, offsets, n_experts, max_rows, hidden, inter, f1, f2, swiglu, h,
-                    q_rows, q_scale, (hipStream_t)stream, [] { return (int)DICE_OK; });
+                    q_rows, q_scale, (hipStream_t)stream, [] { return (int)DICE_OK; }, [](int) {});
 }
 
 namespace dice {
@@ -499,15 +511,13 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
       s1.n_problems = s2.n_problems = 1;
     }
     const bool shared_persist = s1.n_problems && persist_supported(s1, m1) && persist_supported(s2, kFc2);
-    stamp(3, s);
-    rc = mlp_a8_run(3, work.x, work.perm, L->top_k, work.offsets, L->n_experts, max_rows, L->hidden, L->inter, f1,
-                    f2, swiglu, w.h, w.q_rows, w.q_scale, s, [&]() -> int {
-                      int r = DICE_OK;
-                      if (shared_persist) r = launch_persist(s1, m1, L->act_dtype, s);
-                      stamp(4, s);
-                      return r;
-                    });
+    rc = mlp_a8_run(
+        3, work.x, work.perm, L->top_k, work.offsets, L->n_experts, max_rows, L->hidden, L->inter, f1, f2, swiglu,
+        w.h, w.q_rows, w.q_scale, s,
+        [&]() -> int { return shared_persist ? launch_persist(s1, m1, L->act_dtype, s) : (int)DICE_OK; },
+        [&](int i) { stamp(2 + i, s); });   // stages 2..6: quantiser, fc1, shared fc1, quantiser, fc2
     if (rc) return rc;
+    stamp(7, s);
     if (shared_persist) {
       rc = launch_persist(s2, kFc2, L->act_dtype, s);
     } else if (L->shared_inter > 0) {
@@ -516,7 +526,7 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
                             nullptr, L->act_dtype, L->act_variant, w.shared_h, w.shared_out, 0, stream);
     }
     if (rc) return rc;
-    stamp(5, s);
+    stamp(8, s);
     done = true;
   } else if (is_16bit(L->act_dtype) && (LE->w_dtype == L->act_dtype || (w8 && LE->w1_scale && LE->w2_scale))) {
     const bool swiglu = L->act_variant == DICE_ACT_SWIGLU;
@@ -572,39 +582,50 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
       stamp(3, s);
       rc = launch_persist(f1, m1, L->act_dtype, s);
       if (rc) return rc;
+      stamp(4, s);
       if (s1.n_problems) {
         rc = launch_persist(s1, m1, L->act_dtype, s);
         if (rc) return rc;
       }
-      stamp(4, s);
+      stamp(5, s);
+      stamp(6, s);
       rc = launch_persist(f2, kFc2, L->act_dtype, s);
       if (rc) return rc;
+      stamp(7, s);
       if (s2.n_problems) {
         rc = launch_persist(s2, kFc2, L->act_dtype, s);
         if (rc) return rc;
       }
-      stamp(5, s);
+      stamp(8, s);
       done = true;
     }
   }
   if (!done) {
-    rc = dice_grouped_mlp(work.x, L->act_dtype, work.perm, L->top_k, work.offsets, L->n_experts, max_rows,
-                          L->hidden, L->inter, LE->w1, LE->b1, LE->w2, LE->b2, LE->w1_scale, LE->w2_scale,
-                          LE->w_dtype, L->act_variant, w.h, work.rows, 0, stream);
-    if (rc) return rc;
-    if (L->shared_inter > 0) {
-      rc = dice_grouped_mlp(x, L->act_dtype, nullptr, 1, w.shared_offsets, 1, n_tokens, L->hidden,
-                            L->shared_inter, L->shared_w1, L->shared_b1, L->shared_w2, L->shared_b2,
-                            nullptr, nullptr, L->act_dtype, L->act_variant, w.shared_h, w.shared_out, 0,
-                            stream);
+    // Every other case (fp32, shapes the persistent kernels do not take): the
+    // per-stage kernels, one launch per stage and expert set, each in its own
+    // timer stage.
+    const bool shared = L->shared_inter > 0;
+    for (int stage = 1; stage <= 2; ++stage) {
+      stamp(stage == 1 ? 3 : 6, s);
+      rc = grouped_mlp_impl(stage, work.x, L->act_dtype, work.perm, L->top_k, work.offsets, L->n_experts, max_rows,
+                            L->hidden, L->inter, LE->w1, LE->b1, LE->w2, LE->b2, LE->w1_scale, LE->w2_scale,
+                            LE->w_dtype, L->act_variant, w.h, work.rows, 0, stream);
       if (rc) return rc;
+      stamp(stage == 1 ? 4 : 7, s);
+      if (shared) {
+        rc = grouped_mlp_impl(stage, x, L->act_dtype, nullptr, 1, w.shared_offsets, 1, n_tokens, L->hidden,
+                              L->shared_inter, L->shared_w1, L->shared_b1, L->shared_w2, L->shared_b2, nullptr,
+                              nullptr, L->act_dtype, L->act_variant, w.shared_h, w.shared_out, 0, stream);
+        if (rc) return rc;
+      }
+      stamp(stage == 1 ? 5 : 8, s);
     }
   }
   rc = combine_impl(emit.rows, emit.inv_perm, combine_wt, w.shared_out, mask,
                     combine_mode == 2 ? cache_in : nullptr, combine_mode == 1 ? cache_out : nullptr, y,
                     L->act_dtype, n_tokens, L->top_k, L->hidden, resid, caller ? caller->gate : nullptr,
                     caller ? caller->tokens_per_sample : 1, stream);
-  if (done) stamp(6, s);
+  stamp(kStages, s);
   return rc;
 }
 }  // namespace
@@ -673,7 +694,7 @@ extern "C" int dice_profile_read(float *ms_out, int n) {
   using namespace dice;
   DICE_REQUIRE(ms_out && n >= kStages, DICE_ERR_BAD_ARG, "dice_profile_read: need room for %d stages", kStages);
   DICE_REQUIRE(g_timers.mode != 0 && g_timers.recorded > 0, DICE_ERR_BAD_ARG,
-               "dice_profile_read: no timed dice_moe_forward call (bf16 path) since dice_profile_enable");
+               "dice_profile_read: no timed dice_moe_forward call since dice_profile_enable or the last read");
   const int calls = g_timers.recorded;
   const int last = (g_timers.next + kTimerRing - 1) % kTimerRing;
   hipError_t e = hipEventSynchronize(g_timers.ev[last][g_timers.mode == 1 ? kStages : kFc1Stage + 1]);

@@ -378,14 +378,20 @@ int dice_moe_forward_lagged(const dice_moe_layer_t *layer, const dice_moe_layer_
  * Stage timers.  Replace the reference's CudaProfiler scopes around the MoE
  * layer ("moe.gate", "moe.mlp", "moe.mlp_shared": models.py:305,356,375;
  * cudaprof/prof.py:19-60, expertpara/prof_analyse.py:3-17).  When enabled,
- * dice_moe_forward (bf16 path) records HIP events on the caller's stream
+ * dice_moe_forward records HIP events on the caller's stream
  * between its launches (a ring of 64 event sets, so that back-to-back calls
  * need no host synchronisation in between); dice_profile_read waits for the
  * last one and returns, per stage, the mean elapsed milliseconds over the calls
- * made since the previous read (the most recent 64 at most).  on = 1 times
- * every stage; on = 2 only brackets "moe.mlp.fc1" (two events per call, for
- * timing the dominant launch inside a throughput measurement; the other
- * stages read as 0).
+ * made since the previous read (the most recent 64 at most).  Stages, one per
+ * launch: "moe.gate", "moe.dispatch", "moe.gather" (the gathered copy of the
+ * rows where one is made; with act_quant the quantiser of the fc1 input),
+ * "moe.mlp.fc1" (routed experts, and the shared expert where it rides in the
+ * same launch), "moe.mlp.shared_fc1" (its own launch: fp8 routed weights),
+ * "moe.quant_h" (act_quant: quantiser of the fc2 input), "moe.mlp.fc2",
+ * "moe.mlp.shared_fc2", "moe.combine"; a stage without a launch reads as the
+ * gap between two events.  on = 1 times every stage; on = 2 only brackets
+ * "moe.mlp.fc1" (two events per call, for timing the dominant launch inside a
+ * throughput measurement; the other stages read as 0).
  */
 int dice_profile_enable(int on);
 int dice_profile_stage_count(void);
