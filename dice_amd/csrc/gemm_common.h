@@ -168,9 +168,11 @@ constexpr int kMaxPersistProblems = 3;
 struct PersistBatch {
   int n_problems;
   PersistProblem prob[kMaxPersistProblems];
+  int band_tiles;  // tile order: m-tiles per band (a group with more is cut into bands); 0 = the default rule
 };
 bool persist_supported(const PersistBatch &b, int mode);
 int persist_cu_count();  // compute units of the current device
+int persist_band_tiles(int mode);  // tuning hook state: band height of the tile order for this stage (0 = default rule)
 bool gemm_config_allows_persistent(int mode);  // tuning hook state: no tiling of the permutation-addressed kernels is forced for this stage
 int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s);      // bf16
 int launch_grouped_gemm_persist_f16(const PersistBatch &b, int mode, hipStream_t s);  // fp16

@@ -187,8 +187,10 @@ __device__ __forceinline__ Tile unpack_tile(const PackedTile &pk) {
 struct TilePos {
   int m_tile, n_tile;
 };
-__device__ __forceinline__ TilePos tile_pos(int r, int mt, int nt) {
-  constexpr int kBandTiles = 8, kBandFrom = 12;
+// `band_tiles` > 0 (tuning hook) sets the band height for every group with more
+// m-tiles than that.
+__device__ __forceinline__ TilePos tile_pos(int r, int mt, int nt, int band_tiles) {
+  const int kBandTiles = band_tiles > 0 ? band_tiles : 8, kBandFrom = band_tiles > 0 ? band_tiles : 12;
   const int bands = mt > kBandFrom ? (mt + kBandTiles - 1) / kBandTiles : 1;
   const int band_m = (mt + bands - 1) / bands;          // m-tiles per band (the last may have fewer)
   const int per_band = band_m * nt > 0 ? band_m * nt : 1;
@@ -297,7 +299,7 @@ struct TileWalker {
       }
     }
     const int r = idc - base;
-    const TilePos tp = tile_pos(r, mt, (n + BN_OUT - 1) / BN_OUT);
+    const TilePos tp = tile_pos(r, mt, (n + BN_OUT - 1) / BN_OUT, batch.band_tiles);
     const int n_tile = tp.n_tile, m_tile = tp.m_tile;
     const int left = cnt - m_tile * kPBM;
     const int rows = left < kPBM ? left : kPBM;
@@ -361,7 +363,7 @@ struct TileWalker {
     const int base = __builtin_amdgcn_readlane(g_base, g);
     const PersistProblem &pr = batch.prob[pi];
     const int r = idc - base;
-    const TilePos tp = tile_pos(r, mt, (pr.n + BN_OUT - 1) / BN_OUT);
+    const TilePos tp = tile_pos(r, mt, (pr.n + BN_OUT - 1) / BN_OUT, batch.band_tiles);
     const int n_tile = tp.n_tile, m_tile = tp.m_tile;
     const int left = cnt - m_tile * kPBM;
     const int rows = left < kPBM ? left : kPBM;
@@ -1773,7 +1775,9 @@ int launch_grouped_gemm_persist_f8(const PersistBatch &b, int mode, hipStream_t 
     kern = refill ? gemm_persist_kernel_f8<kFc2, true, true> : gemm_persist_kernel_f8<kFc2, true, false>;
   else
     kern = refill ? gemm_persist_kernel_f8<kFc2, false, true> : gemm_persist_kernel_f8<kFc2, false, false>;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kQWaves * kWave), 0, s, b);
+  PersistBatch launch = b;
+  launch.band_tiles = persist_band_tiles(mode);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kQWaves * kWave), 0, s, launch);
   return launch_status("grouped_gemm_persist_f8");
 }
 
@@ -1932,7 +1936,9 @@ int DICE_PERSIST_LAUNCH(const PersistBatch &b, int mode, hipStream_t s) {
       return fail(DICE_ERR_LAUNCH, "persistent expert GEMM: LDS attribute: %s", hipGetErrorString(e));
     configured[slot] = true;
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(waves * kWave), dyn_lds, s, b);
+  PersistBatch launch = b;
+  launch.band_tiles = persist_band_tiles(mode);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(waves * kWave), dyn_lds, s, launch);
   return launch_status("grouped_gemm_persist");
 }
 
