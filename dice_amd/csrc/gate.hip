@@ -1,9 +1,10 @@
-// Router: fp32 logits -> softmax -> top-k, one wavefront per token.
+// Router: fp32 logits -> softmax -> top-k, one wavefront per 64 / E tokens.
 //
 // Replaces MoEGate.forward, inference branch (reference models.py:179-196).
 // HBM-bound: the only large operand is x, read exactly once (n_tokens*hidden
-// elements); the router matrix is staged once per workgroup in LDS.  Each wave
-// keeps 64/E tokens in flight so one LDS read of a router chunk feeds that many
+// elements); the router matrix comes from the vector cache, or, when it is too
+// large for that, from LDS, where each workgroup stages it once.  Each wave
+// keeps 64/E tokens in flight so one read of a router chunk feeds that many
 // dot-product updates.
 #include "common.h"
 
@@ -53,12 +54,13 @@ __device__ __forceinline__ float dot8<bf16_t, bf16_t>(const Vec8<bf16_t> &x, con
   return acc;
 }
 
-// Sums v[0..63] across the 64 lanes; lane l returns the total of v[l].  Each
-// step halves the values a lane keeps (the partner takes the other half), so
-// the whole reduction costs 63 lane exchanges instead of 64 x 6, and the
-// summation order is fixed.
-template <int HALF>
-__device__ __forceinline__ void reduce_transpose_step(float (&v)[64], int lane) {
+// Sums v[0..V-1] across the 64 lanes; lane l returns the total of v[l % V].
+// Each step halves the values a lane keeps (the partner takes the other half),
+// so the reduction over the low log2(V) lane bits costs V - 1 lane exchanges
+// instead of V x log2(V); the remaining lane bits (V < 64) take one plain
+// butterfly each.  The summation order is fixed.
+template <int HALF, int V>
+__device__ __forceinline__ void reduce_transpose_step(float (&v)[V], int lane) {
   const bool upper = lane & HALF;  // partner distance == number of values kept
 #pragma unroll
   for (int i = 0; i < HALF; ++i) {
@@ -67,31 +69,66 @@ __device__ __forceinline__ void reduce_transpose_step(float (&v)[64], int lane) 
     v[i] = keep + __shfl_xor(send, HALF, kWave);
   }
 }
-__device__ __forceinline__ float reduce_transpose64(float (&v)[64], int lane) {
-  reduce_transpose_step<32>(v, lane);
-  reduce_transpose_step<16>(v, lane);
-  reduce_transpose_step<8>(v, lane);
-  reduce_transpose_step<4>(v, lane);
-  reduce_transpose_step<2>(v, lane);
-  reduce_transpose_step<1>(v, lane);
-  return v[0];
+template <int HALF, int V>
+__device__ __forceinline__ void reduce_transpose_from(float (&v)[V], int lane) {
+  if constexpr (HALF >= 1) {
+    reduce_transpose_step<HALF, V>(v, lane);
+    reduce_transpose_from<HALF / 2, V>(v, lane);
+  }
+}
+template <int V>
+__device__ __forceinline__ float reduce_transpose(float (&v)[V], int lane) {
+  reduce_transpose_from<V / 2, V>(v, lane);
+  float r = v[0];
+#pragma unroll
+  for (int o = V; o < kWave; o <<= 1) r += __shfl_xor(r, o, kWave);
+  return r;
 }
 
-// One wavefront routes TOK = 64 / EP tokens at a time: lanes split the hidden
+// One wavefront routes TOK <= 64 / EP tokens at a time: lanes split the hidden
 // dimension, every lane accumulates all TOK x EP dot products, the transposing
-// reduction leaves lane t*EP + e with logit (t, e), and softmax / top-k then
-// run inside each group of EP lanes for all TOK tokens at once.
-template <typename XT, typename WT, int EP, bool W_IN_LDS>
+// reduction leaves lane t*EP + e (and, for TOK x EP < 64, its copies further up)
+// with logit (t, e), and softmax / top-k then run inside each group of EP lanes
+// for all TOK tokens at once.  (TOK = 64 / EP in every launch: a quarter of that
+// per wave, four times the waves, measured slower.)
+template <typename XT, typename WT, int EP, int TOK, bool W_IN_LDS>
 __global__ __launch_bounds__(kGateWaves *kWave) void gate_topk_kernel(
     const XT *__restrict__ x, const WT *__restrict__ w, const float *__restrict__ bias,
     int64_t n_tokens, int hidden, int n_experts, int top_k, int norm_topk,
     int32_t *__restrict__ topk_idx, int64_t *__restrict__ topk_idx64,
     float *__restrict__ topk_weight, float *__restrict__ logits_out) {
-  constexpr int TOK = kWave / EP;
+  constexpr int V = TOK * EP;  // dot products per lane
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const int chunks = hidden / 8;
+
+  const int my_tok = (lane % V) / EP, my_e = lane % EP;
+  const bool live = my_e < n_experts;
+  const int64_t groups = (n_tokens + TOK - 1) / TOK;
+  // A lane's share of a token row is every 64th 16-byte chunk.  Up to kBatch of
+  // them per token are requested at once (a whole 16-bit row up to hidden = 2048), so a
+  // group costs one memory round trip, not one per chunk; the first group's
+  // loads are issued before the router matrix is staged, the next group's before
+  // this group's reduction and softmax.
+  constexpr int kBatch = sizeof(XT) == 4 ? 2 : 4;  // (fp32 rows take twice the registers per chunk)
+  Vec8<XT> xv[kBatch][TOK];
+  auto load_batch = [&](int64_t g, int c0) {
+    const int64_t t0 = g * TOK;
+#pragma unroll
+    for (int r = 0; r < kBatch; ++r) {
+      const int c = c0 + r * kWave + lane;
+      if (c < chunks) {
+#pragma unroll
+        for (int t = 0; t < TOK; ++t) {
+          const int64_t tt = t0 + t < n_tokens ? t0 + t : n_tokens - 1;
+          xv[r][t] = load8(x + tt * hidden + (size_t)c * 8);
+        }
+      }
+    }
+  };
+  int64_t g = (int64_t)blockIdx.x * kGateWaves + wave;
+  if (g < groups) load_batch(g, 0);
 
   const WT *wsrc = w;
   if (W_IN_LDS) {
@@ -103,50 +140,44 @@ __global__ __launch_bounds__(kGateWaves *kWave) void gate_topk_kernel(
     wsrc = wl;
   }
 
-  const int my_tok = lane / EP, my_e = lane % EP;
-  const bool live = my_e < n_experts;
-  const int64_t groups = (n_tokens + TOK - 1) / TOK;
-  for (int64_t g = (int64_t)blockIdx.x * kGateWaves + wave; g < groups;
-       g += (int64_t)gridDim.x * kGateWaves) {
+  for (; g < groups; g += (int64_t)gridDim.x * kGateWaves) {
     const int64_t t0 = g * TOK;
-    float acc[64];
+    float acc[V];
 #pragma unroll
-    for (int i = 0; i < 64; ++i) acc[i] = 0.f;
-    const XT *xrow[TOK];
+    for (int i = 0; i < V; ++i) acc[i] = 0.f;
+    for (int c0 = 0; c0 < chunks; c0 += kBatch * kWave) {
+      if (c0 > 0) load_batch(g, c0);  // rows longer than one batch: the next piece, after the last was consumed
 #pragma unroll
-    for (int t = 0; t < TOK; ++t) {
-      const int64_t tt = t0 + t < n_tokens ? t0 + t : n_tokens - 1;
-      xrow[t] = x + tt * hidden;
-    }
-    // The token rows of the next 64-chunk stride are requested before this one is
-    // multiplied, so two rounds of loads are in flight (the kernel is a handful of
-    // dependent memory round trips long; the arithmetic is negligible).
-    Vec8<XT> xv[TOK], xnext[TOK];
-    if (lane < chunks) {
+      for (int r = 0; r < kBatch; ++r) {
+        const int c = c0 + r * kWave + lane;
+        if (c < chunks) {
+          // Router rows eight experts at a time: the eight reads are issued together
+          // and waited for once (experts past n_experts re-read the last row; their
+          // logits are discarded below), no branch per expert.
+          constexpr int EB = EP < 8 ? EP : 8;
 #pragma unroll
-      for (int t = 0; t < TOK; ++t) xnext[t] = load8(xrow[t] + lane * 8);
-    }
-    for (int c = lane; c < chunks; c += kWave) {
+          for (int e0 = 0; e0 < EP; e0 += EB) {
+            Vec8<WT> wv[EB];
 #pragma unroll
-      for (int t = 0; t < TOK; ++t) xv[t] = xnext[t];
-      if (c + kWave < chunks) {
+            for (int e = 0; e < EB; ++e) {
+              const int row = e0 + e < n_experts ? e0 + e : n_experts - 1;
+              wv[e] = load8(wsrc + ((size_t)row * chunks + c) * 8);
+            }
 #pragma unroll
-        for (int t = 0; t < TOK; ++t) xnext[t] = load8(xrow[t] + (c + kWave) * 8);
-      }
+            for (int e = 0; e < EB; ++e)
 #pragma unroll
-      for (int e = 0; e < EP; ++e) {
-        if (e < n_experts) {
-          const Vec8<WT> wv = load8(wsrc + ((size_t)e * chunks + c) * 8);
-#pragma unroll
-          for (int t = 0; t < TOK; ++t) acc[t * EP + e] = dot8<XT, WT>(xv[t], wv, acc[t * EP + e]);
+              for (int t = 0; t < TOK; ++t) acc[t * EP + e0 + e] = dot8<XT, WT>(xv[r][t], wv[e], acc[t * EP + e0 + e]);
+          }
         }
       }
     }
-    float logit = reduce_transpose64(acc, lane);
+    const int64_t g_next = g + (int64_t)gridDim.x * kGateWaves;
+    if (g_next < groups) load_batch(g_next, 0);
+    float logit = reduce_transpose<V>(acc, lane);
     if (live && bias) logit += bias[my_e];
     if (!live) logit = -INFINITY;
     const int64_t tok = t0 + my_tok;
-    const bool tok_ok = tok < n_tokens;
+    const bool tok_ok = tok < n_tokens && lane < V;  // (lanes from V on hold copies)
     if (logits_out && live && tok_ok) logits_out[tok * n_experts + my_e] = logit;
 
     // softmax inside the EP-lane group
@@ -200,8 +231,11 @@ int launch_gate(const void *x, const void *w, const float *bias, int64_t n_token
   int64_t blocks = (groups + kGateWaves - 1) / kGateWaves;
   if (blocks > 512) blocks = 512;
   if (blocks < 1) blocks = 1;
-  if (w_bytes <= 160 * 1024 - 1024) {
-    auto kern = gate_topk_kernel<XT, WT, EP, true>;
+  // A router matrix that fits the compute unit's vector cache beside the token
+  // rows streaming through it is read from there: staging it in LDS first puts a
+  // load, a store and a workgroup barrier in front of the first product.
+  if (w_bytes > 24 * 1024 && w_bytes <= 160 * 1024 - 1024) {
+    auto kern = gate_topk_kernel<XT, WT, EP, TOK, true>;
     if (w_bytes > 48 * 1024) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)w_bytes);
@@ -211,7 +245,7 @@ int launch_gate(const void *x, const void *w, const float *bias, int64_t n_token
                        (const XT *)x, (const WT *)w, bias, n_tokens, hidden, n_experts, top_k, norm,
                        idx, idx64, wt, logits);
   } else {
-    auto kern = gate_topk_kernel<XT, WT, EP, false>;
+    auto kern = gate_topk_kernel<XT, WT, EP, TOK, false>;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kGateWaves * kWave), 0, stream,
                        (const XT *)x, (const WT *)w, bias, n_tokens, hidden, n_experts, top_k, norm,
                        idx, idx64, wt, logits);
