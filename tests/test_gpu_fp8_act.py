@@ -206,3 +206,47 @@ def test_act_quant_needs_fp8_weights_and_bf16(dev):
     blk.quantize_fp8(activations=True)
     with pytest.raises(DiceError, match="act_quant"):
         blk(torch.zeros(1, 64, D, dtype=torch.float16, device=dev))
+
+
+def test_block_a8_step_lag_and_fused_caller(dev):
+    """The fp8 x fp8 experts behind the other two layer entry points: a
+    displaced (step-lagged) call returns, bit for bit, what the synchronous
+    fp8 block produced two steps earlier, and the fused-caller call equals
+    LayerNorm / modulate -> the same block -> gated residual done by hand."""
+    import torch.nn.functional as F
+    from dice_amd import ParaMode, diep
+    D, E, N = 1024, 8, 1024
+    p = O.make_block_params(D, E, 2, 4, None, seed=21, dtype=torch.bfloat16)
+    sync = block_from_params(p, D, "swiglu", torch.bfloat16, dev)
+    sync.quantize_fp8(activations=True)
+    pm = ParaMode(ep=True, ep_async=True, ep_async_mode="all")
+    lag = block_from_params(p, D, "swiglu", torch.bfloat16, dev, para_mode=pm)
+    lag.quantize_fp8(activations=True)
+    g = _gen(22)
+    xs = [torch.randn(1, N, D, generator=g).bfloat16().to(dev) for _ in range(4)]
+    plain = [sync(x).clone() for x in xs]
+    diep.ep_cache_init(cache_capacity=1)
+    diep.use_latest_expert_weights(False)
+    try:
+        for t, x in enumerate(xs):
+            if t == 0:
+                diep.diep_force_sync()
+                diep.ep_cache_clear()
+            y = lag(x)
+            if t == 0:
+                diep.diep_cancel_sync()
+            src = 0 if t < 2 else t - 2
+            assert torch.equal(y, plain[src]), f"step {t} should return step {src}"
+    finally:
+        diep.ep_cache_init(cache_capacity=1, noskip_step=1)
+        if diep.diep_forced_sync():
+            diep.diep_cancel_sync()
+    # fused caller: x + gate * moe(modulate(norm(x))) with the layer input rounded to bf16 in between
+    B, T = 4, N // 4
+    xb = xs[0].view(B, T, D)
+    shift, scale, gate = ((torch.randn(B, D, generator=g) * 0.3).bfloat16().to(dev) for _ in range(3))
+    got = sync.forward_modulated(xb, shift, scale, gate)
+    h = (F.layer_norm(xb.float(), (D,), None, None, 1e-6) * (1 + scale.float().unsqueeze(1))
+         + shift.float().unsqueeze(1)).bfloat16()
+    want = xb.float() + gate.float().unsqueeze(1) * sync(h).float()
+    assert rel_l2(got.float().cpu(), want.cpu()) < 5e-3          # one bf16 rounding of the sum apart
