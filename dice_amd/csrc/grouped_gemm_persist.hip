@@ -1315,7 +1315,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
 // which multiplies at twice the rate of the bf16 instruction.
 //
 // In bytes this is the 64-k pipeline above: rows of 128 bytes per step (now 128
-// k), two 64 KB LDS slots, operands staged through two register stages four
+// k), two 64 KB LDS slots, operands staged through register stages three
 // steps ahead, the same 256x256 tile, wave tile, epilogue and tile table - so
 // the bytes moved per matrix-pipe cycle are those of the bf16 kernel while every
 // byte carries twice the arithmetic.  What differs:
@@ -1325,6 +1325,9 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
 //     any assignment of k to (lane half, byte) works as long as both operands
 //     use the same one, here: half h of k-block kb takes the row's 16-byte
 //     chunks 4 kb + 2 h and 4 kb + 2 h + 1.
+//   * Three register stages instead of four: two for the weight rows (loaded two
+//     steps before they are written to LDS), one for the activation rows (one
+//     step), see load_quarter.
 //   * Fragments twice the size do not fit twice in the register file, so they
 //     are not double-buffered.  A step is two halves of 16 MFMAs (one per 64-k
 //     block), taken row block by row block; during a half the next half's
@@ -1565,9 +1568,15 @@ __device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) 
     }
   };
   // A step's loads in four quarters of four: the two halves of the activation
-  // rows, then the two halves of the weight rows.
+  // rows, then the two halves of the weight rows.  The weight rows of a step wait
+  // in one of two register stages (by the parity of the step) for two steps, the
+  // activation rows in a single stage for one: weight tiles stream from HBM and
+  // need the longer flight; the activation tiles of an expert are re-read for
+  // every n-tile and come from the L2.  A third stage of 32 registers more does
+  // not fit: the register allocator then keeps one or two loads of every step
+  // in scratch memory, and each such load drains the whole load queue twice.
   auto load_quarter = [&](auto stage_c, auto q_c) {
-    constexpr int P = decltype(stage_c)::value, Q = decltype(q_c)::value;
+    constexpr int Q = decltype(q_c)::value, P = Q < 2 ? 0 : decltype(stage_c)::value;
 #pragma unroll
     for (int l = 4 * Q; l < 4 * Q + 4; ++l) {
       // The row block of a load is folded into its descriptor (base moved on, extent
@@ -1594,12 +1603,13 @@ __device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) 
       }
     }
   };
-  auto write_quarter = [&](auto stage_c, auto q_c) {
-    constexpr int P = decltype(stage_c)::value, Q = decltype(q_c)::value;
+  // Quarter q of the register stage(s) into LDS slot SLOT.
+  auto write_quarter = [&](auto slot_c, auto q_c) {
+    constexpr int SLOT = decltype(slot_c)::value, Q = decltype(q_c)::value, P = Q < 2 ? 0 : SLOT;
 #pragma unroll
     for (int l = 4 * Q; l < 4 * Q + 4; ++l) {
       const int i = l < kCopiesA ? l : l - kCopiesA;
-      unsigned char *dst = (P == 0 ? lds_slot0 : lds_slot1) + (l < kCopiesA ? 0 : kPBM * 128) + i * 32 * 128 + wr_off;
+      unsigned char *dst = (SLOT == 0 ? lds_slot0 : lds_slot1) + (l < kCopiesA ? 0 : kPBM * 128) + i * 32 * 128 + wr_off;
       *reinterpret_cast<u32x4_any_t *>(dst) = stage_regs[P][l];
     }
   };
@@ -1616,17 +1626,16 @@ __device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) 
     for (int i = 0; i < TM; ++i) A[i] = read_a(c0, c0, i);
   };
 
-  // Prologue: steps 0 and 1 through the stages into the slots (of step 1 only
-  // the first two quarters: the rest follows during the first half of step 0, as
-  // in the steady state), step 2 and the first half of step 3 into the stages.
+  // Prologue: step 0 through the stages into slot 0, the activation rows of step
+  // 1 into slot 1 (its weight rows follow during the first half of step 0, as in
+  // the steady state), the weight rows of steps 1 and 2 and the activation rows of
+  // step 2 into the stages.  The load side then stands at step 3.
   load_step(c0);           // step 0
-  load_step(c1);           // step 1
   write_quarter(c0, c0); write_quarter(c0, c1); write_quarter(c0, c2); write_quarter(c0, c3);
-  load_step(c0);           // step 2
+  load_step(c1);           // step 1
   write_quarter(c1, c0);
   write_quarter(c1, c1);
-  load_quarter(c1, c0);    // first half of step 3; the stage keeps quarters 2, 3 of step 1
-  load_quarter(c1, c1);
+  load_step(c0);           // step 2
   init_acc();
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   phase_barrier();
@@ -1637,8 +1646,8 @@ __device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) 
 
   // One half of a step: the 16 MFMAs of the 64-k block whose fragments sit in W
   // and A, while the fragments of block RKB of slot RSLOT replace them, quarters
-  // WQ and WQ + 1 of register stage WSLOT go to LDS slot WSLOT and are loaded
-  // again for the step after next.  BARRIER: the workgroup barrier of the step
+  // WQ and WQ + 1 of their register stage go to LDS slot WSLOT and are loaded
+  // again for the step the load side stands at.  BARRIER: the workgroup barrier of the step
   // sits behind the first row block; everything but MFMAs follows it.
   auto half = [&](auto rslot_c, auto rkb_c, auto wslot_c, auto wq_c, auto barrier_c) {
     constexpr int WQ = decltype(wq_c)::value;
@@ -1683,12 +1692,14 @@ __device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) 
     auto step = [&](auto slot_c) {
       constexpr int S = decltype(slot_c)::value;
       const template_int<S ^ 1> other_c;
-      // first k-block; the other slot receives the second half of the next step
+      // first k-block; the other slot receives the weight rows of the next step,
+      // their stage the weight rows of the step the load side stands at
       half(slot_c, c1, other_c, c2, c0);
-      advance_copy();
-      // second k-block; behind its barrier this slot receives the first half of
-      // the step after next and the next step's first fragments are read
+      // second k-block; behind its barrier this slot receives the activation rows
+      // of the step after next, their stage those of the load side's step, and the
+      // next step's first fragments are read
       half(other_c, c0, slot_c, c0, c1);
+      advance_copy();
     };
     for (int s = 0; s < cp.steps; s += 2) {
       step(c0);
