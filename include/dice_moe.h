@@ -399,9 +399,12 @@ const char *dice_profile_stage_name(int i);
 int dice_profile_read(float *ms_out, int n);
 
 /*
- * Tuning hook, no counterpart in the reference: selects the tile shape of the
- * bf16/fp8 expert GEMMs per stage (0 = library default).  Process-wide; meant
- * for benchmarks that compare tilings, not for the drop-in path.
+ * Tuning hook, no counterpart in the reference: selects the kernel of the
+ * bf16/fp8 expert GEMMs per stage (0 = library default).  1..4 force a tiling
+ * of the permutation-addressed kernels; 20 restricts the persistent launches to
+ * the 32-k pipeline; 30 + b (b = 1..16) walks the persistent launches' tiles in
+ * bands of b m-tiles.  Process-wide; meant for benchmarks that compare kernels,
+ * not for the drop-in path.
  */
 int dice_set_gemm_config(int fc1_cfg, int fc2_cfg);
 
