@@ -1705,8 +1705,13 @@ __device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) 
       step(c0);
       step(c1);
     }
+    // (the lane number is made opaque here: every address the epilogue derives from
+    // it would otherwise be worked out once, ahead of the tile loop, and held in
+    // registers through the k-loop, which has none to spare)
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
     tile_epilogue<MODE, false, kQWaves, TM, TN, true, kEpiReserve, true, HAS_BIAS>(
-        cp, acc, stage_rows, wm * WTM, wave_col0, lane, lds_colscale + scale_buf * kScaleBufFloats,
+        cp, acc, stage_rows, wm * WTM, wave_col0, lane_e, lds_colscale + scale_buf * kScaleBufFloats,
         lds_rowscale + scale_buf * kPBM, lds_bias + scale_buf * kBiasBufFloats);
     // The load side is within the next tile here (every tile has at least
     // kQMinSteps steps).
