@@ -48,13 +48,25 @@ __global__ __launch_bounds__(kModWaves *kWave) void ln_modulate_kernel(
   for (int64_t t = (int64_t)blockIdx.x * kModWaves + wave; t < n_tokens;
        t += (int64_t)gridDim.x * kModWaves) {
     const Chunk<T> *row = x + t * chunks_per_row;
-    Chunk<T> v[MAXC];
-    float sum = 0.f;
+    const int64_t b = t / tokens_per_sample;
+    const Chunk<T> *sh = shift + b * chunks_per_row;
+    const Chunk<T> *sc = scale + b * chunks_per_row;
+    // Everything the row needs is requested at once (the sample's shift and
+    // scale rows with the token row): one memory round trip per token, not two.
+    Chunk<T> v[MAXC], ms[MAXC], mh[MAXC];
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
       const int c = lane + i * kWave;
       if (c < chunks_per_row) {
         v[i] = row[c];
+        ms[i] = sc[c];
+        mh[i] = sh[c];
+      }
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+      if (lane + i * kWave < chunks_per_row) {
 #pragma unroll
         for (int e = 0; e < N; ++e) sum += v[i].get(e);
       }
@@ -72,15 +84,12 @@ __global__ __launch_bounds__(kModWaves *kWave) void ln_modulate_kernel(
       }
     }
     const float rstd = 1.0f / sqrtf(wave_sum(sq) * inv_hidden + eps);
-    const int64_t b = t / tokens_per_sample;
-    const Chunk<T> *sh = shift + b * chunks_per_row;
-    const Chunk<T> *sc = scale + b * chunks_per_row;
     Chunk<T> *dst = out + t * chunks_per_row;
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
       const int c = lane + i * kWave;
       if (c < chunks_per_row) {
-        const Chunk<T> s = sc[c], h = sh[c];
+        const Chunk<T> s = ms[i], h = mh[i];
         Chunk<T> o;
 #pragma unroll
         for (int e = 0; e < N; ++e)
