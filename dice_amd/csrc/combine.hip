@@ -59,6 +59,14 @@ __global__ __launch_bounds__(256) void combine_kernel(
   float acc[Pack<T>::kN];
 #pragma unroll
   for (int e = 0; e < Pack<T>::kN; ++e) acc[e] = 0.f;
+  // (the rows that do not depend on the routing tables are requested first, so
+  // that they travel while the slot rows' addresses are still being looked up)
+  Pack<T> sh{}, res{}, gt{};
+  if (shared_out) sh = shared_out[i];
+  if (resid) {
+    res = resid[i];
+    gt = gate[(t / tokens_per_sample) * vec_per_row + c];
+  }
   for (int j = 0; j < top_k; ++j) {
     const int64_t s = t * top_k + j;
     const float w = topk_weight[s];
@@ -78,15 +86,12 @@ __global__ __launch_bounds__(256) void combine_kernel(
     for (int e = 0; e < Pack<T>::kN; ++e) acc[e] = fmaf(w, row.get(e), acc[e]);
   }
   if (shared_out) {
-    Pack<T> sh = shared_out[i];
 #pragma unroll
     for (int e = 0; e < Pack<T>::kN; ++e) acc[e] += sh.get(e);
   }
   if (resid) {
-    const Pack<T> r = resid[i];
-    const Pack<T> g = gate[(t / tokens_per_sample) * vec_per_row + c];
 #pragma unroll
-    for (int e = 0; e < Pack<T>::kN; ++e) acc[e] = fmaf(g.get(e), acc[e], r.get(e));
+    for (int e = 0; e < Pack<T>::kN; ++e) acc[e] = fmaf(gt.get(e), acc[e], res.get(e));
   }
   Pack<T> o;
 #pragma unroll
