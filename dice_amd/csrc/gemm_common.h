@@ -169,10 +169,18 @@ struct PersistBatch {
   int n_problems;
   PersistProblem prob[kMaxPersistProblems];
   int band_tiles;  // tile order: m-tiles per band (a group with more is cut into bands); 0 = the default rule
+  // Partial-tile slots (persist_split_ws_bytes() bytes) or NULL.  With slots, a
+  // single-problem fc2 launch whose tiles do not fill the workgroups' last turn
+  // cuts that turn's tiles along k, one piece per workgroup, and a second small
+  // launch adds the pieces up; without, every tile is multiplied whole.
+  void *split_ws;
 };
+constexpr int kPersistSplitSlots = 320;  // partial-tile slots: one per workgroup of a launch (one per compute unit)
+size_t persist_split_ws_bytes();         // kPersistSplitSlots tiles of 256 x 256 16-bit values
 bool persist_supported(const PersistBatch &b, int mode);
 int persist_cu_count();  // compute units of the current device
 int persist_band_tiles(int mode);  // tuning hook state: band height of the tile order for this stage (0 = default rule)
+bool persist_split_allowed();      // tuning hook state: fc2 launches of the layer call may cut their last turn along k
 bool gemm_config_allows_persistent(int mode);  // tuning hook state: no tiling of the permutation-addressed kernels is forced for this stage
 int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s);      // bf16
 int launch_grouped_gemm_persist_f16(const PersistBatch &b, int mode, hipStream_t s);  // fp16

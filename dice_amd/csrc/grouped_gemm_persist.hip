@@ -204,12 +204,49 @@ __device__ __forceinline__ TilePos tile_pos(int r, int mt, int nt, int band_tile
   return p;
 }
 
+// Split turn.  The tiles of an XCD's run rarely fill its last turn: with R tiles
+// left for W workgroups, W - R of them would idle for a whole tile.  Where the
+// launch allows it (PersistBatch::split_ws: a plain-epilogue launch, whose
+// products are linear in k) and R <= W / 2, the W workgroups are dealt out over
+// those R tiles - W / R of them per tile, one more for the first W % R tiles, at
+// most kSplitMaxWays - and each multiplies one piece of its tile's k range: runs
+// of an even number of steps, at least kSplitMinSteps, that differ by at most
+// two steps.  A piece writes its partial products, in the output type, to the
+// partial-tile slot of its workgroup, and persist_split_sum_kernel adds the slots
+// of a tile in fp32, in piece order, into the output rows.
+constexpr int kSplitMinSteps = 6;
+constexpr int kSplitMaxWays = 8;
+// One workgroup position of the split turn.
+struct SplitPiece {
+  int tile;    // index of the tile within the turn
+  int piece;   // which piece of it, 0 .. ways - 1
+  int ways;    // pieces of that tile; 0: this position idles
+  int first;   // position of the tile's first piece (pieces sit side by side)
+};
+// Steps [begin, begin + count) of piece `piece` of `ways` of a tile of `steps` steps.
+struct SplitRange {
+  int begin, count;
+};
+__device__ __forceinline__ SplitRange split_range(int steps, int piece, int ways) {
+  const int pairs = steps / 2, base = pairs / ways, rem = pairs % ways;
+  SplitRange r;
+  r.begin = 2 * (piece * base + (piece < rem ? piece : rem));
+  r.count = 2 * (base + (piece < rem ? 1 : 0));
+  return r;
+}
+
 template <int BN_OUT>
 struct TileWalker {
   int g_prob = 0, g_expert = 0, g_row0 = 0, g_cnt = 0, g_mt = 0, g_base = 0, g_end = 0;
-  int run_begin, run_end, wg_in_xcd, wgs_per_xcd;
+  int run_begin, run_end, wg_in_xcd, wgs_per_xcd, xcd_id;
+  int split_turn, split_left;   // the XCD's last, short turn and its tiles
+  int split_q, split_extra;     // positions per tile of that turn when it is cut: q + 1 for the first `extra` tiles, q for the rest
+  int split_cap;                // most pieces a tile's length allows; 0: the turn is not cut
 
-  __device__ __forceinline__ TileWalker(const PersistBatch &batch, int lane) {
+  __device__ __forceinline__ TileWalker(const PersistBatch &batch, int lane)
+      : TileWalker(batch, lane, (int)(blockIdx.x % kNumXcd), (int)(blockIdx.x / kNumXcd), (int)(gridDim.x / kNumXcd)) {}
+  // (as seen by workgroup `wg` of `wgs` of XCD `xcd` of the launch that multiplies)
+  __device__ __forceinline__ TileWalker(const PersistBatch &batch, int lane, int xcd, int wg, int wgs) {
     int g_nt = 0, g_k32 = 1, acc_groups = 0;
     for (int pi = 0; pi < batch.n_problems; ++pi) {
       const PersistProblem &pr = batch.prob[pi];
@@ -244,9 +281,9 @@ struct TileWalker {
     const int total_cost = __shfl(cinc, kWave - 1, kWave);
     // XCD x takes the tiles between the x-th and the (x+1)-th eighth of the total
     // COST, so that every XCD gets the same amount of work whatever the mix.
-    const int xcd = blockIdx.x % kNumXcd;
-    wg_in_xcd = uni((int)(blockIdx.x / kNumXcd));
-    wgs_per_xcd = uni((int)(gridDim.x / kNumXcd));
+    xcd_id = uni(xcd);
+    wg_in_xcd = uni(wg);
+    wgs_per_xcd = uni(wgs);
     auto boundary = [&](int x) {
       if (x >= kNumXcd) return total_tiles;
       const int target = (int)((long long)total_cost * x / kNumXcd);
@@ -260,6 +297,53 @@ struct TileWalker {
     };
     run_begin = uni(boundary(xcd));
     run_end = uni(boundary(xcd + 1));
+    const int len = run_end - run_begin;
+    split_turn = len / wgs_per_xcd;
+    split_left = len - split_turn * wgs_per_xcd;
+    split_q = split_extra = split_cap = 0;
+  }
+
+  // Decides whether the last turn is cut (launches with partial-tile slots
+  // carry one problem, so every tile has prob[0].k / bk steps).
+  __device__ __forceinline__ void plan_split(const PersistBatch &batch, int bk) {
+    split_q = split_extra = split_cap = 0;
+    if (batch.split_ws == nullptr || split_left <= 0) return;
+    const int q = wgs_per_xcd / split_left;
+    const int cap = batch.prob[0].k / bk / kSplitMinSteps;   // pieces of at least kSplitMinSteps steps
+    if (q < 2 || cap < 2) return;
+    split_cap = cap < kSplitMaxWays ? cap : kSplitMaxWays;
+    split_q = q;
+    split_extra = wgs_per_xcd - q * split_left;
+  }
+  // What position `w` of the cut turn multiplies.
+  __device__ __forceinline__ SplitPiece split_piece(int w) const {
+    const int wide = split_extra * (split_q + 1);
+    SplitPiece sp;
+    int width;
+    if (w < wide) {
+      sp.tile = w / (split_q + 1);
+      width = split_q + 1;
+      sp.first = sp.tile * width;
+    } else {
+      const int t = (w - wide) / split_q;
+      sp.tile = split_extra + t;
+      width = split_q;
+      sp.first = wide + t * width;
+    }
+    sp.piece = w - sp.first;
+    sp.ways = width < split_cap ? width : split_cap;
+    if (sp.tile >= split_left || sp.piece >= sp.ways) sp.ways = 0;
+    return sp;
+  }
+  // Position of the first piece of the turn's j-th tile and its number of pieces.
+  __device__ __forceinline__ SplitPiece split_tile(int j) const {
+    return split_piece(j < split_extra ? j * (split_q + 1) : split_extra * (split_q + 1) + (j - split_extra) * split_q);
+  }
+
+  // Partial-tile slot of workgroup position `w` of this XCD (kPBM rows of BN_OUT
+  // columns in the output type).
+  __device__ __forceinline__ uint64_t split_slot(const PersistBatch &batch, int w) const {
+    return (uint64_t)batch.split_ws + (uint64_t)(xcd_id * wgs_per_xcd + w) * (kPBM * BN_OUT * 2);
   }
 
   // Describes 64 of this workgroup's turns at once - lane r works out turn
@@ -270,11 +354,15 @@ struct TileWalker {
   // words 20/21 carry the address of the tile's per-row scales instead.
   __device__ __forceinline__ void build_table(const PersistBatch &batch, int lane, int bk,
                                               uint32_t *table, bool w8 = false, int turn0 = 0,
-                                              bool a8 = false) const {
+                                              bool a8 = false) {
+    plan_split(batch, bk);
     const int turn = turn0 + lane;  // entry `lane` of the table describes this turn
     const int w = (turn & 1) ? wgs_per_xcd - 1 - wg_in_xcd : wg_in_xcd;
-    const int id = run_begin + turn * wgs_per_xcd + w;
-    const bool valid = id < run_end;
+    // (the split turn: positions j S .. j S + S - 1 share the turn's j-th tile)
+    const bool cut = split_cap != 0 && turn == split_turn;
+    const SplitPiece sp = cut ? split_piece(w) : SplitPiece{0, 0, 0, 0};
+    const int id = run_begin + turn * wgs_per_xcd + (cut ? sp.tile : w);
+    const bool valid = id < run_end && (!cut || sp.ways != 0);
     const int idc = valid ? id : 0;
     int n_groups = 0;
     for (int pi = 0; pi < batch.n_problems; ++pi) n_groups += batch.prob[pi].n_experts;
@@ -309,17 +397,35 @@ struct TileWalker {
     // (fp8 weights: one byte per element, and word 22 carries the row of the
     // per-output-channel scale table instead of the gather's reciprocal, which a
     // single-problem launch takes from its arguments)
-    const uint32_t a_pitch = (uint32_t)lda * (a8 ? 1 : 2), b_pitch = (uint32_t)k * (w8 ? 1 : 2), c_pitch = (uint32_t)ldc * 2;
+    const uint32_t a_pitch = (uint32_t)lda * (a8 ? 1 : 2), b_pitch = (uint32_t)k * (w8 ? 1 : 2);
+    uint32_t c_pitch = (uint32_t)ldc * 2, c_extent = (uint32_t)rows * c_pitch;
     const uint64_t wexp = pw + (uint64_t)expert * w_rows * b_pitch;
     // Gathered rows are addressed from the start of the source matrix.
-    const uint64_t ptrs[5] = {prows ? pa : pa + (uint64_t)(row0 + m_tile * kPBM) * a_pitch, wexp + (uint64_t)n0 * b_pitch,
-                              wexp + (uint64_t)(up_offset + n0) * b_pitch,
-                              pc + (uint64_t)(row0 + m_tile * kPBM) * c_pitch,
-                              pbias ? pbias + ((uint64_t)expert * n) * sizeof(float) : 0};
+    uint64_t ptrs[5] = {prows ? pa : pa + (uint64_t)(row0 + m_tile * kPBM) * a_pitch, wexp + (uint64_t)n0 * b_pitch,
+                        wexp + (uint64_t)(up_offset + n0) * b_pitch,
+                        pc + (uint64_t)(row0 + m_tile * kPBM) * c_pitch,
+                        pbias ? pbias + ((uint64_t)expert * n) * sizeof(float) : 0};
+    int steps = k / bk;
+    if (cut && sp.ways != 0) {
+      // This position's piece of the tile: its run of steps (the k offset moves
+      // the operands' base addresses; range checks look at row offsets only), and
+      // the position's partial-tile slot as the output, addressed so that column
+      // n0 is the slot's first.  The bias rides on the first piece.
+      const SplitRange run = split_range(steps, sp.piece, sp.ways);
+      steps = run.count;
+      const uint32_t k0 = (uint32_t)(run.begin * bk);
+      ptrs[0] += (uint64_t)k0 * (a8 ? 1 : 2);
+      ptrs[1] += (uint64_t)k0 * (w8 ? 1 : 2);
+      ptrs[2] += (uint64_t)k0 * (w8 ? 1 : 2);
+      c_pitch = BN_OUT * 2;
+      c_extent = (uint32_t)rows * c_pitch + (uint32_t)n0 * 2;
+      ptrs[3] = split_slot(batch, w) - (uint64_t)n0 * 2;
+      if (sp.piece != 0) ptrs[4] = 0;
+    }
     const uint32_t a_extent = prows ? (uint32_t)a_src_rows * a_pitch : (uint32_t)rows * a_pitch;
     const uint32_t words[10] = {valid ? a_extent : 0u, a_pitch, valid ? (uint32_t)wrows * b_pitch : 0u,
-                                b_pitch, (uint32_t)rows * c_pitch, c_pitch, (uint32_t)n0, (uint32_t)n,
-                                (uint32_t)(k / bk), valid ? 1u : 0u};
+                                b_pitch, c_extent, c_pitch, (uint32_t)n0, (uint32_t)n,
+                                (uint32_t)steps, valid ? 1u : 0u};
     uint32_t *entry = table + lane * kTileWords;
 #pragma unroll
     for (int i = 0; i < 5; ++i) {
@@ -849,6 +955,7 @@ constexpr int kQWaves = 4;
 constexpr int kQSlotBytes = (kPBM + kPBN) * 128;   // 64 KB
 constexpr int kQRingBytes = 2 * kQSlotBytes;       // staging area follows
 constexpr int kQMinSteps = 6;                      // loads run four steps ahead, within the next tile
+static_assert(kSplitMinSteps >= kQMinSteps && kSplitMinSteps % 2 == 0, "a piece of a cut tile is a tile of its own");
 static_assert(kQRingBytes == kPRingBytes, "both pipelines share the LDS budget");
 
 __device__ __forceinline__ int qswizzle(int row) { return (row >> 1) & 7; }
@@ -1471,9 +1578,12 @@ __device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) 
       const uint64_t ptr = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane(pk.words, 9) << 32) |
                            (uint32_t)__builtin_amdgcn_readlane(pk.words, 8);
       const int n0 = __builtin_amdgcn_readlane(pk.words, 16), n = __builtin_amdgcn_readlane(pk.words, 17);
-      if (wave == 0 && ptr != 0) {
+      if (wave == 0) {
+        // A tile without a bias (the later pieces of a tile that is cut along k)
+        // gets zeros: a descriptor that covers no bytes.
         const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)(ptr + (uint64_t)n0 * 4), 0, (uint32_t)(n - n0) * 4, kRsrcFlags);
+            ptr != 0 ? (void *)(ptr + (uint64_t)n0 * 4) : (void *)batch.prob[0].w_scale, 0,
+            ptr != 0 ? (uint32_t)(n - n0) * 4 : 0u, kRsrcFlags);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
             rs, (__attribute__((address_space(3))) void *)(lds_bias + buf * kBiasBufFloats), 16, lane * 16, 0, 0, 0);
       }
@@ -1733,6 +1843,74 @@ __device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) 
 
 #endif  // DICE_PERSIST_F8
 
+// Adds up the pieces of the tiles that the launch before it cut along k (see
+// TileWalker): workgroup (xcd, j, part) re-derives XCD xcd's split turn from the
+// same batch, and adds the partial-tile slots of its j-th tile, 16 rows per
+// workgroup, in fp32 and in piece order into the tile's output rows.  `wgs` is
+// the multiplying launch's workgroups per XCD, `bk` its k extent per step.
+// (Many small workgroups, every piece of a chunk requested at once: the kernel
+// moves a few tens of MB and is over in the time of a few memory round trips.)
+constexpr int kSplitSumParts = 16, kSplitSumRows = kPBM / kSplitSumParts;
+template <int BN_OUT>
+__device__ __forceinline__ void persist_split_sum_body(const PersistBatch &batch, int wgs, int bk) {
+  const int lane = threadIdx.x & 63;
+  const int part = blockIdx.x % kSplitSumParts;
+  const int j = (blockIdx.x / kSplitSumParts) % (wgs / 2);
+  const int xcd = blockIdx.x / kSplitSumParts / (wgs / 2);
+  TileWalker<BN_OUT> walk(batch, lane, xcd, 0, wgs);
+  walk.plan_split(batch, bk);
+  if (walk.split_cap == 0 || j >= walk.split_left) return;
+  const SplitPiece sp = walk.split_tile(j);
+  const Tile t = walk.decode(batch, walk.run_begin + walk.split_turn * wgs + j, bk);
+  if (!t.valid || sp.ways == 0) return;
+  constexpr int kChunks = BN_OUT / 8;  // 16-byte chunks per slot row
+  const int ways = sp.ways;
+  const unsigned char *slot0 = (const unsigned char *)walk.split_slot(batch, sp.first);
+  for (int idx = threadIdx.x; idx < kSplitSumRows * kChunks; idx += blockDim.x) {
+    const int r = part * kSplitSumRows + idx / kChunks, c = (idx % kChunks) * 8;
+    if (r >= t.rows || t.n0 + c >= t.n) continue;
+    h16x8_t v[kSplitMaxWays];
+#pragma unroll
+    for (int p = 0; p < kSplitMaxWays; ++p)
+      if (p < ways)
+        v[p] = *reinterpret_cast<const h16x8_t *>(slot0 + (size_t)p * (kPBM * BN_OUT * 2) +
+                                                  ((size_t)r * BN_OUT + c) * 2);
+    float sum[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sum[e] = 0.f;
+#pragma unroll
+    for (int p = 0; p < kSplitMaxWays; ++p)
+      if (p < ways) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sum[e] += (float)v[p][e];
+      }
+    h16x8_t o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (h16_t)sum[e];
+    *reinterpret_cast<h16x8_t *>(t.c + (size_t)r * t.c_pitch + (size_t)(t.n0 + c) * 2) = o;
+  }
+}
+template <int BN_OUT>
+__global__ __launch_bounds__(256) void persist_split_sum_kernel(PersistBatch batch, int wgs, int bk) {
+  persist_split_sum_body<BN_OUT>(batch, wgs, bk);
+}
+// Whether a launch of `grid` workgroups over batch `b` (one problem) can leave a
+// short last turn at all: a single group of known height whose tiles fill
+// every workgroup's turns exactly never does (the shared expert at round sizes).
+bool split_may_apply(const PersistBatch &b, int grid, int bn_out) {
+  const PersistProblem &p = b.prob[0];
+  if (p.n_experts != 1) return true;   // group heights live on the device
+  const int64_t tiles = ((int64_t)p.max_rows + kPBM - 1) / kPBM * ((p.n + bn_out - 1) / bn_out);
+  return tiles % grid != 0;
+}
+// Launches the sum for a multiplying launch of `grid` workgroups.
+template <int BN_OUT>
+void launch_split_sum(const PersistBatch &launch, int grid, int bk, hipStream_t s) {
+  const int wgs = grid / kNumXcd;
+  hipLaunchKernelGGL(persist_split_sum_kernel<BN_OUT>, dim3(kNumXcd * (wgs / 2) * kSplitSumParts), dim3(256), 0,
+                     s, launch, wgs, bk);
+}
+
 // The kernels are thin wrappers: builtins and inline assembly that only exist
 // for the device must not appear in a __global__ template's own body, or the
 // host pass silently drops its definition.
@@ -1793,7 +1971,11 @@ int launch_grouped_gemm_persist_f8(const PersistBatch &b, int mode, hipStream_t 
     kern = refill ? gemm_persist_kernel_f8<kFc2, false, true> : gemm_persist_kernel_f8<kFc2, false, false>;
   PersistBatch launch = b;
   launch.band_tiles = persist_band_tiles(mode);
+  // (a last turn cut along k: only the plain epilogue is linear in k)
+  if (mode != kFc2 || grid / kNumXcd < 2 || grid > kPersistSplitSlots || !split_may_apply(b, grid, kPBN))
+    launch.split_ws = nullptr;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kQWaves * kWave), 0, s, launch);
+  if (launch.split_ws) launch_split_sum<kPBN>(launch, grid, 128 /* k per step of the fp8 pipeline */, s);
   return launch_status("grouped_gemm_persist_f8");
 }
 
@@ -1890,6 +2072,7 @@ int persist_variant(const PersistBatch &b, int mode) {
 }
 
 bool persist_supported(const PersistBatch &b, int mode) { return persist_variant(b, mode) != 0; }
+size_t persist_split_ws_bytes() { return (size_t)kPersistSplitSlots * kPBM * kPBN * 2; }
 #endif  // !DICE_PERSIST_F16
 
 namespace {
@@ -1954,7 +2137,16 @@ int DICE_PERSIST_LAUNCH(const PersistBatch &b, int mode, hipStream_t s) {
   }
   PersistBatch launch = b;
   launch.band_tiles = persist_band_tiles(mode);
+  // (a last turn cut along k: the plain epilogue is linear in k; the 32-k kernel
+  // does not read its tiles from the table that describes the pieces)
+  if (mode != kFc2 || waves != 4 || b.n_problems != 1 || grid / kNumXcd < 2 || grid > kPersistSplitSlots ||
+      !split_may_apply(b, grid, narrow ? 192 : kPBN))
+    launch.split_ws = nullptr;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(waves * kWave), dyn_lds, s, launch);
+  if (launch.split_ws) {
+    if (narrow) launch_split_sum<192>(launch, grid, kQBK, s);
+    else launch_split_sum<kPBN>(launch, grid, kQBK, s);
+  }
   return launch_status("grouped_gemm_persist");
 }
 

@@ -37,6 +37,7 @@ struct LayerWorkspace {
   size_t dispatch_ws_bytes;
   void *h, *slot_out, *shared_h, *shared_out, *modulated;
   int32_t *shared_offsets;
+  void *split_ws;    // partial-tile slots of fc2 launches whose last turn is cut along k (16-bit activations)
   uint8_t *q_rows;   // (act_quant) fp8 rows of the GEMM about to run: [slots, max(hidden, inter)]
   float *q_scale;    // ... and their scales [slots]
   size_t total;
@@ -65,6 +66,7 @@ LayerWorkspace carve_layer(const dice_moe_layer_t *L, int64_t n_tokens, void *ws
     w.shared_h = w.shared_out = nullptr;
   }
   w.modulated = c.take_bytes((size_t)n_tokens * L->hidden * es);  // layer input when the caller's prologue runs here
+  w.split_ws = is_16bit(L->act_dtype) ? c.take_bytes(persist_split_ws_bytes()) : nullptr;
   w.q_rows = nullptr;
   w.q_scale = nullptr;
   if (L->act_quant) {
@@ -510,6 +512,7 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
                                   swiglu ? nullptr : L->shared_b2, w.shared_out, L->hidden, L->hidden, si, (int)n_tokens};
       s1.n_problems = s2.n_problems = 1;
     }
+    f2.split_ws = s2.split_ws = persist_split_allowed() ? w.split_ws : nullptr;
     const bool shared_persist = s1.n_problems && persist_supported(s1, m1) && persist_supported(s2, kFc2);
     rc = mlp_a8_run(
         3, work.x, work.perm, L->top_k, work.offsets, L->n_experts, max_rows, L->hidden, L->inter, f1, f2, swiglu,
@@ -561,6 +564,7 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
         f1.n_problems = f2.n_problems = 2;
       }
     }
+    f2.split_ws = s2.split_ws = persist_split_allowed() ? w.split_ws : nullptr;
     const bool shared_ok =
         s1.n_problems == 0 || (persist_supported(s1, m1) && persist_supported(s2, kFc2));
     // Where the kernel can address the activation rows through the permutation

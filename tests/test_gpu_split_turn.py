@@ -1,0 +1,124 @@
+"""The fc2 launch of the layer call cuts the tiles of a short last turn along k
+(each idle workgroup multiplies one piece; a small second launch adds the
+pieces in fp32): the same block with the cut switched off (tuning hook,
+fc2 = 50) must agree to the rounding of the 16-bit partial tiles, and both
+must meet the oracle (models.py:252-273, 292-296, 302-382) at the bar of the
+other block tests.
+
+Shapes are chosen so that every XCD's run leaves a handful of tiles for its
+32 workgroups (a few dozen tiles per launch, at least 12 steps per tile): the
+cut applies in every launch checked here, with even and uneven pieces, which
+the tests confirm by asking for outputs that are close but not bit-identical.
+"""
+import copy
+
+import pytest
+import torch
+
+from oracle import dice_oracle as O
+from tests.helpers import block_from_params, check_rows, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL, SAME_QUANT_TOL, FP8_TOL = 2e-2, 1e-2, 5e-2
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from dice_amd import lib
+    lib.load()
+    return torch.device("cuda:0")
+
+
+def _gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def _bias_params(p, seed, dtype=torch.bfloat16):
+    g = _gen(seed)
+    for e in list(p.experts) + ([p.shared] if p.shared is not None else []):
+        e.fc1_b = (torch.randn(e.fc1_b.shape, generator=g) * 0.1).to(dtype)
+        e.fc2_b = (torch.randn(e.fc2_b.shape, generator=g) * 0.1).to(dtype)
+    return p
+
+
+def _whole_and_cut(blk, x):
+    """The block's output with every fc2 tile multiplied whole, then with the
+    default schedule."""
+    from dice_amd import lib
+    lib.load().dice_set_gemm_config(0, 50)
+    try:
+        whole = blk(x).clone()
+    finally:
+        lib.load().dice_set_gemm_config(0, 0)
+    return whole.cpu(), blk(x).cpu()
+
+
+@pytest.mark.parametrize("variant,D,ratio,E,n_shared,N", [
+    ("swiglu", 768, 2, 4, 0, 1024),      # 192-wide fc2 tiles, no shared expert: one problem per launch
+    ("gelu_tanh", 768, 2, 4, 0, 1024),   # ... with biases: added by a tile's first piece only
+    ("gelu_tanh", 1024, 2, 4, 0, 1536),  # 256-wide fc2 tiles: the bias enters through the accumulators
+    ("swiglu", 1024, 3, 8, 0, 777),      # ragged groups, 48 steps
+    ("swiglu", 1152, 2, 8, 0, 2000),     # 36 steps in pieces of 8 to 14
+    ("gelu_tanh", 1152, 1, 4, 0, 900),   # 18 steps: at most three pieces of 6
+])
+def test_bf16_block_cut_last_turn(dev, variant, D, ratio, E, n_shared, N):
+    p = O.make_block_params(D, E, 2, ratio, n_shared, seed=21, dtype=torch.bfloat16, variant=variant)
+    if variant == "gelu_tanh":
+        _bias_params(p, 22)
+    x = torch.randn(1, N, D, generator=_gen(23)).bfloat16()
+    blk = block_from_params(p, D, variant, torch.bfloat16, dev)
+    whole, cut = _whole_and_cut(blk, x.to(dev))
+    want, _, _, logits = O.sparse_moe_block_forward(p, x)
+    ok = ~O.gate_tie_rows(logits, 2).view(-1)
+    check_rows(whole.view(-1, D)[ok], want.view(-1, D)[ok], BF16_TOL, "whole tiles vs oracle")
+    check_rows(cut.view(-1, D)[ok], want.view(-1, D)[ok], BF16_TOL, "cut last turn vs oracle")
+    assert not torch.equal(cut, whole), "the cut did not apply: the test's shape no longer exercises it"
+    check_rows(cut.view(-1, D), whole.view(-1, D), 4e-3, "cut last turn vs whole tiles")
+
+
+@pytest.mark.parametrize("variant", ["swiglu", "gelu_tanh"])
+@pytest.mark.parametrize("activations", [False, True])
+def test_fp8_block_cut_last_turn(dev, variant, activations):
+    """fp8 weights (bf16 matrix pipe) and fp8 weights x fp8 activations (fp8
+    matrix pipe), shared expert in launches of its own (which cut theirs too)."""
+    D, E, N = 1024, 8, 1280
+    p = O.make_block_params(D, E, 2, 3, 2, seed=31, dtype=torch.bfloat16, variant=variant)
+    if variant == "gelu_tanh":
+        _bias_params(p, 32)
+    x = torch.randn(1, N, D, generator=_gen(33)).bfloat16()
+    blk = block_from_params(p, D, variant, torch.bfloat16, dev)
+    blk.quantize_fp8(activations=activations)
+    whole, cut = _whole_and_cut(blk, x.to(dev))
+    if activations:   # against the oracle with the same quantisation
+        ref = copy.copy(p)
+        ref.experts = [O.Fp8ActExpert(e) for e in p.experts]
+        tol = SAME_QUANT_TOL
+    else:             # against the bf16 master weights
+        ref, tol = p, FP8_TOL
+    want, _, _, logits = O.sparse_moe_block_forward(ref, x)
+    ok = ~O.gate_tie_rows(logits, 2).view(-1)
+    check_rows(whole.view(-1, D)[ok], want.view(-1, D)[ok], tol, "whole tiles vs oracle")
+    check_rows(cut.view(-1, D)[ok], want.view(-1, D)[ok], tol, "cut last turn vs oracle")
+    assert not torch.equal(cut, whole), "the cut did not apply: the test's shape no longer exercises it"
+    check_rows(cut.view(-1, D), whole.view(-1, D), 4e-3, "cut last turn vs whole tiles")
+
+
+def test_cut_turn_is_deterministic_and_leaves_the_stage_calls_alone(dev):
+    """Two calls give the same bits (pieces are added in a fixed order), and a
+    skip step fed its own cache still reproduces the plain step."""
+    from dice_amd import lib
+    D, E, N = 768, 4, 1024
+    p = O.make_block_params(D, E, 2, 2, 0, seed=41, dtype=torch.bfloat16)
+    x = torch.randn(N, D, generator=_gen(42)).bfloat16().to(dev)
+    blk = block_from_params(p, D, "swiglu", torch.bfloat16, dev)
+    a = blk.run(x).clone()
+    b = blk.run(x).clone()
+    assert torch.equal(a, b)
+    mask = O.skip_mask(2 * N, "high").to(dev)
+    cache = torch.empty_like(x)
+    put = blk.run(x, lib.MODE_PUT, mask, None, cache).clone()
+    assert torch.equal(put, a)
+    skip = blk.run(x, lib.MODE_SKIP, mask, cache, None)
+    assert rel_l2(skip, a) < 4e-3   # (half the rows: another tile count, another cut)
