@@ -11,7 +11,11 @@
 // only one lane per expert touches the LDS counter.  The order inside an expert
 // group is therefore (span, round, lane) = ascending slot index: stable and
 // independent of any atomic's timing.  Integer/byte work, HBM traffic is
-// 4 B read + 8 B written per slot.
+// 4 B read + 8 B written per slot.  At the layer's sizes the kernels run for a
+// few microseconds and are bound by latency, not by bytes: a wave requests all
+// its slots (and its share of the count table) before it looks at any of them,
+// nothing branches around a load, and the code is kept short - such a kernel
+// spends a good part of its time fetching its own instructions.
 #include <mutex>
 
 #include "common.h"
@@ -23,7 +27,8 @@ constexpr int kMaxExperts = 256;
 constexpr int kFusedWaves = 16;       // single-workgroup path: 1024 threads
 constexpr int64_t kFusedMaxSlots = 2048;    // one workgroup, one launch: launch-latency bound sizes
 constexpr int kMidRounds = 4;               // two-launch path: 256 slots per wave
-constexpr int64_t kMidMaxTable = 1 << 16;   // ... while units x experts stays this small
+constexpr int64_t kMidMaxWork = 1 << 22;    // ... while every wave summing the whole table (units^2 x experts reads) stays
+                                            // cheaper than a third launch
 constexpr int kTileWaves = 4;         // multi-workgroup path: 256 threads
 constexpr int kTileRounds = 8;        // 512 slots per wave
 
@@ -45,53 +50,63 @@ struct SlotInfo {
   bool valid;     // in range, not skipped, expert id legal
 };
 
-__device__ __forceinline__ SlotInfo read_slot(const int32_t *idx, const uint8_t *skip,
-                                              int64_t n_slots, int n_experts, int64_t slot) {
-  SlotInfo s;
-  s.slot = slot;
-  s.in_range = slot < n_slots;
-  s.e = 0;
-  s.valid = false;
-  if (s.in_range) {
-    const int e = idx[slot];
-    const bool dropped = skip && skip[slot];
-    s.valid = !dropped && e >= 0 && e < n_experts;
-    s.e = s.valid ? e : 0;
+// A wave's span of ROUNDS x 64 slots, every round requested before the first is
+// used: one memory round trip for the span instead of one per round.
+template <int ROUNDS>
+__device__ __forceinline__ void read_span(const int32_t *idx, const uint8_t *skip, int64_t n_slots,
+                                          int n_experts, int64_t span_begin, int lane, SlotInfo (&s)[ROUNDS]) {
+  // (without a mask a byte of the index array is read and ignored: no branch around a load)
+  const uint8_t *mask = skip != nullptr ? skip : reinterpret_cast<const uint8_t *>(idx);
+  int e[ROUNDS];
+  uint8_t m[ROUNDS];
+#pragma unroll
+  for (int r = 0; r < ROUNDS; ++r) {
+    const int64_t slot = span_begin + (int64_t)r * kWave + lane;
+    const int64_t at = slot < n_slots ? slot : 0;   // slots past the end re-read slot 0
+    e[r] = idx[at];
+    m[r] = mask[at];
   }
-  return s;
+  // every load is on its way before the first value is looked at
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int r = 0; r < ROUNDS; ++r) {
+    s[r].slot = span_begin + (int64_t)r * kWave + lane;
+    s[r].in_range = s[r].slot < n_slots;
+    const bool dropped = (m[r] != 0) & (skip != nullptr);
+    s[r].valid = s[r].in_range && !dropped && e[r] >= 0 && e[r] < n_experts;
+    s[r].e = s[r].valid ? e[r] : 0;
+  }
 }
 
 // Adds this wave's per-expert counts over its span into row[] (LDS).
-__device__ __forceinline__ void count_span(const int32_t *idx, const uint8_t *skip, int64_t n_slots,
-                                           int n_experts, int nbits, int64_t span_begin, int rounds,
-                                           volatile int32_t *row, int lane) {
-  for (int r = 0; r < rounds; ++r) {
-    SlotInfo s = read_slot(idx, skip, n_slots, n_experts, span_begin + (int64_t)r * kWave + lane);
-    const uint64_t m = peers_of(s.e, s.valid, nbits);
-    if (s.valid && (__ffsll((unsigned long long)m) - 1) == lane) row[s.e] += __popcll(m);
-    __builtin_amdgcn_wave_barrier();
+template <int ROUNDS>
+__device__ __forceinline__ void count_span(const SlotInfo (&s)[ROUNDS], int nbits, int32_t *row, int lane) {
+#pragma unroll
+  for (int r = 0; r < ROUNDS; ++r) {
+    const uint64_t m = peers_of(s[r].e, s[r].valid, nbits);
+    if (s[r].valid && (__ffsll((unsigned long long)m) - 1) == lane) row[s[r].e] += __popcll(m);
+    wave_lds_sync();
   }
 }
 
 // Writes perm / inv_perm for this wave's span; row[] holds the next free
 // grouped position per expert and is advanced as the span is walked.
-__device__ __forceinline__ void rank_span(const int32_t *idx, const uint8_t *skip, int64_t n_slots,
-                                          int n_experts, int nbits, int64_t span_begin, int rounds,
-                                          volatile int32_t *row, int lane, int32_t *perm,
-                                          int32_t *inv_perm) {
+template <int ROUNDS>
+__device__ __forceinline__ void rank_span(const SlotInfo (&s)[ROUNDS], int nbits, int32_t *row, int lane,
+                                          int32_t *perm, int32_t *inv_perm) {
   const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-  for (int r = 0; r < rounds; ++r) {
-    SlotInfo s = read_slot(idx, skip, n_slots, n_experts, span_begin + (int64_t)r * kWave + lane);
-    const uint64_t m = peers_of(s.e, s.valid, nbits);
+#pragma unroll
+  for (int r = 0; r < ROUNDS; ++r) {
+    const uint64_t m = peers_of(s[r].e, s[r].valid, nbits);
     int pos = -1;
-    if (s.valid) pos = row[s.e] + __popcll(m & below);
-    __builtin_amdgcn_wave_barrier();
-    if (s.valid) {
-      perm[pos] = (int32_t)s.slot;
-      if ((__ffsll((unsigned long long)m) - 1) == lane) row[s.e] += __popcll(m);
+    if (s[r].valid) pos = row[s[r].e] + __popcll(m & below);
+    wave_lds_sync();
+    if (s[r].valid) {
+      perm[pos] = (int32_t)s[r].slot;
+      if ((__ffsll((unsigned long long)m) - 1) == lane) row[s[r].e] += __popcll(m);
     }
-    if (s.in_range) inv_perm[s.slot] = pos;
-    __builtin_amdgcn_wave_barrier();
+    if (s[r].in_range) inv_perm[s[r].slot] = pos;
+    wave_lds_sync();
   }
 }
 
@@ -106,7 +121,7 @@ __global__ __launch_bounds__(kFusedWaves *kWave) void dispatch_fused_kernel(
     int n_experts, int nbits, int rounds, int32_t *__restrict__ counts,
     int32_t *__restrict__ offsets, int32_t *__restrict__ perm, int32_t *__restrict__ inv_perm,
     int32_t *__restrict__ range_out, int32_t range_n) {
-  __shared__ volatile int32_t wrow[kFusedWaves][kMaxExperts];
+  __shared__ int32_t wrow[kFusedWaves][kMaxExperts];
   if (range_out && threadIdx.x == 0) {
     range_out[0] = 0;
     range_out[1] = range_n;
@@ -119,19 +134,33 @@ __global__ __launch_bounds__(kFusedWaves *kWave) void dispatch_fused_kernel(
 
   int code[MAXR];
 #pragma unroll
-  for (int r = 0; r < MAXR; ++r) {
-    const int64_t slot = begin + (int64_t)r * kWave + lane;
-    code[r] = -2;
-    if (r < rounds && slot < n_slots) {
-      const int e = idx[slot];
-      const bool dropped = skip && skip[slot];
-      code[r] = (!dropped && e >= 0 && e < n_experts) ? e : -1;
+  for (int r = 0; r < MAXR; ++r) code[r] = -2;
+  if (n_slots > 0) {  // (an empty call may come without an index array)
+    // No branch around a load (slots past the end re-read slot 0; without a mask a
+    // byte of the index array is read and ignored), and every load issued before
+    // the first value is looked at.
+    const uint8_t *mask = skip != nullptr ? skip : reinterpret_cast<const uint8_t *>(idx);
+    int e[MAXR];
+    uint8_t m[MAXR];
+#pragma unroll
+    for (int r = 0; r < MAXR; ++r) {
+      const int64_t slot = begin + (int64_t)r * kWave + lane;
+      const int64_t at = (r < rounds && slot < n_slots) ? slot : 0;
+      e[r] = idx[at];
+      m[r] = mask[at];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int r = 0; r < MAXR; ++r) {
+      const int64_t slot = begin + (int64_t)r * kWave + lane;
+      const bool dropped = (m[r] != 0) & (skip != nullptr);
+      if (r < rounds && slot < n_slots) code[r] = (!dropped && e[r] >= 0 && e[r] < n_experts) ? e[r] : -1;
     }
   }
 
   for (int e = lane; e < n_experts; e += kWave) wrow[wave][e] = 0;
   __syncthreads();
-  volatile int32_t *row = wrow[wave];
+  int32_t *row = wrow[wave];
 #pragma unroll
   for (int r = 0; r < MAXR; ++r) {
     if (r < rounds) {
@@ -139,7 +168,7 @@ __global__ __launch_bounds__(kFusedWaves *kWave) void dispatch_fused_kernel(
       const int e = valid ? code[r] : 0;
       const uint64_t m = peers_of(e, valid, nbits);
       if (valid && (__ffsll((unsigned long long)m) - 1) == lane) row[e] += __popcll(m);
-      __builtin_amdgcn_wave_barrier();
+      wave_lds_sync();
     }
   }
   __syncthreads();
@@ -191,31 +220,33 @@ __global__ __launch_bounds__(kFusedWaves *kWave) void dispatch_fused_kernel(
       const uint64_t m = peers_of(e, valid, nbits);
       int pos = -1;
       if (valid) pos = row[e] + __popcll(m & below);
-      __builtin_amdgcn_wave_barrier();
+      wave_lds_sync();
       if (valid) {
         perm[pos] = (int32_t)slot;
         if ((__ffsll((unsigned long long)m) - 1) == lane) row[e] += __popcll(m);
       }
       if (code[r] != -2) inv_perm[slot] = pos;
-      __builtin_amdgcn_wave_barrier();
+      wave_lds_sync();
     }
   }
   const int total = eoff[n_experts];
   for (int64_t i = total + threadIdx.x; i < n_slots; i += blockDim.x) perm[i] = -1;
 }
 
+template <int ROUNDS>
 __global__ __launch_bounds__(kTileWaves *kWave) void dispatch_count_kernel(
     const int32_t *__restrict__ idx, const uint8_t *__restrict__ skip, int64_t n_slots,
-    int n_experts, int nbits, int units, int rounds, int32_t *__restrict__ unit_cnt) {
-  __shared__ volatile int32_t wrow[kTileWaves][kMaxExperts];
+    int n_experts, int nbits, int units, int32_t *__restrict__ unit_cnt) {
+  __shared__ int32_t wrow[kTileWaves][kMaxExperts];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const int unit = blockIdx.x * kTileWaves + wave;
+  SlotInfo span[ROUNDS];
+  if (unit < units) read_span<ROUNDS>(idx, skip, n_slots, n_experts, (int64_t)unit * ROUNDS * kWave, lane, span);
   for (int e = lane; e < n_experts; e += kWave) wrow[wave][e] = 0;
   __syncthreads();
   if (unit < units) {
-    count_span(idx, skip, n_slots, n_experts, nbits, (int64_t)unit * rounds * kWave, rounds, wrow[wave],
-               lane);
+    count_span<ROUNDS>(span, nbits, wrow[wave], lane);
     for (int e = lane; e < n_experts; e += kWave) unit_cnt[(size_t)e * units + unit] = wrow[wave][e];
   }
 }
@@ -272,15 +303,17 @@ __global__ __launch_bounds__(kTileWaves *kWave) void dispatch_rank_kernel(
     int n_experts, int nbits, int units, const int32_t *__restrict__ unit_base,
     const int32_t *__restrict__ offsets, int32_t *__restrict__ perm,
     int32_t *__restrict__ inv_perm) {
-  __shared__ volatile int32_t wrow[kTileWaves][kMaxExperts];
+  __shared__ int32_t wrow[kTileWaves][kMaxExperts];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const int unit = blockIdx.x * kTileWaves + wave;
   if (unit >= units) return;
   for (int e = lane; e < n_experts; e += kWave) wrow[wave][e] = unit_base[(size_t)e * units + unit];
-  __builtin_amdgcn_wave_barrier();
+  wave_lds_sync();
   const int64_t begin = (int64_t)unit * kTileRounds * kWave;
-  rank_span(idx, skip, n_slots, n_experts, nbits, begin, kTileRounds, wrow[wave], lane, perm, inv_perm);
+  SlotInfo span[kTileRounds];
+  read_span<kTileRounds>(idx, skip, n_slots, n_experts, begin, lane, span);
+  rank_span<kTileRounds>(span, nbits, wrow[wave], lane, perm, inv_perm);
   const int total = offsets[n_experts];
   for (int r = 0; r < kTileRounds; ++r) {
     const int64_t i = begin + (int64_t)r * kWave + lane;
@@ -292,13 +325,13 @@ __global__ __launch_bounds__(kTileWaves *kWave) void dispatch_rank_kernel(
 // unit table itself - totals per expert for the offsets, and the counts of the
 // units before its own for its start positions - then ranks its unit.  The
 // table is units x experts integers, a few KB, and comes out of the L2.
+template <int ROUNDS>
 __global__ __launch_bounds__(kTileWaves *kWave) void dispatch_scan_rank_kernel(
     const int32_t *__restrict__ idx, const uint8_t *__restrict__ skip, int64_t n_slots,
-    int n_experts, int nbits, int units, int rounds, const int32_t *__restrict__ unit_cnt,
+    int n_experts, int nbits, int units, const int32_t *__restrict__ unit_cnt,
     int32_t *__restrict__ counts, int32_t *__restrict__ offsets, int32_t *__restrict__ perm,
     int32_t *__restrict__ inv_perm, int32_t *__restrict__ range_out, int32_t range_n) {
-  __shared__ volatile int32_t wrow[kTileWaves][kMaxExperts];
-  __shared__ int32_t wtot[kTileWaves][kMaxExperts];
+  __shared__ int32_t wrow[kTileWaves][kMaxExperts];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const int unit = blockIdx.x * kTileWaves + wave;
@@ -307,28 +340,45 @@ __global__ __launch_bounds__(kTileWaves *kWave) void dispatch_scan_rank_kernel(
     range_out[1] = range_n;
   }
   if (unit >= units) return;
+  // The wave's slots are requested first: they arrive while the table is summed.
+  const int64_t begin = (int64_t)unit * ROUNDS * kWave;
+  SlotInfo span[ROUNDS];
+  read_span<ROUNDS>(idx, skip, n_slots, n_experts, begin, lane, span);
   // per expert: total over all units and total over the units before this one.
   // The lanes read an expert's unit counts side by side (one coalesced load per
-  // 64 units) and reduce across the wave; lane e % 64 keeps expert e's sums.
+  // 64 units), eight experts' rows requested together, and reduce across the
+  // wave; lane e % 64 keeps expert e's sums.
+  constexpr int kRows = 8;
   int carry = 0;  // running exclusive offset over experts
   for (int c = 0; c < n_experts; c += kWave) {
     const int e = c + lane;
     int tot = 0, before = 0;
     const int chunk_experts = n_experts - c < kWave ? n_experts - c : kWave;
-    for (int ee = 0; ee < chunk_experts; ++ee) {
-      const int32_t *rowp = unit_cnt + (size_t)(c + ee) * units;
-      int t = 0, b = 0;
+    for (int ee0 = 0; ee0 < chunk_experts; ee0 += kRows) {
+      int t[kRows], b[kRows];
+#pragma unroll
+      for (int k = 0; k < kRows; ++k) t[k] = b[k] = 0;
       for (int u0 = 0; u0 < units; u0 += kWave) {
         const int u = u0 + lane;
-        const int v = u < units ? rowp[u] : 0;
-        t += v;
-        b += u < unit ? v : 0;
+        int v[kRows];
+#pragma unroll
+        for (int k = 0; k < kRows; ++k) {
+          const int ee = ee0 + k < chunk_experts ? ee0 + k : chunk_experts - 1;  // (past the chunk: the last row again, unused)
+          v[k] = u < units ? unit_cnt[(size_t)(c + ee) * units + u] : 0;
+        }
+#pragma unroll
+        for (int k = 0; k < kRows; ++k) {
+          t[k] += v[k];
+          b[k] += u < unit ? v[k] : 0;
+        }
       }
-      t = wave_sum_i32(t);
-      b = wave_sum_i32(b);
-      if (lane == ee) {
-        tot = t;
-        before = b;
+#pragma unroll
+      for (int k = 0; k < kRows; ++k) {
+        const int ts = wave_sum_i32(t[k]), bs = wave_sum_i32(b[k]);
+        if (lane == ee0 + k && ee0 + k < chunk_experts) {
+          tot = ts;
+          before = bs;
+        }
       }
     }
     int inc = tot;
@@ -340,7 +390,6 @@ __global__ __launch_bounds__(kTileWaves *kWave) void dispatch_scan_rank_kernel(
     if (e < n_experts) {
       const int off = carry + inc - tot;
       wrow[wave][e] = off + before;
-      wtot[wave][e] = tot;
       if (unit == 0) {
         counts[e] = tot;
         offsets[e] = off;
@@ -349,11 +398,86 @@ __global__ __launch_bounds__(kTileWaves *kWave) void dispatch_scan_rank_kernel(
     carry += __shfl(inc, kWave - 1, kWave);
   }
   if (unit == 0 && lane == 0) offsets[n_experts] = carry;
-  __builtin_amdgcn_wave_barrier();
-  const int64_t begin = (int64_t)unit * rounds * kWave;
-  rank_span(idx, skip, n_slots, n_experts, nbits, begin, rounds, wrow[wave], lane, perm, inv_perm);
+  wave_lds_sync();
+  rank_span<ROUNDS>(span, nbits, wrow[wave], lane, perm, inv_perm);
   const int total = carry;
-  for (int r = 0; r < rounds; ++r) {
+#pragma unroll
+  for (int r = 0; r < ROUNDS; ++r) {
+    const int64_t i = begin + (int64_t)r * kWave + lane;
+    if (i >= total && i < n_slots) perm[i] = -1;
+  }
+}
+
+// dispatch_scan_rank_kernel for small tables (at most EMAX experts and 64 UMAX
+// units): the wave's slots and its whole share of the table are requested in
+// one go, in straight-line code, so the kernel costs one memory round trip
+// before it ranks (around a loop the compiler waits for every load in flight).
+template <int ROUNDS, int EMAX, int UMAX>
+__global__ __launch_bounds__(kTileWaves *kWave) void dispatch_scan_rank_small_kernel(
+    const int32_t *__restrict__ idx, const uint8_t *__restrict__ skip, int64_t n_slots,
+    int n_experts, int nbits, int units, const int32_t *__restrict__ unit_cnt,
+    int32_t *__restrict__ counts, int32_t *__restrict__ offsets, int32_t *__restrict__ perm,
+    int32_t *__restrict__ inv_perm, int32_t *__restrict__ range_out, int32_t range_n) {
+  static_assert(EMAX <= kWave, "expert e's sums live in lane e");
+  __shared__ int32_t wrow[kTileWaves][kMaxExperts];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int unit = blockIdx.x * kTileWaves + wave;
+  if (range_out && blockIdx.x == 0 && threadIdx.x == 0) {
+    range_out[0] = 0;
+    range_out[1] = range_n;
+  }
+  if (unit >= units) return;
+  int v[EMAX][UMAX];
+#pragma unroll
+  for (int e = 0; e < EMAX; ++e)
+#pragma unroll
+    for (int j = 0; j < UMAX; ++j) {
+      const int u = j * kWave + lane;
+      const int row = e < n_experts ? e : n_experts - 1;   // (rows past the table: the last one again, unused)
+      v[e][j] = unit_cnt[(size_t)row * units + (u < units ? u : 0)];
+    }
+  const int64_t begin = (int64_t)unit * ROUNDS * kWave;
+  SlotInfo span[ROUNDS];
+  read_span<ROUNDS>(idx, skip, n_slots, n_experts, begin, lane, span);
+  int tot = 0, before = 0;
+#pragma unroll
+  for (int e = 0; e < EMAX; ++e) {
+    int t = 0, b = 0;
+#pragma unroll
+    for (int j = 0; j < UMAX; ++j) {
+      const int u = j * kWave + lane;
+      t += u < units ? v[e][j] : 0;
+      b += u < unit ? v[e][j] : 0;
+    }
+    t = wave_sum_i32(t);
+    b = wave_sum_i32(b);
+    if (lane == e) {
+      tot = t;
+      before = b;
+    }
+  }
+  if (lane >= n_experts) tot = before = 0;
+  int inc = tot;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    const int up = __shfl_up(inc, o, kWave);
+    if (lane >= o) inc += up;
+  }
+  const int off = inc - tot;
+  if (lane < n_experts) {
+    wrow[wave][lane] = off + before;
+    if (unit == 0) {
+      counts[lane] = tot;
+      offsets[lane] = off;
+    }
+  }
+  const int total = __shfl(inc, kWave - 1, kWave);
+  if (unit == 0 && lane == 0) offsets[n_experts] = total;
+  wave_lds_sync();
+  rank_span<ROUNDS>(span, nbits, wrow[wave], lane, perm, inv_perm);
+#pragma unroll
+  for (int r = 0; r < ROUNDS; ++r) {
     const int64_t i = begin + (int64_t)r * kWave + lane;
     if (i >= total && i < n_slots) perm[i] = -1;
   }
@@ -394,7 +518,7 @@ extern "C" size_t dice_dispatch_workspace_bytes(int64_t n_slots, int n_experts) 
   using namespace dice;
   if (n_slots <= kFusedMaxSlots || n_experts <= 0) return 256;
   const int64_t mid_units = (n_slots + kMidRounds * kWave - 1) / (kMidRounds * kWave);
-  const int64_t units = mid_units * n_experts <= kMidMaxTable
+  const int64_t units = mid_units * mid_units * n_experts <= kMidMaxWork
                             ? mid_units
                             : (n_slots + kTileRounds * kWave - 1) / (kTileRounds * kWave);
   return align_up((size_t)units * n_experts * sizeof(int32_t), 256);
@@ -427,23 +551,39 @@ int dispatch_impl(const int32_t *flat_idx, const uint8_t *skip_mask, int64_t n_s
                "dice_dispatch: workspace %zu < %zu bytes", workspace_bytes, need);
   int32_t *unit_cnt = (int32_t *)workspace;
   const int64_t mid_units = (n_slots + kMidRounds * kWave - 1) / (kMidRounds * kWave);
-  if (mid_units * n_experts <= kMidMaxTable) {
+  if (mid_units * mid_units * n_experts <= kMidMaxWork) {
     // Mid sizes: per-wave histograms, then one kernel that scans the (small)
     // table in every wave and ranks.
     const int units = (int)mid_units;
     const int blocks = (units + kTileWaves - 1) / kTileWaves;
-    hipLaunchKernelGGL(dispatch_count_kernel, dim3(blocks), dim3(kTileWaves * kWave), 0, s, flat_idx,
-                       skip_mask, n_slots, n_experts, nbits, units, kMidRounds, unit_cnt);
-    hipLaunchKernelGGL(dispatch_scan_rank_kernel, dim3(blocks), dim3(kTileWaves * kWave), 0, s, flat_idx,
-                       skip_mask, n_slots, n_experts, nbits, units, kMidRounds, unit_cnt, counts, offsets,
-                       perm, inv_perm, range_out, range_n);
+    hipLaunchKernelGGL(dispatch_count_kernel<kMidRounds>, dim3(blocks), dim3(kTileWaves * kWave), 0, s, flat_idx,
+                       skip_mask, n_slots, n_experts, nbits, units, unit_cnt);
+    // (the instantiation that just covers the table: these kernels run for a few
+    // microseconds, most of them spent fetching their own code)
+#define DICE_SCAN_RANK_SMALL(EMAX, UMAX)                                                                      \
+  hipLaunchKernelGGL((dispatch_scan_rank_small_kernel<kMidRounds, EMAX, UMAX>), dim3(blocks),                 \
+                     dim3(kTileWaves * kWave), 0, s, flat_idx, skip_mask, n_slots, n_experts, nbits, units,   \
+                     unit_cnt, counts, offsets, perm, inv_perm, range_out, range_n)
+    if (n_experts <= 8 && units <= kWave)
+      DICE_SCAN_RANK_SMALL(8, 1);
+    else if (n_experts <= 8 && units <= 2 * kWave)
+      DICE_SCAN_RANK_SMALL(8, 2);
+    else if (n_experts <= 16 && units <= kWave)
+      DICE_SCAN_RANK_SMALL(16, 1);
+    else if (n_experts <= 16 && units <= 2 * kWave)
+      DICE_SCAN_RANK_SMALL(16, 2);
+#undef DICE_SCAN_RANK_SMALL
+    else
+      hipLaunchKernelGGL(dispatch_scan_rank_kernel<kMidRounds>, dim3(blocks), dim3(kTileWaves * kWave), 0, s,
+                         flat_idx, skip_mask, n_slots, n_experts, nbits, units, unit_cnt, counts, offsets, perm,
+                         inv_perm, range_out, range_n);
     return launch_status("dice_dispatch");
   }
   const int64_t units64 = (n_slots + kTileRounds * kWave - 1) / (kTileRounds * kWave);
   const int units = (int)units64;
   const int blocks = (units + kTileWaves - 1) / kTileWaves;
-  hipLaunchKernelGGL(dispatch_count_kernel, dim3(blocks), dim3(kTileWaves * kWave), 0, s, flat_idx,
-                     skip_mask, n_slots, n_experts, nbits, units, kTileRounds, unit_cnt);
+  hipLaunchKernelGGL(dispatch_count_kernel<kTileRounds>, dim3(blocks), dim3(kTileWaves * kWave), 0, s, flat_idx,
+                     skip_mask, n_slots, n_experts, nbits, units, unit_cnt);
   hipLaunchKernelGGL(dispatch_scan_kernel, dim3(1), dim3(1024), 0, s, unit_cnt, n_experts, units,
                      counts, offsets, range_out, range_n);
   hipLaunchKernelGGL(dispatch_rank_kernel, dim3(blocks), dim3(kTileWaves * kWave), 0, s, flat_idx,
