@@ -1,11 +1,17 @@
-// Router: fp32 logits -> softmax -> top-k, one wavefront per 64 / E tokens.
+// Router: fp32 logits -> softmax -> top-k.
 //
 // Replaces MoEGate.forward, inference branch (reference models.py:179-196).
 // HBM-bound: the only large operand is x, read exactly once (n_tokens*hidden
-// elements); the router matrix comes from the vector cache, or, when it is too
-// large for that, from LDS, where each workgroup stages it once.  Each wave
-// keeps 64/E tokens in flight so one read of a router chunk feeds that many
-// dot-product updates.
+// elements).  Two kernels: 16-bit activations with a router matrix of the same
+// type and at most 32 experts (every DiT-MoE size) multiply on the matrix pipe,
+// 32 tokens per workgroup (gate_topk_mfma_kernel, below); everything else -
+// fp32, an fp32 router matrix for 16-bit activations, more experts, odd hidden
+// sizes - takes gate_topk_kernel, one wavefront per 64 / E tokens, where the
+// router matrix comes from the vector cache, or, when it is too large for
+// that, from LDS, and each wave keeps 64/E tokens in flight so one read of a
+// router chunk feeds that many dot-product updates.
+#include <type_traits>
+
 #include "common.h"
 
 namespace dice {
@@ -253,10 +259,183 @@ int launch_gate(const void *x, const void *w, const float *bias, int64_t n_token
   return launch_status("dice_gate_topk");
 }
 
+
+// ---------------------------------------------------------------------------
+// The router on the matrix pipe (16-bit activations and router matrix, at most
+// 32 experts).  The kernel above spends its time issuing instructions - about
+// 3000 per wave for eight tokens - not waiting for memory; here a workgroup
+// routes 32 tokens with v_mfma_f32_32x32x16: the experts are the 32 rows of the
+// left operand (rows past n_experts repeat the last one and are ignored), the
+// tokens the 32 columns of the right one, so lane l supplies 16 bytes of token
+// l % 32 per step - straight from memory, no LDS staging.  The hidden dimension
+// is cut into 2 x WPB contiguous segments, one per (wave, lane half): a wave
+// requests its whole share (at most kRouterMaxSteps x 2 loads of 1 KB) before
+// the first product, the WPB partial logit tiles are added in wave order
+// through LDS, and the first wave finishes softmax and top-k with all of a
+// token's logits in one lane.  Summation order is fixed (per lane half, per
+// wave, then over the waves), so results do not depend on timing.
+constexpr int kRouterMaxSteps = 18;
+template <typename T> struct RouterMfma;
+template <> struct RouterMfma<bf16_t> {
+  static __device__ __forceinline__ f32x16_t mul(bf16x8_t a, bf16x8_t b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct RouterMfma<f16_t> {
+  static __device__ __forceinline__ f32x16_t mul(f16x8_t a, f16x8_t b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+template <typename T, int EP, int WPB>
+__device__ __forceinline__ void gate_topk_mfma_body(
+    const T *__restrict__ x, const T *__restrict__ w, const float *__restrict__ bias, int64_t n_tokens,
+    int hidden, int n_experts, int top_k, int norm_topk, int32_t *__restrict__ topk_idx,
+    int64_t *__restrict__ topk_idx64, float *__restrict__ topk_weight, float *__restrict__ logits_out) {
+  constexpr int NR = EP / 2;  // accumulator registers of a lane that hold experts below EP
+  __shared__ float part[WPB][NR][kWave];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int col = lane & 31, half = lane >> 5;
+  const int64_t tok = (int64_t)blockIdx.x * 32 + col;
+  const int64_t tok_c = tok < n_tokens ? tok : n_tokens - 1;   // (columns past the end repeat the last token)
+  const int steps = hidden / 16 / WPB;                         // per wave; at most kRouterMaxSteps
+  const int seg = (wave * 2 + half) * steps * 8;               // this lane's segment of the hidden dimension
+  const T *xp = x + tok_c * hidden + seg;
+  const T *wp = w + (size_t)(col < n_experts ? col : n_experts - 1) * hidden + seg;
+  Vec8<T> xv[kRouterMaxSteps], wv[kRouterMaxSteps];
+#pragma unroll
+  for (int s = 0; s < kRouterMaxSteps; ++s) {
+    const int at = s < steps ? s : 0;   // (no branch around a load: steps past the end re-read the first chunk)
+    xv[s] = load8(xp + at * 8);
+    wv[s] = load8(wp + at * 8);
+  }
+  f32x16_t acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+  for (int s = 0; s < kRouterMaxSteps; ++s)
+    if (s < steps) acc = RouterMfma<T>::mul(wv[s].v, xv[s].v, acc);
+  // lane (col, half), register a: logit of expert 8 (a / 4) + 4 half + a % 4 for token col
+#pragma unroll
+  for (int a = 0; a < NR; ++a) part[wave][a][lane] = acc[a];
+  __syncthreads();
+  if (wave != 0) return;
+  float mine[NR], other[NR];
+#pragma unroll
+  for (int a = 0; a < NR; ++a) {
+    float v = part[0][a][lane];
+#pragma unroll
+    for (int q = 1; q < WPB; ++q) v += part[q][a][lane];
+    mine[a] = v;
+  }
+#pragma unroll
+  for (int a = 0; a < NR; ++a) other[a] = __shfl_xor(mine[a], 32, kWave);
+  float score[EP];
+  float m = -INFINITY;
+#pragma unroll
+  for (int e = 0; e < EP; ++e) {
+    const int a = (e / 8) * 4 + e % 4;
+    float logit = ((e % 8) / 4 == half) ? mine[a] : other[a];
+    if (e < n_experts) {
+      if (bias) logit += bias[e];
+      if (logits_out && half == 0 && tok < n_tokens) logits_out[tok * n_experts + e] = logit;
+    } else {
+      logit = -INFINITY;
+    }
+    score[e] = logit;
+    m = fmaxf(m, logit);
+  }
+  float denom = 0.f;
+#pragma unroll
+  for (int e = 0; e < EP; ++e) {
+    score[e] = e < n_experts ? expf(score[e] - m) : 0.f;
+    denom += score[e];
+  }
+#pragma unroll
+  for (int e = 0; e < EP; ++e) score[e] = e < n_experts ? score[e] / denom : -1.f;
+  // top-k: repeated arg-max, ties to the lower expert id (ascending scan, strict compare)
+  float sel_w[8];
+  int sel_i[8];
+  float picked_sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    sel_w[j] = 0.f;
+    sel_i[j] = 0;
+    if (j < top_k) {
+      float bv = -2.f;
+      int bi = 0;
+#pragma unroll
+      for (int e = 0; e < EP; ++e)
+        if (score[e] > bv) {
+          bv = score[e];
+          bi = e;
+        }
+#pragma unroll
+      for (int e = 0; e < EP; ++e)
+        if (e == bi) score[e] = -1.f;
+      sel_w[j] = bv;
+      sel_i[j] = bi;
+      picked_sum += bv;
+    }
+  }
+  if (half != 0 || tok >= n_tokens) return;
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    if (j < top_k) {
+      const float wgt = (norm_topk && top_k > 1) ? sel_w[j] / (picked_sum + 1e-20f) : sel_w[j];
+      topk_idx[tok * top_k + j] = sel_i[j];
+      if (topk_idx64) topk_idx64[tok * top_k + j] = sel_i[j];
+      topk_weight[tok * top_k + j] = wgt;
+    }
+}
+// (builtins that only exist for the device stay out of the __global__ template's own body)
+template <typename T, int EP, int WPB>
+__global__ __launch_bounds__(WPB *kWave) void gate_topk_mfma_kernel(
+    const T *__restrict__ x, const T *__restrict__ w, const float *__restrict__ bias, int64_t n_tokens,
+    int hidden, int n_experts, int top_k, int norm_topk, int32_t *__restrict__ topk_idx,
+    int64_t *__restrict__ topk_idx64, float *__restrict__ topk_weight, float *__restrict__ logits_out) {
+  gate_topk_mfma_body<T, EP, WPB>(x, w, bias, n_tokens, hidden, n_experts, top_k, norm_topk, topk_idx, topk_idx64,
+                                  topk_weight, logits_out);
+}
+
+// Waves per 32-token workgroup of the matrix-pipe router for this hidden size
+// (0: it does not apply).
+inline int router_mfma_waves(int hidden) {
+  if (hidden % 64 != 0) return 0;
+  const int steps = hidden / 16;
+  if (steps / 4 <= kRouterMaxSteps) return 4;
+  if (steps % 8 == 0 && steps / 8 <= kRouterMaxSteps) return 8;
+  return 0;
+}
+template <typename T, int EP>
+int launch_gate_mfma(const void *x, const void *w, const float *bias, int64_t n_tokens, int hidden, int n_experts,
+                     int top_k, int norm, int32_t *idx, int64_t *idx64, float *wt, float *logits,
+                     hipStream_t stream) {
+  const int wpb = router_mfma_waves(hidden);
+  const unsigned blocks = (unsigned)((n_tokens + 31) / 32);
+  if (wpb == 4)
+    hipLaunchKernelGGL((gate_topk_mfma_kernel<T, EP, 4>), dim3(blocks), dim3(4 * kWave), 0, stream, (const T *)x,
+                       (const T *)w, bias, n_tokens, hidden, n_experts, top_k, norm, idx, idx64, wt, logits);
+  else
+    hipLaunchKernelGGL((gate_topk_mfma_kernel<T, EP, 8>), dim3(blocks), dim3(8 * kWave), 0, stream, (const T *)x,
+                       (const T *)w, bias, n_tokens, hidden, n_experts, top_k, norm, idx, idx64, wt, logits);
+  return launch_status("dice_gate_topk");
+}
+
 template <typename XT, typename WT>
 int dispatch_experts(const void *x, const void *w, const float *bias, int64_t n_tokens, int hidden,
                      int n_experts, int top_k, int norm, int32_t *idx, int64_t *idx64, float *wt,
                      float *logits, hipStream_t s) {
+  if constexpr (std::is_same<XT, WT>::value && sizeof(XT) == 2) {
+    if (n_experts <= 32 && n_tokens < (1ll << 31) / 32 && router_mfma_waves(hidden) != 0) {
+      if (n_experts <= 8)
+        return launch_gate_mfma<XT, 8>(x, w, bias, n_tokens, hidden, n_experts, top_k, norm, idx, idx64, wt, logits, s);
+      if (n_experts <= 16)
+        return launch_gate_mfma<XT, 16>(x, w, bias, n_tokens, hidden, n_experts, top_k, norm, idx, idx64, wt, logits, s);
+      return launch_gate_mfma<XT, 32>(x, w, bias, n_tokens, hidden, n_experts, top_k, norm, idx, idx64, wt, logits, s);
+    }
+  }
   if (n_experts <= 8)
     return launch_gate<XT, WT, 8>(x, w, bias, n_tokens, hidden, n_experts, top_k, norm, idx, idx64, wt, logits, s);
   if (n_experts <= 16)

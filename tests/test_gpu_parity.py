@@ -56,6 +56,13 @@ def _check_gate(dev, x, w, k, norm=False, bias=None):
     (1000, 768, 16, 4, torch.float16),
     (517, 1024, 5, 3, torch.float32),      # ragged token count, odd expert count
     (3, 64, 64, 8, torch.float32),
+    # 16-bit activations and router matrix, at most 32 experts: the matrix-pipe router
+    (777, 1152, 7, 2, torch.bfloat16),     # ragged token count (25 column blocks, the last with 9 tokens), odd expert count
+    (300, 2304, 32, 8, torch.float16),     # 32 experts, top-8, eight waves per token block
+    (64, 192, 24, 3, torch.bfloat16),      # three steps per wave
+    (33, 1024, 1, 1, torch.bfloat16),      # a single expert
+    (100, 4096, 8, 2, torch.bfloat16),     # too long for it: the dot-product router
+    (50, 72, 8, 2, torch.bfloat16),        # hidden not a multiple of 64: the dot-product router
 ])
 def test_gate_matches_oracle(dev, N, D, E, k, dtype):
     g = _gen(N + E)
