@@ -169,6 +169,7 @@ struct PersistBatch {
   int n_problems;
   PersistProblem prob[kMaxPersistProblems];
   int band_tiles;  // tile order: m-tiles per band (a group with more is cut into bands); 0 = the default rule
+  int xcd_split;   // how the tiles are shared out over the XCDs (set by the launcher; see TileWalker)
   // Partial-tile slots (persist_split_ws_bytes() bytes) or NULL.  With slots, a
   // single-problem fc2 launch whose tiles do not fill the workgroups' last turn
   // cuts that turn's tiles along k, one piece per workgroup, and a second small

@@ -41,6 +41,10 @@
 // widening differ; shared host-side helpers live in the bf16 compilation.
 #include <type_traits>
 
+#include <algorithm>
+#include <cstring>
+#include <vector>
+
 #include "gemm_common.h"
 
 #ifndef DICE_PERSIST_F16
@@ -176,8 +180,8 @@ __device__ __forceinline__ Tile unpack_tile(const PackedTile &pk) {
 // the index of its first tile (at most 64 groups); a tile id is mapped back to
 // its group with one ballot.  Tiles are ordered problem-major, expert-major,
 // then n-tile with the m-tile fastest; callers list the problem with the longest
-// k first.  XCD x (= blockIdx.x % 8) owns the x-th eighth of that order and its
-// workgroups take tiles of the run in turns.
+// k first.  XCD x (= blockIdx.x % 8) owns the x-th eighth of every problem's tiles
+// and its workgroups take the tiles of that run in turns.
 // Position of tile `r` inside one (problem, expert) group of mt x nt tiles.
 // The m-tile runs fastest, so that the workgroups of an XCD that work side by
 // side share weight tiles; a group with many m-tiles (large batches) is cut
@@ -238,7 +242,10 @@ __device__ __forceinline__ SplitRange split_range(int steps, int piece, int ways
 template <int BN_OUT>
 struct TileWalker {
   int g_prob = 0, g_expert = 0, g_row0 = 0, g_cnt = 0, g_mt = 0, g_base = 0, g_end = 0;
-  int run_begin, run_end, wg_in_xcd, wgs_per_xcd, xcd_id;
+  // This XCD's tiles: of every problem the x-th eighth of its tiles (sub_first:
+  // id of the first, sub_len: how many), taken problem after problem.
+  int sub_first[kMaxPersistProblems], sub_len[kMaxPersistProblems], run_len;
+  int wg_in_xcd, wgs_per_xcd, xcd_id;
   int split_turn, split_left;   // the XCD's last, short turn and its tiles
   int split_q, split_extra;     // positions per tile of that turn when it is cut: q + 1 for the first `extra` tiles, q for the rest
   int split_cap;                // most pieces a tile's length allows; 0: the turn is not cut
@@ -277,30 +284,80 @@ struct TileWalker {
     }
     g_base = inc - tiles;
     g_end = inc;
-    const int total_tiles = __shfl(inc, kWave - 1, kWave);
-    const int total_cost = __shfl(cinc, kWave - 1, kWave);
-    // XCD x takes the tiles between the x-th and the (x+1)-th eighth of the total
-    // COST, so that every XCD gets the same amount of work whatever the mix.
     xcd_id = uni(xcd);
     wg_in_xcd = uni(wg);
     wgs_per_xcd = uni(wgs);
-    auto boundary = [&](int x) {
-      if (x >= kNumXcd) return total_tiles;
-      const int target = (int)((long long)total_cost * x / kNumXcd);
-      const uint64_t hit = __ballot(cost > 0 && target >= cinc - cost && target < cinc);
-      if (!hit) return total_tiles;
-      const int g = __builtin_ctzll(hit);
-      const int base = __builtin_amdgcn_readlane(g_base, g);
-      const int cbase = __builtin_amdgcn_readlane(cinc - cost, g);
-      const int k32 = __builtin_amdgcn_readlane(g_k32, g);
-      return base + (target - cbase + k32 / 2) / k32;
-    };
-    run_begin = uni(boundary(xcd));
-    run_end = uni(boundary(xcd + 1));
-    const int len = run_end - run_begin;
-    split_turn = len / wgs_per_xcd;
-    split_left = len - split_turn * wgs_per_xcd;
+    // Two ways to give every XCD the same amount of work (the launcher picks one
+    // per shape, see persist_xcd_split):
+    //  0: XCD x takes the tiles between the x-th and the (x+1)-th eighth of the
+    //     total COST in problem order.  XCDs then differ in their mix - some get
+    //     only long tiles, some only short ones - which spreads the tiles with the
+    //     most bytes per step over the whole launch, but an XCD whose long tiles
+    //     just spill into another turn waits a whole long tile for a few of them
+    //     (a skip step's fc2: 39 tiles of 72 steps for 32 workgroups).
+    //  1: XCD x takes the x-th eighth of the tiles of EVERY problem (the tiles of
+    //     one problem cost the same): the same mix everywhere; a workgroup's turns
+    //     run from the longest tiles to the shortest, and one that got a long tile
+    //     less makes up for it with short ones.
+    int run_begin = 0, run_end = 0x7fffffff;   // (split 0) the XCD's stretch of the tile order
+    if (batch.xcd_split == 0) {
+      const int total_tiles = __shfl(inc, kWave - 1, kWave);
+      const int total_cost = __shfl(cinc, kWave - 1, kWave);
+      auto boundary = [&](int x) {
+        if (x >= kNumXcd) return total_tiles;
+        const int target = (int)((long long)total_cost * x / kNumXcd);
+        const uint64_t hit = __ballot(cost > 0 && target >= cinc - cost && target < cinc);
+        if (!hit) return total_tiles;
+        const int g = __builtin_ctzll(hit);
+        const int base = __builtin_amdgcn_readlane(g_base, g);
+        const int cbase = __builtin_amdgcn_readlane(cinc - cost, g);
+        const int k32 = __builtin_amdgcn_readlane(g_k32, g);
+        return base + (target - cbase + k32 / 2) / k32;
+      };
+      run_begin = uni(boundary(xcd));
+      run_end = uni(boundary(xcd + 1));
+    }
+    run_len = 0;
+    int first_group = 0;
+#pragma unroll
+    for (int pi = 0; pi < kMaxPersistProblems; ++pi) {
+      sub_first[pi] = sub_len[pi] = 0;
+      if (pi < batch.n_problems) {
+        const int last_group = first_group + batch.prob[pi].n_experts - 1;
+        const int p_base = __builtin_amdgcn_readlane(g_base, first_group);
+        const int p_end = __builtin_amdgcn_readlane(g_end, last_group);
+        int lo, hi;
+        if (batch.xcd_split == 0) {   // the problem's part of the XCD's stretch
+          lo = run_begin > p_base ? run_begin : p_base;
+          hi = run_end < p_end ? run_end : p_end;
+        } else {
+          const int p_tiles = p_end - p_base;
+          lo = p_base + (int)((long long)p_tiles * xcd / kNumXcd);
+          hi = p_base + (int)((long long)p_tiles * (xcd + 1) / kNumXcd);
+        }
+        sub_first[pi] = uni(lo);
+        sub_len[pi] = uni(hi > lo ? hi - lo : 0);
+        run_len += sub_len[pi];
+        first_group = last_group + 1;
+      }
+    }
+    split_turn = run_len / wgs_per_xcd;
+    split_left = run_len - split_turn * wgs_per_xcd;
     split_q = split_extra = split_cap = 0;
+  }
+
+  // The id of the i-th tile of this XCD's run (kNoTile past its end).
+  static constexpr int kNoTile = 0x7fffffff;
+  __device__ __forceinline__ int run_tile(int i) const {
+    int id = kNoTile;
+#pragma unroll
+    for (int pi = kMaxPersistProblems - 1; pi >= 0; --pi) {
+      int before = 0;
+#pragma unroll
+      for (int q = 0; q < pi; ++q) before += sub_len[q];
+      if (i >= before && i < before + sub_len[pi]) id = sub_first[pi] + (i - before);
+    }
+    return i >= 0 ? id : kNoTile;
   }
 
   // Decides whether the last turn is cut (launches with partial-tile slots
@@ -361,8 +418,8 @@ struct TileWalker {
     // (the split turn: positions j S .. j S + S - 1 share the turn's j-th tile)
     const bool cut = split_cap != 0 && turn == split_turn;
     const SplitPiece sp = cut ? split_piece(w) : SplitPiece{0, 0, 0, 0};
-    const int id = run_begin + turn * wgs_per_xcd + (cut ? sp.tile : w);
-    const bool valid = id < run_end && (!cut || sp.ways != 0);
+    const int id = run_tile(turn * wgs_per_xcd + (cut ? sp.tile : w));
+    const bool valid = id != kNoTile && (!cut || sp.ways != 0);
     const int idc = valid ? id : 0;
     int n_groups = 0;
     for (int pi = 0; pi < batch.n_problems; ++pi) n_groups += batch.prob[pi].n_experts;
@@ -449,7 +506,7 @@ struct TileWalker {
   // the last long tiles get the fewest short ones.
   __device__ __forceinline__ int tile_id(int round) const {
     const int w = (round & 1) ? wgs_per_xcd - 1 - wg_in_xcd : wg_in_xcd;
-    return uni(run_begin + round * wgs_per_xcd + w);
+    return uni(run_tile(round * wgs_per_xcd + w));
   }
 
   // Tile `id` of the order (ids past this XCD's run give an invalid tile whose
@@ -457,7 +514,7 @@ struct TileWalker {
   __device__ __forceinline__ Tile decode(const PersistBatch &batch, int id, int bk) const {
     Tile t;
     id = uni(id);  // wave-uniform by construction; says so to the compiler (scalar arithmetic below)
-    t.valid = id < run_end;
+    t.valid = id != kNoTile;
     const int idc = t.valid ? id : 0;
     const uint64_t hit = __ballot(idc >= g_base && idc < g_end);
     const int g = hit ? __builtin_ctzll(hit) : 0;
@@ -1861,7 +1918,7 @@ __device__ __forceinline__ void persist_split_sum_body(const PersistBatch &batch
   walk.plan_split(batch, bk);
   if (walk.split_cap == 0 || j >= walk.split_left) return;
   const SplitPiece sp = walk.split_tile(j);
-  const Tile t = walk.decode(batch, walk.run_begin + walk.split_turn * wgs + j, bk);
+  const Tile t = walk.decode(batch, walk.run_tile(walk.split_turn * wgs + j), bk);
   if (!t.valid || sp.ways == 0) return;
   constexpr int kChunks = BN_OUT / 8;  // 16-byte chunks per slot row
   const int ways = sp.ways;
@@ -1902,6 +1959,114 @@ bool split_may_apply(const PersistBatch &b, int grid, int bn_out) {
   if (p.n_experts != 1) return true;   // group heights live on the device
   const int64_t tiles = ((int64_t)p.max_rows + kPBM - 1) / kPBM * ((p.n + bn_out - 1) / bn_out);
   return tiles % grid != 0;
+}
+// The order of a launch's problems and which of TileWalker's two ways of
+// sharing the tiles out over the XCDs it takes.  The group heights live on the
+// device, so the pick is made from a model: evenly loaded groups, every
+// workgroup's load in k steps (same arithmetic as the device) for the caller's
+// order and for longest-k-first, under both splits.  The caller's order with
+// the cost split stands unless another arrangement shortens the longest
+// workgroup by 7 % or more: with equal makespans it measures fastest (it does
+// not start all the long tiles, which move the most bytes per step, at the same
+// time on every XCD).  A launch of one problem has nothing to choose.  The model
+// costs a few microseconds of host time, so the last few shapes are remembered.
+struct PersistPlan {
+  bool longest_first;   // sort the problems by k, longest first
+  int xcd_split;
+};
+int64_t model_makespan(const PersistProblem *prob, int n_problems, int bn_out, int wgs, int split) {
+  int64_t tiles[kMaxPersistProblems], steps[kMaxPersistProblems], base[kMaxPersistProblems], total_cost = 0, total = 0;
+  for (int p = 0; p < n_problems; ++p) {
+    const PersistProblem &pr = prob[p];
+    const int64_t per = pr.max_rows / pr.n_experts, rem = pr.max_rows % pr.n_experts;
+    const int64_t m_tiles = rem * ((per + 1 + kPBM - 1) / kPBM) + (pr.n_experts - rem) * ((per + kPBM - 1) / kPBM);
+    tiles[p] = m_tiles * ((pr.n + bn_out - 1) / bn_out);
+    steps[p] = pr.k / 32;
+    base[p] = total;
+    total += tiles[p];
+    total_cost += tiles[p] * steps[p];
+  }
+  auto boundary = [&](int x) -> int64_t {   // (split 0) first tile of XCD x's stretch
+    if (x >= kNumXcd) return total;
+    const int64_t target = total_cost * x / kNumXcd;
+    int64_t cbase = 0;
+    for (int p = 0; p < n_problems; ++p) {
+      const int64_t c = tiles[p] * steps[p];
+      if (c > 0 && target >= cbase && target < cbase + c) return base[p] + (target - cbase + steps[p] / 2) / steps[p];
+      cbase += c;
+    }
+    return total;
+  };
+  int64_t makespan = 0;
+  std::vector<int64_t> load(wgs);
+  for (int x = 0; x < kNumXcd; ++x) {
+    std::fill(load.begin(), load.end(), 0);
+    int64_t i = 0;   // position in the XCD's run
+    for (int p = 0; p < n_problems; ++p) {
+      int64_t lo, hi;
+      if (split == 0) {
+        lo = std::max(boundary(x), base[p]);
+        hi = std::min(boundary(x + 1), base[p] + tiles[p]);
+      } else {
+        lo = base[p] + tiles[p] * x / kNumXcd;
+        hi = base[p] + tiles[p] * (x + 1) / kNumXcd;
+      }
+      for (int64_t t = lo; t < hi; ++t, ++i) {
+        const int turn = (int)(i / wgs), w = (int)(i % wgs);
+        load[(turn & 1) ? wgs - 1 - w : w] += steps[p];
+      }
+    }
+    makespan = std::max(makespan, *std::max_element(load.begin(), load.end()));
+  }
+  return makespan;
+}
+PersistPlan persist_plan(const PersistBatch &b, int bn_out, int grid) {
+  if (b.n_problems < 2) return PersistPlan{false, 1};
+  struct Shape {
+    int n_problems, bn_out, grid, rows[kMaxPersistProblems], experts[kMaxPersistProblems], n[kMaxPersistProblems],
+        k[kMaxPersistProblems];
+    PersistPlan plan;
+  };
+  Shape key{};
+  key.n_problems = b.n_problems;
+  key.bn_out = bn_out;
+  key.grid = grid;
+  for (int p = 0; p < b.n_problems; ++p) {
+    key.rows[p] = b.prob[p].max_rows;
+    key.experts[p] = b.prob[p].n_experts;
+    key.n[p] = b.prob[p].n;
+    key.k[p] = b.prob[p].k;
+  }
+  constexpr int kRemembered = 8;
+  static thread_local Shape seen[kRemembered];
+  static thread_local int n_seen = 0, next = 0;
+  for (int i = 0; i < n_seen; ++i) {
+    Shape c = seen[i];
+    c.plan = PersistPlan{};
+    if (memcmp(&c, &key, sizeof(Shape)) == 0) return seen[i].plan;
+  }
+  PersistProblem sorted[kMaxPersistProblems];
+  std::copy(b.prob, b.prob + b.n_problems, sorted);
+  std::stable_sort(sorted, sorted + b.n_problems,
+                   [](const PersistProblem &x, const PersistProblem &y) { return x.k > y.k; });
+  const int wgs = grid / kNumXcd;
+  // in order of preference
+  const PersistPlan plans[4] = {{false, 0}, {true, 0}, {false, 1}, {true, 1}};
+  PersistPlan pick = plans[0];
+  int64_t best = model_makespan(b.prob, b.n_problems, bn_out, wgs, 0);
+  for (int i = 1; i < 4; ++i) {
+    const int64_t m = model_makespan(plans[i].longest_first ? sorted : b.prob, b.n_problems, bn_out, wgs,
+                                     plans[i].xcd_split);
+    if (m * 100 < best * 93) {
+      best = m;
+      pick = plans[i];
+    }
+  }
+  key.plan = pick;
+  seen[next] = key;
+  next = (next + 1) % kRemembered;
+  if (n_seen < kRemembered) ++n_seen;
+  return pick;
 }
 // Launches the sum for a multiplying launch of `grid` workgroups.
 template <int BN_OUT>
@@ -1971,6 +2136,7 @@ int launch_grouped_gemm_persist_f8(const PersistBatch &b, int mode, hipStream_t 
     kern = refill ? gemm_persist_kernel_f8<kFc2, false, true> : gemm_persist_kernel_f8<kFc2, false, false>;
   PersistBatch launch = b;
   launch.band_tiles = persist_band_tiles(mode);
+  launch.xcd_split = 1;   // (one problem: the two splits are the same)
   // (a last turn cut along k: only the plain epilogue is linear in k)
   if (mode != kFc2 || grid / kNumXcd < 2 || grid > kPersistSplitSlots || !split_may_apply(b, grid, kPBN))
     launch.split_ws = nullptr;
@@ -2023,21 +2189,18 @@ bool persist_common_ok(const PersistBatch &b, int mode) {
 
 // Whether every workgroup's turns fit the LDS tile table of the 64-k kernel
 // (the last entry stays an invalid tile), bounded from the host-side row
-// bounds: an XCD gets 1/8 of the total cost, in the worst case all of it in its
-// shortest tiles.  Launches that do not fit take the table-rewriting kernels.
+// bounds: an XCD gets an eighth of every problem's tiles.  Launches that do not
+// fit take the table-rewriting kernels.
 bool persist64_fits_table(const PersistBatch &b, int mode) {
-  int64_t cost = 0;
-  int min_k32 = 1 << 30;
+  int64_t tiles_per_xcd = 0;
   for (int i = 0; i < b.n_problems; ++i) {
     const PersistProblem &p = b.prob[i];
     const int bn_out = mode == kFc1Swiglu ? kPBN / 2 : (p.n % 192 == 0 && p.n % 256 != 0 ? 192 : kPBN);
     const int64_t m_tiles = ((int64_t)p.max_rows + kPBM - 1) / kPBM + p.n_experts;
     const int64_t n_tiles = (p.n + bn_out - 1) / bn_out;
-    cost += m_tiles * n_tiles * (p.k / 32);
-    min_k32 = p.k / 32 < min_k32 ? p.k / 32 : min_k32;
+    tiles_per_xcd += m_tiles * n_tiles / kNumXcd + 1;
   }
   const int wgs_per_xcd = cu_count() / kNumXcd;
-  const int64_t tiles_per_xcd = cost / kNumXcd / min_k32 + 2;
   return (tiles_per_xcd + wgs_per_xcd - 1) / wgs_per_xcd + 2 <= kTableTurns;
 }
 
@@ -2137,6 +2300,11 @@ int DICE_PERSIST_LAUNCH(const PersistBatch &b, int mode, hipStream_t s) {
   }
   PersistBatch launch = b;
   launch.band_tiles = persist_band_tiles(mode);
+  const PersistPlan plan = persist_plan(b, mode == kFc1Swiglu ? kPBN / 2 : narrow ? 192 : kPBN, grid);
+  if (plan.longest_first)
+    std::stable_sort(launch.prob, launch.prob + launch.n_problems,
+                     [](const PersistProblem &x, const PersistProblem &y) { return x.k > y.k; });
+  launch.xcd_split = plan.xcd_split;
   // (a last turn cut along k: the plain epilogue is linear in k; the 32-k kernel
   // does not read its tiles from the table that describes the pieces)
   if (mode != kFc2 || waves != 4 || b.n_problems != 1 || grid / kNumXcd < 2 || grid > kPersistSplitSlots ||
