@@ -42,7 +42,6 @@
 #include <type_traits>
 
 #include <algorithm>
-#include <cstring>
 #include <vector>
 
 #include "gemm_common.h"
@@ -2040,11 +2039,14 @@ PersistPlan persist_plan(const PersistBatch &b, int bn_out, int grid) {
   constexpr int kRemembered = 8;
   static thread_local Shape seen[kRemembered];
   static thread_local int n_seen = 0, next = 0;
-  for (int i = 0; i < n_seen; ++i) {
-    Shape c = seen[i];
-    c.plan = PersistPlan{};
-    if (memcmp(&c, &key, sizeof(Shape)) == 0) return seen[i].plan;
-  }
+  auto same = [](const Shape &a, const Shape &c) {
+    if (a.n_problems != c.n_problems || a.bn_out != c.bn_out || a.grid != c.grid) return false;
+    for (int p = 0; p < a.n_problems; ++p)
+      if (a.rows[p] != c.rows[p] || a.experts[p] != c.experts[p] || a.n[p] != c.n[p] || a.k[p] != c.k[p]) return false;
+    return true;
+  };
+  for (int i = 0; i < n_seen; ++i)
+    if (same(seen[i], key)) return seen[i].plan;
   PersistProblem sorted[kMaxPersistProblems];
   std::copy(b.prob, b.prob + b.n_problems, sorted);
   std::stable_sort(sorted, sorted + b.n_problems,
