@@ -20,7 +20,7 @@ from tests.helpers import block_from_params, check_rows, rel_l2
 
 pytestmark = pytest.mark.gpu
 
-BF16_TOL, SAME_QUANT_TOL, FP8_TOL = 2e-2, 1e-2, 5e-2
+BF16_TOL, F16_TOL, SAME_QUANT_TOL, FP8_TOL = 2e-2, 4e-3, 1e-2, 5e-2
 
 
 @pytest.fixture(scope="module")
@@ -55,27 +55,30 @@ def _whole_and_cut(blk, x):
     return whole.cpu(), blk(x).cpu()
 
 
-@pytest.mark.parametrize("variant,D,ratio,E,n_shared,N", [
-    ("swiglu", 768, 2, 4, 0, 1024),      # 192-wide fc2 tiles, no shared expert: one problem per launch
-    ("gelu_tanh", 768, 2, 4, 0, 1024),   # ... with biases: added by a tile's first piece only
-    ("gelu_tanh", 1024, 2, 4, 0, 1536),  # 256-wide fc2 tiles: the bias enters through the accumulators
-    ("swiglu", 1024, 3, 8, 0, 777),      # ragged groups, 48 steps
-    ("swiglu", 1152, 2, 8, 0, 2000),     # 36 steps in pieces of 8 to 14
-    ("gelu_tanh", 1152, 1, 4, 0, 900),   # 18 steps: at most three pieces of 6
+@pytest.mark.parametrize("variant,D,ratio,E,n_shared,N,dtype", [
+    ("swiglu", 768, 2, 4, 0, 1024, torch.bfloat16),      # 192-wide fc2 tiles, no shared expert: one problem per launch
+    ("gelu_tanh", 768, 2, 4, 0, 1024, torch.bfloat16),   # ... with biases: added by a tile's first piece only
+    ("gelu_tanh", 1024, 2, 4, 0, 1536, torch.bfloat16),  # 256-wide fc2 tiles: the bias enters through the accumulators
+    ("swiglu", 1024, 3, 8, 0, 777, torch.bfloat16),      # ragged groups, 48 steps
+    ("swiglu", 1152, 2, 8, 0, 2000, torch.bfloat16),     # 36 steps in pieces of 8 to 14
+    ("gelu_tanh", 1152, 1, 4, 0, 900, torch.bfloat16),   # 18 steps: at most three pieces of 6
+    ("swiglu", 768, 2, 4, 0, 1024, torch.float16),       # the fp16 build of the same kernels (pieces in fp16)
+    ("gelu_tanh", 1024, 2, 4, 0, 1536, torch.float16),
 ])
-def test_bf16_block_cut_last_turn(dev, variant, D, ratio, E, n_shared, N):
-    p = O.make_block_params(D, E, 2, ratio, n_shared, seed=21, dtype=torch.bfloat16, variant=variant)
+def test_16bit_block_cut_last_turn(dev, variant, D, ratio, E, n_shared, N, dtype):
+    p = O.make_block_params(D, E, 2, ratio, n_shared, seed=21, dtype=dtype, variant=variant)
     if variant == "gelu_tanh":
-        _bias_params(p, 22)
-    x = torch.randn(1, N, D, generator=_gen(23)).bfloat16()
-    blk = block_from_params(p, D, variant, torch.bfloat16, dev)
+        _bias_params(p, 22, dtype)
+    x = torch.randn(1, N, D, generator=_gen(23)).to(dtype)
+    blk = block_from_params(p, D, variant, dtype, dev)
     whole, cut = _whole_and_cut(blk, x.to(dev))
     want, _, _, logits = O.sparse_moe_block_forward(p, x)
     ok = ~O.gate_tie_rows(logits, 2).view(-1)
-    check_rows(whole.view(-1, D)[ok], want.view(-1, D)[ok], BF16_TOL, "whole tiles vs oracle")
-    check_rows(cut.view(-1, D)[ok], want.view(-1, D)[ok], BF16_TOL, "cut last turn vs oracle")
+    tol = BF16_TOL if dtype == torch.bfloat16 else F16_TOL
+    check_rows(whole.view(-1, D)[ok], want.view(-1, D)[ok], tol, "whole tiles vs oracle")
+    check_rows(cut.view(-1, D)[ok], want.view(-1, D)[ok], tol, "cut last turn vs oracle")
     assert not torch.equal(cut, whole), "the cut did not apply: the test's shape no longer exercises it"
-    check_rows(cut.view(-1, D), whole.view(-1, D), 4e-3, "cut last turn vs whole tiles")
+    check_rows(cut.view(-1, D), whole.view(-1, D), tol / 5, "cut last turn vs whole tiles")
 
 
 @pytest.mark.parametrize("variant", ["swiglu", "gelu_tanh"])
