@@ -210,7 +210,7 @@ __device__ __forceinline__ TilePos tile_pos(int r, int mt, int nt, int band_tile
 // Split turn.  The tiles of an XCD's run rarely fill its last turn: with R tiles
 // left for W workgroups, W - R of them would idle for a whole tile.  Where the
 // launch allows it (PersistBatch::split_ws: a plain-epilogue launch, whose
-// products are linear in k) and R <= W / 2, the W workgroups are dealt out over
+// products are linear in k) and R <= W / 3, the W workgroups are dealt out over
 // those R tiles - W / R of them per tile, one more for the first W % R tiles, at
 // most kSplitMaxWays - and each multiplies one piece of its tile's k range: runs
 // of an even number of steps, at least kSplitMinSteps, that differ by at most
@@ -366,7 +366,13 @@ struct TileWalker {
     if (batch.split_ws == nullptr || split_left <= 0) return;
     const int q = wgs_per_xcd / split_left;
     const int cap = batch.prob[0].k / bk / kSplitMinSteps;   // pieces of at least kSplitMinSteps steps
-    if (q < 2 || cap < 2) return;
+    // (A cut turn has no operand reuse between its workgroups: it runs at the
+    // rate at which the XCD can bring in its tiles' operands, about a twelfth of a
+    // tile's multiply time per tile, whatever the number of pieces - 8 tiles per
+    // XCD at 2048 x 8192 took 55 us where a whole tile takes 93.  With fewer
+    // than three workgroups per tile the cut no longer pays for itself and the
+    // sum of its pieces.)
+    if (q < 3 || cap < 2) return;
     split_cap = cap < kSplitMaxWays ? cap : kSplitMaxWays;
     split_q = q;
     split_extra = wgs_per_xcd - q * split_left;

@@ -1,4 +1,6 @@
 """Shared helpers of the GPU parity tests."""
+import contextlib
+
 import torch
 
 from oracle import dice_oracle as O
@@ -64,3 +66,19 @@ def zipf_bias(E, s=1.2):
     pr = torch.tensor([(e + 1.0) ** -s for e in range(E)])
     pr = pr / pr.sum()
     return pr.log()
+
+
+@contextlib.contextmanager
+def whole_fc2_tiles():
+    """Every fc2 tile multiplied whole (tuning hook, fc2 = 50).  By default an fc2
+    launch may cut the left-over tiles of a short last turn along k; how many
+    depends on the tile count, and the sums of the 16-bit pieces differ from a
+    whole tile's in the last bit, so tests that ask for bit-identical outputs
+    from calls with different token counts run under this
+    (tests/test_gpu_split_turn.py covers the cut itself)."""
+    from dice_amd import lib
+    lib.load().dice_set_gemm_config(0, 50)
+    try:
+        yield
+    finally:
+        lib.load().dice_set_gemm_config(0, 0)

@@ -11,7 +11,7 @@ import pytest
 import torch
 
 from oracle import dice_oracle as O
-from tests.helpers import block_from_params, check_rows, rel_l2, zipf_bias
+from tests.helpers import block_from_params, check_rows, rel_l2, whole_fc2_tiles, zipf_bias
 
 pytestmark = pytest.mark.gpu
 
@@ -656,13 +656,14 @@ def test_block_many_tokens_per_workgroup(dev):
     D, E, N = 384, 8, 172032
     p = O.make_block_params(D, E, 2, 4, 2, seed=5, dtype=torch.bfloat16, variant="swiglu")
     x = torch.randn(1, N, D, generator=_gen(5)).bfloat16()
-    blk, y = _run_block(dev, p, x, "swiglu", torch.bfloat16)
+    with whole_fc2_tiles():
+        blk, y = _run_block(dev, p, x, "swiglu", torch.bfloat16)
+        xq = x.view(4, N // 4, D).to(dev)
+        parts = torch.cat([blk(xq[i:i + 1]).cpu() for i in range(4)], dim=1)
     sub = torch.randperm(N, generator=_gen(6))[:256]
     want, _, logits = _subset_oracle(p, x.view(-1, D), sub, torch.bfloat16)
     ties = O.gate_tie_rows(logits, 2).view(-1)
     assert rel_l2(y.view(-1, D)[sub][~ties], want[~ties]) < BF16_TOL
-    xq = x.view(4, N // 4, D).to(dev)
-    parts = torch.cat([blk(xq[i:i + 1]).cpu() for i in range(4)], dim=1)
     assert torch.equal(parts.view(-1, D), y.view(-1, D))
 
 
@@ -674,9 +675,10 @@ def test_block_xl_width_large_batch_matches_chunks(dev):
     D, E, N = 1152, 8, 73728
     p = O.make_block_params(D, E, 2, 4, 2, seed=8, dtype=torch.bfloat16)
     x = torch.randn(1, N, D, generator=_gen(8)).bfloat16()
-    blk, y = _run_block(dev, p, x, "swiglu", torch.bfloat16)
-    xq = x.view(N // 8192, 8192, D).to(dev)
-    parts = torch.cat([blk(xq[i:i + 1]).cpu() for i in range(N // 8192)], dim=1)
+    with whole_fc2_tiles():
+        blk, y = _run_block(dev, p, x, "swiglu", torch.bfloat16)
+        xq = x.view(N // 8192, 8192, D).to(dev)
+        parts = torch.cat([blk(xq[i:i + 1]).cpu() for i in range(N // 8192)], dim=1)
     assert torch.equal(parts.view(-1, D), y.view(-1, D))
     sub = torch.randperm(N, generator=_gen(9))[:128]
     want, _, logits = _subset_oracle(p, x.view(-1, D), sub, torch.bfloat16)
@@ -703,18 +705,10 @@ def test_rewritten_tile_table_other_kernels(dev, variant, dtype, fp8, N):
     if fp8:
         blk.quantize_fp8()
     x = torch.randn(1, N, D, generator=torch.Generator(device=dev).manual_seed(14), device=dev).to(dtype)
-    from dice_amd import lib
-    # Whole fc2 tiles only: a single-problem fc2 launch otherwise cuts the tiles of a
-    # short last turn along k, how many depends on the tile count, and the sums
-    # of its 16-bit pieces differ from a whole tile's in the last bit
-    # (tests/test_gpu_split_turn.py covers that path).
-    lib.load().dice_set_gemm_config(0, 50)
-    try:
+    with whole_fc2_tiles():
         y = blk(x)
         chunk = N // 8
         parts = torch.cat([blk(x[:, i:i + chunk]) for i in range(0, N, chunk)], dim=1)
-    finally:
-        lib.load().dice_set_gemm_config(0, 0)
     assert torch.equal(parts, y)
     assert torch.isfinite(y.float()).all() and float(y.float().abs().max()) > 0
 
@@ -807,8 +801,13 @@ def test_skip_full_size_identities(dev):
         cache = torch.empty_like(x)
         put = blk.run(x, MODE_PUT, mask, None, cache).clone()
         assert torch.equal(put, plain)
-        skip = blk.run(x, MODE_SKIP, mask, cache, None).clone()
-        assert torch.equal(skip, plain)
+        # (bit for bit with whole fc2 tiles; by default a skip step, with half the
+        # rows, may cut other left-over tiles along k than the full step did)
+        with whole_fc2_tiles():
+            assert torch.equal(blk.run(x, MODE_PLAIN), plain)
+            skip = blk.run(x, MODE_SKIP, mask, cache, None).clone()
+            assert torch.equal(skip, plain)
+        check_rows(blk.run(x, MODE_SKIP, mask, cache, None).cpu(), plain.cpu(), 4e-3, "skip step on its own cache")
         # a drifted input with the stale cache stays close to its own full result
         x2 = (x.float() + 0.05 * torch.randn(N, D, generator=_gen(8)).to(dev)).bfloat16()
         full2 = blk.run(x2, MODE_PLAIN).clone()

@@ -5,8 +5,9 @@ fc2 = 50) must agree to the rounding of the 16-bit partial tiles, and both
 must meet the oracle (models.py:252-273, 292-296, 302-382) at the bar of the
 other block tests.
 
-Shapes are chosen so that every XCD's run leaves a handful of tiles for its
-32 workgroups (a few dozen tiles per launch, at least 12 steps per tile): the
+Shapes are chosen so that every XCD's run leaves a handful of tiles (at most
+a third of its 32 workgroups' worth; a few dozen tiles per launch, at least
+12 steps per tile): the
 cut applies in every launch checked here, with even and uneven pieces, which
 the tests confirm by asking for outputs that are close but not bit-identical.
 """
@@ -60,7 +61,7 @@ def _whole_and_cut(blk, x):
     ("gelu_tanh", 768, 2, 4, 0, 1024, torch.bfloat16),   # ... with biases: added by a tile's first piece only
     ("gelu_tanh", 1024, 2, 4, 0, 1536, torch.bfloat16),  # 256-wide fc2 tiles: the bias enters through the accumulators
     ("swiglu", 1024, 3, 8, 0, 777, torch.bfloat16),      # ragged groups, 48 steps
-    ("swiglu", 1152, 2, 8, 0, 2000, torch.bfloat16),     # 36 steps in pieces of 8 to 14
+    ("swiglu", 1152, 2, 8, 0, 1000, torch.bfloat16),     # 36 steps in pieces of 8 to 14
     ("gelu_tanh", 1152, 1, 4, 0, 900, torch.bfloat16),   # 18 steps: at most three pieces of 6
     ("swiglu", 768, 2, 4, 0, 1024, torch.float16),       # the fp16 build of the same kernels (pieces in fp16)
     ("gelu_tanh", 1024, 2, 4, 0, 1536, torch.float16),
