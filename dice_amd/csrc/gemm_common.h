@@ -134,10 +134,14 @@ __device__ __forceinline__ float sigmoid_fast(float z) {
   return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * z));
 }
 __device__ __forceinline__ float silu_fast(float g) { return g * sigmoid_fast(g); }
-// 0.5 x (1 + tanh(u)) = x sigmoid(2u)
+// 0.5 x (1 + tanh(u)) = x sigmoid(2u), u = k0 (x + k1 x^3): the exponent of the
+// sigmoid is x (c0 + c1 x^2) with the constants folded (three multiplies and one
+// fused multiply-add per value beside the two transcendentals).
 __device__ __forceinline__ float gelu_tanh_fast(float x) {
-  const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-  return x * sigmoid_fast(2.0f * k0 * (x + k1 * x * x * x));
+  constexpr float k0 = 0.7978845608028654f, k1 = 0.044715f;
+  constexpr float c0 = -2.0f * k0 * 1.4426950408889634f, c1 = c0 * k1;
+  const float z = x * __builtin_fmaf(x * x, c1, c0);
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(z));
 }
 
 // One grouped GEMM of a persistent launch: grouped activation rows (row r of
