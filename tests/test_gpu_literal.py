@@ -134,6 +134,44 @@ def test_literal_block_rewritten_tile_table(dev):
     assert torch.equal(parts, y)
 
 
+@pytest.mark.parametrize("mode", ["high", "rand"])
+def test_literal_block_full_and_skip_step(dev, mode):
+    """The config-literal block (GELU-tanh, biases, shared expert with the longer
+    k) through a full step that fills the cache and a skip step on a drifted
+    input, every token against the oracle (moe_infer_ep with the same mask and
+    cache, ep_fwd.py:49-66,176-193).  The skip step's fc2 launch is the one that
+    re-orders its problems (longest k first) and takes an eighth of every
+    problem's tiles per XCD."""
+    from dice_amd.lib import MODE_PUT, MODE_SKIP
+    D, E, N = 1152, 8, 8192
+    p = _literal_params(D, E, seed=41)
+    blk = block_from_params(p, D, "gelu_tanh", torch.bfloat16, dev)
+    g = _gen(42)
+    mask = O.skip_mask(2 * N, mode)
+    if mode == "rand":
+        m2 = torch.zeros((N, 2), dtype=torch.bool)
+        m2[torch.arange(N), torch.randint(0, 2, (N,), generator=g)] = True
+        mask = m2.view(-1)
+    mask_d = mask.to(dev)
+    x = torch.randn(N, D, generator=g).bfloat16()
+    ocache = O.EPSkipCache(1)
+    cache_d = torch.empty(N, D, dtype=torch.bfloat16, device=dev)
+    y = blk.run(x.to(dev), MODE_PUT, mask_d, None, cache_d).cpu()
+    want, _, _, logits = O.sparse_moe_block_forward(p, x.unsqueeze(0), skip_mask_=mask, skip_now_=False,
+                                                    cache=ocache, cache_key=0)
+    ok = ~O.gate_tie_rows(logits, 2).view(-1)
+    check_rows(y[ok], want[0][ok], BF16_TOL, "full step")
+    cache = cache_d.cpu()
+    check_rows(cache[ok], ocache.get(0)[ok], BF16_TOL, "cache rows written by the full step")
+    x2 = (x.float() + 0.05 * torch.randn(N, D, generator=g)).bfloat16()
+    y2 = blk.run(x2.to(dev), MODE_SKIP, mask_d, cache_d, None).cpu()
+    ocache.put(0, cache)
+    want2, _, _, logits2 = O.sparse_moe_block_forward(p, x2.unsqueeze(0), skip_mask_=mask, skip_now_=True,
+                                                      cache=ocache, cache_key=0)
+    ok2 = ~O.gate_tie_rows(logits2, 2).view(-1)
+    check_rows(y2[ok2], want2[0][ok2], BF16_TOL, f"skip step ({mode})")
+
+
 # --------------------------------------------------------------------------- #
 # configs[3]: the staleness loop at full size in bf16
 # --------------------------------------------------------------------------- #
