@@ -308,7 +308,7 @@ def time_lagged(cfg, variant, dev, x, steps, warmup, pipeline):
         diep.use_latest_expert_weights(False)
 
 
-def time_caller(cfg, blk, x, steps, warmup):
+def time_caller(cfg, blk, x, steps, warmup, hook=(0, 0)):
     """The MoE line of the reference's DiTBlock.forward, x + gate * moe(modulate(norm2(x))):
     ms per call with the prologue / epilogue inside the library, with them as torch eager ops
     around the plain layer call (what the reference's DiTBlock does), and the prologue kernel
@@ -331,16 +331,26 @@ def time_caller(cfg, blk, x, steps, warmup):
     def prologue():
         ops.ln_modulate(xs, shift, scale)
 
+    from dice_amd import lib
     res = {}
-    for name, fn in (("fused", fused), ("eager_caller", eager), ("ln_modulate_kernel", prologue)):
-        for _ in range(warmup):
-            fn()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            fn()
-        torch.cuda.synchronize()
-        res[name] = (time.perf_counter() - t0) / steps * 1e3
+    # "fused": prologue and router in one launch; "fused_router_own_launch": the same call with
+    # the router behind the prologue kernel as a launch of its own (tuning hook).
+    for name, fn in (("fused", fused), ("fused_router_own_launch", fused), ("eager_caller", eager),
+                     ("ln_modulate_kernel", prologue)):
+        if name == "fused_router_own_launch":
+            lib.load().dice_set_gemm_config(50, hook[1])
+        try:
+            for _ in range(warmup):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                fn()
+            torch.cuda.synchronize()
+            res[name] = (time.perf_counter() - t0) / steps * 1e3
+        finally:
+            if name == "fused_router_own_launch":
+                lib.load().dice_set_gemm_config(*hook)
     res["ln_modulate_frac_of_hbm_peak"] = (2 * cfg["tokens"] * D * x.element_size()
                                            / (res["ln_modulate_kernel"] * 1e-3) / 1e9 / PEAK_HBM_GBS)
     return res
@@ -581,7 +591,7 @@ def main():
         if key in res:
             out[key] = res[key]
     if not args.no_caller:
-        out["block_moe_half_ms"] = time_caller(cfg, blk, x, args.steps, args.warmup)
+        out["block_moe_half_ms"] = time_caller(cfg, blk, x, args.steps, args.warmup, (args.fc1_cfg, args.fc2_cfg))
     if not args.no_staleness and main_cfg == "c2":
         # configs[3] on the same block shape (not part of `value`)
         out["staleness_loop_50_steps"] = time_staleness(CONFIGS["c4"], args.variant, dev, x)

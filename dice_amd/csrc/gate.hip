@@ -9,10 +9,12 @@
 // sizes - takes gate_topk_kernel, one wavefront per 64 / E tokens, where the
 // router matrix comes from the vector cache, or, when it is too large for
 // that, from LDS, and each wave keeps 64/E tokens in flight so one read of a
-// router chunk feeds that many dot-product updates.
+// router chunk feeds that many dot-product updates.  A third kernel
+// (ln_modulate_route_kernel) runs the caller's LayerNorm + modulation prologue
+// and the matrix-pipe router in one launch.
 #include <type_traits>
 
-#include "common.h"
+#include "modulate_row.h"
 
 namespace dice {
 
@@ -287,46 +289,22 @@ template <> struct RouterMfma<f16_t> {
   }
 };
 
-template <typename T, int EP, int WPB>
-__device__ __forceinline__ void gate_topk_mfma_body(
-    const T *__restrict__ x, const T *__restrict__ w, const float *__restrict__ bias, int64_t n_tokens,
-    int hidden, int n_experts, int top_k, int norm_topk, int32_t *__restrict__ topk_idx,
-    int64_t *__restrict__ topk_idx64, float *__restrict__ topk_weight, float *__restrict__ logits_out) {
-  constexpr int NR = EP / 2;  // accumulator registers of a lane that hold experts below EP
-  __shared__ float part[WPB][NR][kWave];
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
-  const int col = lane & 31, half = lane >> 5;
-  const int64_t tok = (int64_t)blockIdx.x * 32 + col;
-  const int64_t tok_c = tok < n_tokens ? tok : n_tokens - 1;   // (columns past the end repeat the last token)
-  const int steps = hidden / 16 / WPB;                         // per wave; at most kRouterMaxSteps
-  const int seg = (wave * 2 + half) * steps * 8;               // this lane's segment of the hidden dimension
-  const T *xp = x + tok_c * hidden + seg;
-  const T *wp = w + (size_t)(col < n_experts ? col : n_experts - 1) * hidden + seg;
-  Vec8<T> xv[kRouterMaxSteps], wv[kRouterMaxSteps];
-#pragma unroll
-  for (int s = 0; s < kRouterMaxSteps; ++s) {
-    const int at = s < steps ? s : 0;   // (no branch around a load: steps past the end re-read the first chunk)
-    xv[s] = load8(xp + at * 8);
-    wv[s] = load8(wp + at * 8);
-  }
-  f32x16_t acc;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-#pragma unroll
-  for (int s = 0; s < kRouterMaxSteps; ++s)
-    if (s < steps) acc = RouterMfma<T>::mul(wv[s].v, xv[s].v, acc);
-  // lane (col, half), register a: logit of expert 8 (a / 4) + 4 half + a % 4 for token col
-#pragma unroll
-  for (int a = 0; a < NR; ++a) part[wave][a][lane] = acc[a];
-  __syncthreads();
-  if (wave != 0) return;
+// Second half of the matrix-pipe router, run by one wave: adds the `waves`
+// partial logit tiles in `part` ([waves][EP / 2][64] floats in LDS, lane (col,
+// half), register a = expert 8 (a / 4) + 4 half + a % 4 of token col) in wave
+// order, then softmax and top-k with all of a token's logits in one lane.
+template <int EP>
+__device__ __forceinline__ void router_mfma_finish(
+    const float *part, int waves, int lane, int64_t tok, const float *__restrict__ bias, int64_t n_tokens,
+    int n_experts, int top_k, int norm_topk, int32_t *__restrict__ topk_idx, int64_t *__restrict__ topk_idx64,
+    float *__restrict__ topk_weight, float *__restrict__ logits_out) {
+  constexpr int NR = EP / 2;
+  const int half = lane >> 5;
   float mine[NR], other[NR];
 #pragma unroll
   for (int a = 0; a < NR; ++a) {
-    float v = part[0][a][lane];
-#pragma unroll
-    for (int q = 1; q < WPB; ++q) v += part[q][a][lane];
+    float v = part[a * kWave + lane];
+    for (int q = 1; q < waves; ++q) v += part[(q * NR + a) * kWave + lane];
     mine[a] = v;
   }
 #pragma unroll
@@ -389,6 +367,43 @@ __device__ __forceinline__ void gate_topk_mfma_body(
       topk_weight[tok * top_k + j] = wgt;
     }
 }
+template <typename T, int EP, int WPB>
+__device__ __forceinline__ void gate_topk_mfma_body(
+    const T *__restrict__ x, const T *__restrict__ w, const float *__restrict__ bias, int64_t n_tokens,
+    int hidden, int n_experts, int top_k, int norm_topk, int32_t *__restrict__ topk_idx,
+    int64_t *__restrict__ topk_idx64, float *__restrict__ topk_weight, float *__restrict__ logits_out) {
+  constexpr int NR = EP / 2;  // accumulator registers of a lane that hold experts below EP
+  __shared__ float part[WPB][NR][kWave];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int col = lane & 31, half = lane >> 5;
+  const int64_t tok = (int64_t)blockIdx.x * 32 + col;
+  const int64_t tok_c = tok < n_tokens ? tok : n_tokens - 1;   // (columns past the end repeat the last token)
+  const int steps = hidden / 16 / WPB;                         // per wave; at most kRouterMaxSteps
+  const int seg = (wave * 2 + half) * steps * 8;               // this lane's segment of the hidden dimension
+  const T *xp = x + tok_c * hidden + seg;
+  const T *wp = w + (size_t)(col < n_experts ? col : n_experts - 1) * hidden + seg;
+  Vec8<T> xv[kRouterMaxSteps], wv[kRouterMaxSteps];
+#pragma unroll
+  for (int s = 0; s < kRouterMaxSteps; ++s) {
+    const int at = s < steps ? s : 0;   // (no branch around a load: steps past the end re-read the first chunk)
+    xv[s] = load8(xp + at * 8);
+    wv[s] = load8(wp + at * 8);
+  }
+  f32x16_t acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+  for (int s = 0; s < kRouterMaxSteps; ++s)
+    if (s < steps) acc = RouterMfma<T>::mul(wv[s].v, xv[s].v, acc);
+  // lane (col, half), register a: logit of expert 8 (a / 4) + 4 half + a % 4 for token col
+#pragma unroll
+  for (int a = 0; a < NR; ++a) part[wave][a][lane] = acc[a];
+  __syncthreads();
+  if (wave != 0) return;
+  router_mfma_finish<EP>(&part[0][0][0], WPB, lane, tok, bias, n_tokens, n_experts, top_k, norm_topk, topk_idx,
+                         topk_idx64, topk_weight, logits_out);
+}
 // (builtins that only exist for the device stay out of the __global__ template's own body)
 template <typename T, int EP, int WPB>
 __global__ __launch_bounds__(WPB *kWave) void gate_topk_mfma_kernel(
@@ -421,6 +436,142 @@ int launch_gate_mfma(const void *x, const void *w, const float *bias, int64_t n_
     hipLaunchKernelGGL((gate_topk_mfma_kernel<T, EP, 8>), dim3(blocks), dim3(8 * kWave), 0, stream, (const T *)x,
                        (const T *)w, bias, n_tokens, hidden, n_experts, top_k, norm, idx, idx64, wt, logits);
   return launch_status("dice_gate_topk");
+}
+
+// ---------------------------------------------------------------------------
+// The caller's prologue and the router in one launch: a workgroup of 16 waves
+// takes 32 tokens.  Each wave normalises and modulates two rows in registers
+// (both requested up front: one memory round trip), writes them to the layer
+// input in HBM and to LDS; after one barrier the first `wpb` waves multiply the
+// LDS copy with the router matrix exactly as gate_topk_mfma_body multiplies the
+// rows it loads from memory (same segments of the hidden dimension per wave and
+// lane half, same order of products and sums: bit-identical logits), and the
+// first wave finishes.  Against the two separate launches the modulated rows
+// are not read back from memory and one launch ramp goes away.  LDS rows are
+// one 16-byte chunk longer than the row, so the 32 lanes of a half-wave, which
+// read the same chunk of 32 different rows, fall into different banks.
+constexpr int kRouteWaves = 16;
+constexpr int kRouteChunks = 3;   // 16-byte chunks of a row per lane: rows up to 1536 16-bit elements
+
+template <typename T, int EP>
+__device__ __forceinline__ void ln_modulate_route_body(
+    const Chunk<T> *__restrict__ x, const Chunk<T> *__restrict__ shift, const Chunk<T> *__restrict__ scale,
+    Chunk<T> *__restrict__ out, int64_t n_tokens, int chunks_per_row, int64_t tokens_per_sample, float inv_hidden,
+    float eps, const T *__restrict__ w, const float *__restrict__ bias, int n_experts, int top_k, int norm_topk,
+    int wpb, int32_t *__restrict__ topk_idx, float *__restrict__ topk_weight) {
+  constexpr int NR = EP / 2;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const int pitch = chunks_per_row + 1;                         // LDS row pitch in chunks
+  Chunk<T> *rows = reinterpret_cast<Chunk<T> *>(lds_raw);       // [32][pitch]
+  float *part = reinterpret_cast<float *>(lds_raw + (size_t)32 * pitch * sizeof(Chunk<T>));  // [wpb][NR][64]
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int64_t t_base = (int64_t)blockIdx.x * 32;
+
+  Chunk<T> v[2][kRouteChunks], ms[2][kRouteChunks], mh[2][kRouteChunks];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int64_t t = t_base + wave * 2 + j;
+    const int64_t tt = t < n_tokens ? t : n_tokens - 1;         // (rows past the end repeat the last token)
+    const int64_t b = tt / tokens_per_sample;
+    const Chunk<T> *row = x + tt * chunks_per_row;
+    const Chunk<T> *sc = scale + b * chunks_per_row;
+    const Chunk<T> *sh = shift + b * chunks_per_row;
+#pragma unroll
+    for (int i = 0; i < kRouteChunks; ++i) {
+      const int c = lane + i * kWave;
+      if (c < chunks_per_row) {
+        v[j][i] = row[c];
+        ms[j][i] = sc[c];
+        mh[j][i] = sh[c];
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    ln_modulate_row<T, kRouteChunks>(v[j], ms[j], mh[j], lane, chunks_per_row, inv_hidden, eps);
+    const int64_t t = t_base + wave * 2 + j;
+    Chunk<T> *dst = out + t * chunks_per_row;
+    Chunk<T> *lrow = rows + (wave * 2 + j) * pitch;
+#pragma unroll
+    for (int i = 0; i < kRouteChunks; ++i) {
+      const int c = lane + i * kWave;
+      if (c < chunks_per_row) {
+        if (t < n_tokens) dst[c] = v[j][i];
+        lrow[c] = v[j][i];
+      }
+    }
+  }
+
+  const int col = lane & 31, half = lane >> 5;
+  const int steps = chunks_per_row / 2 / wpb;                   // per wave; at most kRouterMaxSteps
+  const int seg = (wave * 2 + half) * steps;                    // this lane's segment, in chunks
+  Vec8<T> wv[kRouterMaxSteps];
+  if (wave < wpb) {
+    const T *wp = w + ((size_t)(col < n_experts ? col : n_experts - 1) * chunks_per_row + seg) * 8;
+#pragma unroll
+    for (int s = 0; s < kRouterMaxSteps; ++s) wv[s] = load8(wp + (s < steps ? s : 0) * 8);
+  }
+  __syncthreads();
+  if (wave < wpb) {
+    const Chunk<T> *xp = rows + col * pitch + seg;
+    f32x16_t acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+    for (int s = 0; s < kRouterMaxSteps; ++s)
+      if (s < steps) acc = RouterMfma<T>::mul(wv[s].v, xp[s].v, acc);
+#pragma unroll
+    for (int a = 0; a < NR; ++a) part[(wave * NR + a) * kWave + lane] = acc[a];
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  router_mfma_finish<EP>(part, wpb, lane, t_base + col, bias, n_tokens, n_experts, top_k, norm_topk, topk_idx,
+                         nullptr, topk_weight, nullptr);
+}
+template <typename T, int EP>
+__global__ __launch_bounds__(kRouteWaves *kWave) void ln_modulate_route_kernel(
+    const Chunk<T> *__restrict__ x, const Chunk<T> *__restrict__ shift, const Chunk<T> *__restrict__ scale,
+    Chunk<T> *__restrict__ out, int64_t n_tokens, int chunks_per_row, int64_t tokens_per_sample, float inv_hidden,
+    float eps, const T *__restrict__ w, const float *__restrict__ bias, int n_experts, int top_k, int norm_topk,
+    int wpb, int32_t *__restrict__ topk_idx, float *__restrict__ topk_weight) {
+  ln_modulate_route_body<T, EP>(x, shift, scale, out, n_tokens, chunks_per_row, tokens_per_sample, inv_hidden, eps,
+                                w, bias, n_experts, top_k, norm_topk, wpb, topk_idx, topk_weight);
+}
+
+template <typename T, int EP>
+int launch_ln_modulate_route(const void *x, const void *shift, const void *scale, void *out, int64_t n_tokens,
+                             int hidden, int64_t tokens_per_sample, float eps, const void *w, const float *bias,
+                             int n_experts, int top_k, int norm, int32_t *idx, float *wt, hipStream_t stream) {
+  const int chunks = hidden / 8;
+  const int wpb = router_mfma_waves(hidden);
+  const size_t lds = (size_t)32 * (chunks + 1) * 16 + (size_t)wpb * (EP / 2) * kWave * sizeof(float);
+  auto kern = ln_modulate_route_kernel<T, EP>;
+  static size_t lds_allowed = 64 * 1024;   // (per instantiation: the attribute belongs to the kernel, not to a call)
+  if (lds > lds_allowed) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail(DICE_ERR_LAUNCH, "ln_modulate + router: LDS attribute: %s", hipGetErrorString(e));
+    lds_allowed = lds;
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)((n_tokens + 31) / 32)), dim3(kRouteWaves * kWave), lds, stream,
+                     (const Chunk<T> *)x, (const Chunk<T> *)shift, (const Chunk<T> *)scale, (Chunk<T> *)out, n_tokens,
+                     chunks, tokens_per_sample, 1.0f / (float)hidden, eps, (const T *)w, bias, n_experts, top_k, norm,
+                     wpb, idx, wt);
+  return launch_status("dice_moe_forward_modulated");
+}
+template <typename T>
+int ln_modulate_route_experts(const void *x, const void *shift, const void *scale, void *out, int64_t n_tokens,
+                              int hidden, int64_t tokens_per_sample, float eps, const void *w, const float *bias,
+                              int n_experts, int top_k, int norm, int32_t *idx, float *wt, hipStream_t s) {
+  if (n_experts <= 8)
+    return launch_ln_modulate_route<T, 8>(x, shift, scale, out, n_tokens, hidden, tokens_per_sample, eps, w, bias,
+                                          n_experts, top_k, norm, idx, wt, s);
+  if (n_experts <= 16)
+    return launch_ln_modulate_route<T, 16>(x, shift, scale, out, n_tokens, hidden, tokens_per_sample, eps, w, bias,
+                                           n_experts, top_k, norm, idx, wt, s);
+  return launch_ln_modulate_route<T, 32>(x, shift, scale, out, n_tokens, hidden, tokens_per_sample, eps, w, bias,
+                                         n_experts, top_k, norm, idx, wt, s);
 }
 
 template <typename XT, typename WT>
@@ -458,6 +609,34 @@ int dispatch_wtype(int x_dtype, int w_dtype, const void *x, const void *w, const
 }
 
 }  // namespace
+
+bool ln_modulate_route_applies(int act_dtype, int gate_w_dtype, int64_t n_tokens, int hidden, int n_experts) {
+  return (act_dtype == DICE_BF16 || act_dtype == DICE_F16) && gate_w_dtype == act_dtype && n_experts <= 32 &&
+         n_tokens >= 1 && n_tokens < (1ll << 31) / 32 && hidden <= kRouteChunks * kWave * 8 &&
+         router_mfma_waves(hidden) != 0;
+}
+
+int ln_modulate_route_impl(const void *x, const void *shift, const void *scale, void *out, int dtype,
+                           int64_t n_tokens, int hidden, int64_t tokens_per_sample, float eps, const void *gate_w,
+                           const float *gate_bias, int n_experts, int top_k, int norm_topk_prob, int32_t *topk_idx,
+                           float *topk_weight, void *stream) {
+  DICE_REQUIRE(ln_modulate_route_applies(dtype, dtype, n_tokens, hidden, n_experts), DICE_ERR_UNSUPPORTED,
+               "ln_modulate + router: dtype %d, hidden %d, %d experts are outside the fused kernel", dtype, hidden,
+               n_experts);
+  DICE_REQUIRE(x && shift && scale && out && gate_w && topk_idx && topk_weight, DICE_ERR_BAD_ARG,
+               "ln_modulate + router: null pointer");
+  DICE_REQUIRE(tokens_per_sample >= 1 && eps >= 0.f, DICE_ERR_BAD_ARG,
+               "ln_modulate + router: tokens_per_sample %lld, eps %g", (long long)tokens_per_sample, (double)eps);
+  DICE_REQUIRE(top_k >= 1 && top_k <= 8 && top_k <= n_experts, DICE_ERR_BAD_ARG,
+               "ln_modulate + router: top_k %d outside [1, min(8, n_experts)]", top_k);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == DICE_BF16)
+    return ln_modulate_route_experts<bf16_t>(x, shift, scale, out, n_tokens, hidden, tokens_per_sample, eps, gate_w,
+                                             gate_bias, n_experts, top_k, norm_topk_prob, topk_idx, topk_weight, s);
+  return ln_modulate_route_experts<f16_t>(x, shift, scale, out, n_tokens, hidden, tokens_per_sample, eps, gate_w,
+                                          gate_bias, n_experts, top_k, norm_topk_prob, topk_idx, topk_weight, s);
+}
+
 }  // namespace dice
 
 extern "C" int dice_gate_topk(const void *x, int x_dtype, const void *w, int w_dtype,

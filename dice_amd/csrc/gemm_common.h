@@ -186,6 +186,7 @@ bool persist_supported(const PersistBatch &b, int mode);
 int persist_cu_count();  // compute units of the current device
 int persist_band_tiles(int mode);  // tuning hook state: band height of the tile order for this stage (0 = default rule)
 bool persist_split_allowed();      // tuning hook state: fc2 launches of the layer call may cut their last turn along k
+bool route_in_prologue_allowed();   // tuning hook state: the modulated layer call may route inside its prologue kernel
 bool gemm_config_allows_persistent(int mode);  // tuning hook state: no tiling of the permutation-addressed kernels is forced for this stage
 int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s);      // bf16
 int launch_grouped_gemm_persist_f16(const PersistBatch &b, int mode, hipStream_t s);  // fp16
@@ -197,6 +198,15 @@ int launch_grouped_gemm_persist_f8(const PersistBatch &b, int mode, hipStream_t 
 // caller's residual / gate epilogue behind it (modulate.hip, combine.hip).
 int ln_modulate_impl(const void *x, const void *shift, const void *scale, void *out, int dtype,
                      int64_t n_tokens, int hidden, int64_t tokens_per_sample, float eps, void *stream);
+// The same prologue with the router in the same launch (gate.hip): writes the
+// modulated rows and their top-k routing; `applies` says whether the shape is
+// one the kernel takes (16-bit rows of at most 1536 elements, a router matrix
+// of the same type, at most 32 experts).
+bool ln_modulate_route_applies(int act_dtype, int gate_w_dtype, int64_t n_tokens, int hidden, int n_experts);
+int ln_modulate_route_impl(const void *x, const void *shift, const void *scale, void *out, int dtype,
+                           int64_t n_tokens, int hidden, int64_t tokens_per_sample, float eps, const void *gate_w,
+                           const float *gate_bias, int n_experts, int top_k, int norm_topk_prob, int32_t *topk_idx,
+                           float *topk_weight, void *stream);
 int combine_impl(const void *slot_out, const int32_t *inv_perm, const float *topk_weight,
                  const void *shared_out, const uint8_t *skip_mask, const void *cache_in, void *cache_out,
                  void *y, int dtype, int64_t n_tokens, int top_k, int hidden, const void *resid,

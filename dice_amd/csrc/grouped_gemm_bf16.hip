@@ -411,6 +411,7 @@ int persist_band_tiles(int mode) {
   return cfg > 30 && cfg <= 46 ? cfg - 30 : 0;
 }
 bool persist_split_allowed() { return g_cfg_fc2 != 50; }
+bool route_in_prologue_allowed() { return g_cfg_fc1 != 50; }
 }  // namespace dice
 
 // Tuning hook, per GEMM stage.  0 (default) and values >= 20: dice_grouped_mlp
@@ -421,7 +422,8 @@ bool persist_split_allowed() { return g_cfg_fc2 != 50; }
 // persistent launches of that stage in bands of b m-tiles (each band taken
 // through every n-tile before the next); 50 (fc2) has the layer call multiply every
 // tile of its fc2 launches whole instead of cutting the tiles of a short last turn
-// along k.  1 .. 4 name a tiling of this file's kernels for
+// along k; 50 (fc1) has dice_moe_forward_modulated launch the router on its own
+// instead of inside the prologue kernel.  1 .. 4 name a tiling of this file's kernels for
 // dice_grouped_mlp whatever the shape (1: 256x256 / 8 waves; 2: 256x128 / 4
 // waves; 3: 64x64 outputs / 4 waves; 4: 128x128).  Not part of the drop-in
 // surface; used by the benchmark and the tests to compare kernels.

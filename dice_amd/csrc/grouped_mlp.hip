@@ -449,17 +449,26 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
   // straight into the entry that outlives the call when there is one; x itself
   // is then only the residual of the epilogue.
   const void *resid = nullptr;
+  bool routed = false;
   if (caller) {
     void *hm = put ? put->x : w.modulated;
     DICE_REQUIRE(hm != x, DICE_ERR_BAD_ARG, "%s: the entry's input buffer aliases x", who);
-    rc = ln_modulate_impl(x, caller->shift, caller->scale, hm, L->act_dtype, n_tokens, L->hidden,
-                          caller->tokens_per_sample, caller->ln_eps, stream);
+    // The router runs inside the prologue kernel where that kernel takes the
+    // shape: the modulated rows are then routed from LDS, not read back.
+    routed = route_in_prologue_allowed() &&
+             ln_modulate_route_applies(L->act_dtype, L->gate_w_dtype, n_tokens, L->hidden, L->n_experts);
+    rc = routed ? ln_modulate_route_impl(x, caller->shift, caller->scale, hm, L->act_dtype, n_tokens, L->hidden,
+                                         caller->tokens_per_sample, caller->ln_eps, L->gate_w, L->gate_bias,
+                                         L->n_experts, L->top_k, L->norm_topk_prob, idx, wt, stream)
+                : ln_modulate_impl(x, caller->shift, caller->scale, hm, L->act_dtype, n_tokens, L->hidden,
+                                   caller->tokens_per_sample, caller->ln_eps, stream);
     if (rc) return rc;
     resid = x;
     x = hm;
   }
-  rc = dice_gate_topk(x, L->act_dtype, L->gate_w, L->gate_w_dtype, L->gate_bias, n_tokens, L->hidden,
-                      L->n_experts, L->top_k, L->norm_topk_prob, idx, nullptr, wt, nullptr, stream);
+  if (!routed)
+    rc = dice_gate_topk(x, L->act_dtype, L->gate_w, L->gate_w_dtype, L->gate_bias, n_tokens, L->hidden,
+                        L->n_experts, L->top_k, L->norm_topk_prob, idx, nullptr, wt, nullptr, stream);
   if (rc) return rc;
   if (put && topk_weight_out)
     DICE_HIP(hipMemcpyAsync(topk_weight_out, wt, slots * sizeof(float), hipMemcpyDeviceToDevice, s));

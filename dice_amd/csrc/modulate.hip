@@ -10,30 +10,10 @@
 // kMaxChunks 16-byte chunks per lane), mean and variance are two exact passes
 // over those registers in fp32 (variance around the mean, biased, eps inside
 // the square root, as torch.nn.LayerNorm), and the result is rounded once.
-#include "common.h"
+#include "modulate_row.h"
 
 namespace dice {
 namespace {
-
-template <typename T> struct Chunk;  // 16 bytes of a row
-template <> struct Chunk<float> {
-  static constexpr int kN = 4;
-  f32x4_t v;
-  __device__ __forceinline__ float get(int i) const { return v[i]; }
-  __device__ __forceinline__ void set(int i, float f) { v[i] = f; }
-};
-template <> struct Chunk<bf16_t> {
-  static constexpr int kN = 8;
-  bf16x8_t v;
-  __device__ __forceinline__ float get(int i) const { return (float)v[i]; }
-  __device__ __forceinline__ void set(int i, float f) { v[i] = (bf16_t)f; }
-};
-template <> struct Chunk<f16_t> {
-  static constexpr int kN = 8;
-  f16x8_t v;
-  __device__ __forceinline__ float get(int i) const { return (float)v[i]; }
-  __device__ __forceinline__ void set(int i, float f) { v[i] = (f16_t)f; }
-};
 
 constexpr int kModWaves = 4;
 
@@ -42,7 +22,6 @@ __global__ __launch_bounds__(kModWaves *kWave) void ln_modulate_kernel(
     const Chunk<T> *__restrict__ x, const Chunk<T> *__restrict__ shift,
     const Chunk<T> *__restrict__ scale, Chunk<T> *__restrict__ out, int64_t n_tokens,
     int chunks_per_row, int64_t tokens_per_sample, float inv_hidden, float eps) {
-  constexpr int N = Chunk<T>::kN;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   for (int64_t t = (int64_t)blockIdx.x * kModWaves + wave; t < n_tokens;
@@ -63,39 +42,12 @@ __global__ __launch_bounds__(kModWaves *kWave) void ln_modulate_kernel(
         mh[i] = sh[c];
       }
     }
-    float sum = 0.f;
-#pragma unroll
-    for (int i = 0; i < MAXC; ++i) {
-      if (lane + i * kWave < chunks_per_row) {
-#pragma unroll
-        for (int e = 0; e < N; ++e) sum += v[i].get(e);
-      }
-    }
-    const float mean = wave_sum(sum) * inv_hidden;
-    float sq = 0.f;
-#pragma unroll
-    for (int i = 0; i < MAXC; ++i) {
-      if (lane + i * kWave < chunks_per_row) {
-#pragma unroll
-        for (int e = 0; e < N; ++e) {
-          const float d = v[i].get(e) - mean;
-          sq = fmaf(d, d, sq);
-        }
-      }
-    }
-    const float rstd = 1.0f / sqrtf(wave_sum(sq) * inv_hidden + eps);
+    ln_modulate_row<T, MAXC>(v, ms, mh, lane, chunks_per_row, inv_hidden, eps);
     Chunk<T> *dst = out + t * chunks_per_row;
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
       const int c = lane + i * kWave;
-      if (c < chunks_per_row) {
-        const Chunk<T> s = ms[i], h = mh[i];
-        Chunk<T> o;
-#pragma unroll
-        for (int e = 0; e < N; ++e)
-          o.set(e, fmaf((v[i].get(e) - mean) * rstd, 1.0f + s.get(e), h.get(e)));
-        dst[c] = o;
-      }
+      if (c < chunks_per_row) dst[c] = v[i];
     }
   }
 }

@@ -403,8 +403,9 @@ int dice_profile_read(float *ms_out, int n);
  * bf16/fp8 expert GEMMs per stage (0 = library default).  1..4 force a tiling
  * of the permutation-addressed kernels; 20 restricts the persistent launches to
  * the 32-k pipeline; 30 + b (b = 1..16) walks the persistent launches' tiles in
- * bands of b m-tiles; fc2_cfg = 50 has the layer calls multiply every fc2 tile
- * whole.  (By default a single-problem fc2 launch - fp8 routed weights, or no
+ * bands of b m-tiles; fc1_cfg = 50 has dice_moe_forward_modulated launch the
+ * router on its own behind the prologue kernel instead of inside it (same
+ * results); fc2_cfg = 50 has the layer calls multiply every fc2 tile whole.  (By default a single-problem fc2 launch - fp8 routed weights, or no
  * shared expert - whose tiles leave most workgroups idle in their last turn
  * cuts that turn's tiles along k, one piece per workgroup, and adds the 16-bit
  * pieces in fp32 in a fixed order: results are deterministic, but a token's last

@@ -62,6 +62,18 @@ def block_from_params(p: O.MoEBlockParams, D, variant="swiglu", dtype=torch.floa
     return blk
 
 
+@contextlib.contextmanager
+def router_own_launch():
+    """The modulated layer call with the router as a launch of its own behind the
+    prologue kernel (tuning hook, fc1 = 50) instead of inside it."""
+    from dice_amd import lib
+    lib.load().dice_set_gemm_config(50, 0)
+    try:
+        yield
+    finally:
+        lib.load().dice_set_gemm_config(0, 0)
+
+
 def zipf_bias(E, s=1.2):
     pr = torch.tensor([(e + 1.0) ** -s for e in range(E)])
     pr = pr / pr.sum()
