@@ -37,6 +37,14 @@ __device__ __forceinline__ void wave_lds_sync() {
   __builtin_amdgcn_wave_barrier();
 }
 
+// Workgroup barrier for data exchanged through LDS: waits for this wave's LDS
+// traffic only, not for its outstanding global loads and stores (which
+// __syncthreads() would drain first).
+__device__ __forceinline__ void block_lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+}
+
 // Records a printf-style message for dice_last_error() and returns `code`.
 int fail(int code, const char *fmt, ...);
 

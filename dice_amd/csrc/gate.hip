@@ -488,21 +488,12 @@ __device__ __forceinline__ void ln_modulate_route_body(
     }
   }
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
+  for (int j = 0; j < 2; ++j)
     ln_modulate_row<T, kRouteChunks>(v[j], ms[j], mh[j], lane, chunks_per_row, inv_hidden, eps);
-    const int64_t t = t_base + wave * 2 + j;
-    Chunk<T> *dst = out + t * chunks_per_row;
-    Chunk<T> *lrow = rows + (wave * 2 + j) * pitch;
-#pragma unroll
-    for (int i = 0; i < kRouteChunks; ++i) {
-      const int c = lane + i * kWave;
-      if (c < chunks_per_row) {
-        if (t < n_tokens) dst[c] = v[j][i];
-        lrow[c] = v[j][i];
-      }
-    }
-  }
 
+  // The router matrix is requested before the rows are stored: the wait for it
+  // behind the barrier then does not wait for the stores as well (one counter
+  // covers both, in issue order).
   const int col = lane & 31, half = lane >> 5;
   const int steps = chunks_per_row / 2 / wpb;                   // per wave; at most kRouterMaxSteps
   const int seg = (wave * 2 + half) * steps;                    // this lane's segment, in chunks
@@ -512,19 +503,43 @@ __device__ __forceinline__ void ln_modulate_route_body(
 #pragma unroll
     for (int s = 0; s < kRouterMaxSteps; ++s) wv[s] = load8(wp + (s < steps ? s : 0) * 8);
   }
-  __syncthreads();
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int64_t t = t_base + wave * 2 + j;
+    Chunk<T> *dst = out + t * chunks_per_row;
+    Chunk<T> *lrow = rows + (wave * 2 + j) * pitch;
+#pragma unroll
+    for (int i = 0; i < kRouteChunks; ++i) {
+      const int c = lane + i * kWave;
+      if (c < chunks_per_row) {
+        lrow[c] = v[j][i];
+        if (t < n_tokens) dst[c] = v[j][i];
+      }
+    }
+  }
+  block_lds_barrier();   // (LDS only: the rows' way to memory is not waited for)
   if (wave < wpb) {
     const Chunk<T> *xp = rows + col * pitch + seg;
     f32x16_t acc;
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+    // LDS reads six at a time in front of their products (no branch around a read:
+    // steps past the end re-read the first chunk)
+    constexpr int kReads = 6;
 #pragma unroll
-    for (int s = 0; s < kRouterMaxSteps; ++s)
-      if (s < steps) acc = RouterMfma<T>::mul(wv[s].v, xp[s].v, acc);
+    for (int s0 = 0; s0 < kRouterMaxSteps; s0 += kReads) {
+      Chunk<T> xb[kReads];
+#pragma unroll
+      for (int i = 0; i < kReads; ++i) xb[i] = xp[s0 + i < steps ? s0 + i : 0];
+#pragma unroll
+      for (int i = 0; i < kReads; ++i)
+        if (s0 + i < steps) acc = RouterMfma<T>::mul(wv[s0 + i].v, xb[i].v, acc);
+    }
 #pragma unroll
     for (int a = 0; a < NR; ++a) part[(wave * NR + a) * kWave + lane] = acc[a];
   }
-  __syncthreads();
+  block_lds_barrier();
   if (wave != 0) return;
   router_mfma_finish<EP>(part, wpb, lane, t_base + col, bias, n_tokens, n_experts, top_k, norm_topk, topk_idx,
                          nullptr, topk_weight, nullptr);
@@ -547,12 +562,15 @@ int launch_ln_modulate_route(const void *x, const void *shift, const void *scale
   const int wpb = router_mfma_waves(hidden);
   const size_t lds = (size_t)32 * (chunks + 1) * 16 + (size_t)wpb * (EP / 2) * kWave * sizeof(float);
   auto kern = ln_modulate_route_kernel<T, EP>;
-  static size_t lds_allowed = 64 * 1024;   // (per instantiation: the attribute belongs to the kernel, not to a call)
-  if (lds > lds_allowed) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return fail(DICE_ERR_LAUNCH, "ln_modulate + router: LDS attribute: %s", hipGetErrorString(e));
-    lds_allowed = lds;
+  // More than 64 KB of dynamic LDS has to be allowed per kernel and device, once.
+  constexpr int kMaxDevices = 64;
+  static size_t lds_allowed[kMaxDevices] = {};   // (per instantiation)
+  int dev = 0;
+  DICE_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices || lds > lds_allowed[dev]) {
+    DICE_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                 (int)lds));
+    if (dev >= 0 && dev < kMaxDevices) lds_allowed[dev] = lds;
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)((n_tokens + 31) / 32)), dim3(kRouteWaves * kWave), lds, stream,
                      (const Chunk<T> *)x, (const Chunk<T> *)shift, (const Chunk<T> *)scale, (Chunk<T> *)out, n_tokens,
