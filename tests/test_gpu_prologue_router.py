@@ -92,3 +92,46 @@ def test_prologue_router_twice_and_smaller(dev):
             b = _run(blk, x, shift, scale, gate)
         for u, v in zip(a, b):
             assert torch.equal(u, v)
+
+
+def test_prologue_router_in_lagged_calls(dev):
+    """Displaced mode through the fused caller: the prologue writes the modulated
+    rows and the routing straight into the entry that outlives the call; four
+    steps with the router inside the prologue equal four with it as its own
+    launch, bit for bit."""
+    from dice_amd import ParaMode, diep
+    B, T, D = 2, 96, 256
+    p = O.make_block_params(D, 8, 2, 2, 2, seed=3, dtype=torch.bfloat16, gate_std=0.1)
+    pm = ParaMode(ep=True, ep_async=True, ep_async_mode="all")
+    blk = block_from_params(p, D, "swiglu", torch.bfloat16, dev, para_mode=pm)
+
+    def four_steps():
+        diep.ep_cache_init(cache_capacity=1)
+        diep.use_latest_expert_weights(True)
+        outs = []
+        try:
+            for t in range(4):
+                g = torch.Generator().manual_seed(20 + t)
+                x = (torch.randn(B, T, D, generator=g) * 2 + 0.5).to(torch.bfloat16).to(dev)
+                shift, scale, gate = ((torch.randn(B, D, generator=g) * 0.3).to(torch.bfloat16).to(dev)
+                                      for _ in range(3))
+                if t == 0:
+                    diep.diep_force_sync()
+                    diep.ep_cache_clear()
+                outs.append(blk.forward_modulated(x, shift, scale, gate).cpu())
+                if t == 0:
+                    diep.diep_cancel_sync()
+        finally:
+            diep.ep_cache_init(cache_capacity=1)
+            diep.use_latest_expert_weights(False)
+            if diep.diep_forced_sync():
+                diep.diep_cancel_sync()
+        return outs
+
+    a = four_steps()
+    with router_own_launch():
+        b = four_steps()
+    for t, (u, v) in enumerate(zip(a, b)):
+        assert torch.isfinite(u.float()).all()
+        assert torch.equal(u, v), f"step {t}"
+    assert not torch.equal(a[1], a[2])
