@@ -187,12 +187,21 @@ int persist_cu_count();  // compute units of the current device
 int persist_band_tiles(int mode);  // tuning hook state: band height of the tile order for this stage (0 = default rule)
 bool persist_split_allowed();      // tuning hook state: fc2 launches of the layer call may cut their last turn along k
 bool route_in_prologue_allowed();   // tuning hook state: the modulated layer call may route inside its prologue kernel
+bool gemm_config_is_default(int mode);  // tuning hook state: nothing is set for this stage
 bool gemm_config_allows_persistent(int mode);  // tuning hook state: no tiling of the permutation-addressed kernels is forced for this stage
 int launch_grouped_gemm_persist(const PersistBatch &b, int mode, hipStream_t s);      // bf16
 int launch_grouped_gemm_persist_f16(const PersistBatch &b, int mode, hipStream_t s);  // fp16
 // fp8 activations (a_scale) and weights (w_scale) on the fp8 matrix pipe, bf16 output
 bool persist_f8_supported(const PersistBatch &b, int mode);
 int launch_grouped_gemm_persist_f8(const PersistBatch &b, int mode, hipStream_t s);
+
+// Few rows per group (at most 128 on average): a 256-row tile of the persistent
+// kernels is then mostly padding - its matrix-pipe time is that of a full tile -
+// and a launch a single short turn, while the permutation-addressed kernels
+// with 64-row tiles only stream the weights (DiT-XL width, 8 experts: 63 against
+// 117 us for both stages at 128 slots, 98 against 120 at 1024, 155 against 135
+// at 2048).
+inline bool few_rows_per_group(int64_t max_rows, int n_groups) { return max_rows <= 128ll * n_groups; }
 
 // LayerNorm + adaLN modulation in front of the layer, and the combine with the
 // caller's residual / gate epilogue behind it (modulate.hip, combine.hip).

@@ -412,6 +412,7 @@ int persist_band_tiles(int mode) {
 }
 bool persist_split_allowed() { return g_cfg_fc2 != 50; }
 bool route_in_prologue_allowed() { return g_cfg_fc1 != 50; }
+bool gemm_config_is_default(int mode) { return (mode == kFc2 ? g_cfg_fc2 : g_cfg_fc1) == 0; }
 }  // namespace dice
 
 // Tuning hook, per GEMM stage.  0 (default) and values >= 20: dice_grouped_mlp
@@ -423,7 +424,10 @@ bool route_in_prologue_allowed() { return g_cfg_fc1 != 50; }
 // through every n-tile before the next); 50 (fc2) has the layer call multiply every
 // tile of its fc2 launches whole instead of cutting the tiles of a short last turn
 // along k; 50 (fc1) has dice_moe_forward_modulated launch the router on its own
-// instead of inside the prologue kernel.  1 .. 4 name a tiling of this file's kernels for
+// instead of inside the prologue kernel.  Any value from 20 on also keeps a
+// dice_grouped_mlp stage whose groups average at most 128 rows on the persistent
+// kernels (21 does only that; by default such a stage takes this file's 64-row
+// tiles).  1 .. 4 name a tiling of this file's kernels for
 // dice_grouped_mlp whatever the shape (1: 256x256 / 8 waves; 2: 256x128 / 4
 // waves; 3: 64x64 outputs / 4 waves; 4: 128x128).  Not part of the drop-in
 // surface; used by the benchmark and the tests to compare kernels.

@@ -271,8 +271,10 @@ int grouped_mlp_impl(int stages, const void *x, int act_dtype, const int32_t *pe
       pb1.prob[0].w_scale = w1_scale;
       pb2.prob[0].w_scale = w2_scale;
     }
-    fc1_persist = gemm_config_allows_persistent(m1) && persist_supported(pb1, m1);
-    fc2_persist = !scatter_to_slots && gemm_config_allows_persistent(kFc2) && persist_supported(pb2, kFc2);
+    const bool few = few_rows_per_group(max_rows, n_experts);
+    fc1_persist = gemm_config_allows_persistent(m1) && !(few && gemm_config_is_default(m1)) && persist_supported(pb1, m1);
+    fc2_persist = !scatter_to_slots && gemm_config_allows_persistent(kFc2) &&
+                  !(few && gemm_config_is_default(kFc2)) && persist_supported(pb2, kFc2);
   }
 
   if (stages & 1) {

@@ -405,7 +405,10 @@ int dice_profile_read(float *ms_out, int n);
  * the 32-k pipeline; 30 + b (b = 1..16) walks the persistent launches' tiles in
  * bands of b m-tiles; fc1_cfg = 50 has dice_moe_forward_modulated launch the
  * router on its own behind the prologue kernel instead of inside it (same
- * results); fc2_cfg = 50 has the layer calls multiply every fc2 tile whole.  (By default a single-problem fc2 launch - fp8 routed weights, or no
+ * results); fc2_cfg = 50 has the layer calls multiply every fc2 tile whole;
+ * any value from 20 on (21 does nothing else) keeps a dice_grouped_mlp stage
+ * whose groups average at most 128 rows on the persistent kernels, which by
+ * default leave it to the 64-row tiles of the permutation-addressed ones.  (By default a single-problem fc2 launch - fp8 routed weights, or no
  * shared expert - whose tiles leave most workgroups idle in their last turn
  * cuts that turn's tiles along k, one piece per workgroup, and adds the 16-bit
  * pieces in fp32 in a fixed order: results are deterministic, but a token's last

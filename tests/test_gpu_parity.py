@@ -317,6 +317,17 @@ def test_mlp_bf16_persistent_kernels(dev, variant, cfg):
     _check_mlp_persistent(dev, 512, 512, 8, 2, variant, cfg, counts=[1024, 0, 0, 0, 0, 0, 0, 0])
 
 
+@pytest.mark.parametrize("cfg", [0, 21])   # 0: groups of few rows take the 64-row tiles; 21: they stay on the persistent kernels
+@pytest.mark.parametrize("variant", ["swiglu", "gelu_tanh"])
+def test_mlp_few_rows_per_group(dev, variant, cfg):
+    """Small sampling batches through the per-stage entry point: at most 128 rows
+    per expert on average, both kernel families against the oracle."""
+    _check_mlp(dev, 64, 1152, 8, 4, torch.bfloat16, variant, cfg=(cfg, cfg))     # 16 rows per expert
+    _check_mlp(dev, 300, 768, 8, 4, torch.float16, variant, cfg=(cfg, cfg), tol=F16_TOL)
+    _check_mlp(dev, 512, 1152, 8, 4, torch.bfloat16, variant, cfg=(cfg, cfg))    # exactly 128 on average
+    _check_mlp(dev, 7, 512, 8, 2, torch.bfloat16, variant, cfg=(cfg, cfg), counts=[0, 1, 0, 0, 13, 0, 0, 0])
+
+
 def test_mlp_bf16_biased_tiles_across_experts(dev):
     """GELU experts with non-zero biases at XL width, enough rows that every
     workgroup multiplies several tiles in a row, of different experts and
