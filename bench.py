@@ -332,25 +332,33 @@ def time_caller(cfg, blk, x, steps, warmup, hook=(0, 0)):
         ops.ln_modulate(xs, shift, scale)
 
     from dice_amd import lib
-    res = {}
     # "fused": prologue and router in one launch; "fused_router_own_launch": the same call with
-    # the router behind the prologue kernel as a launch of its own (tuning hook).
-    for name, fn in (("fused", fused), ("fused_router_own_launch", fused), ("eager_caller", eager),
-                     ("ln_modulate_kernel", prologue)):
-        if name == "fused_router_own_launch":
-            lib.load().dice_set_gemm_config(50, hook[1])
-        try:
-            for _ in range(warmup):
-                fn()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(steps):
-                fn()
-            torch.cuda.synchronize()
-            res[name] = (time.perf_counter() - t0) / steps * 1e3
-        finally:
+    # the router behind the prologue kernel as a launch of its own (tuning hook).  The legs take
+    # turns in short rounds, so that a drift of the board's clocks falls on all of them alike.
+    legs = (("fused", fused), ("fused_router_own_launch", fused), ("eager_caller", eager),
+            ("ln_modulate_kernel", prologue))
+    rounds = 5
+    per_round = max(1, steps // rounds)
+    total = {name: 0.0 for name, _ in legs}
+    reps = {name: 20 if name == "ln_modulate_kernel" else 1 for name, _ in legs}   # (a 10 us kernel: more calls per wait)
+    for r in range(rounds):
+        for name, fn in legs:
             if name == "fused_router_own_launch":
-                lib.load().dice_set_gemm_config(*hook)
+                lib.load().dice_set_gemm_config(50, hook[1])
+            try:
+                for _ in range(warmup if r == 0 else 2):
+                    fn()
+                n = per_round * reps[name]
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(n):
+                    fn()
+                torch.cuda.synchronize()
+                total[name] += time.perf_counter() - t0
+            finally:
+                if name == "fused_router_own_launch":
+                    lib.load().dice_set_gemm_config(*hook)
+    res = {name: total[name] / (rounds * per_round * reps[name]) * 1e3 for name, _ in legs}
     res["ln_modulate_frac_of_hbm_peak"] = (2 * cfg["tokens"] * D * x.element_size()
                                            / (res["ln_modulate_kernel"] * 1e-3) / 1e9 / PEAK_HBM_GBS)
     return res
