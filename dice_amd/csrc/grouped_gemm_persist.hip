@@ -962,10 +962,12 @@ __device__ __forceinline__ void gemm_persist_body(const PersistBatch &batch) {
   #pragma unroll
         for (int kk = 0; kk < 2; ++kk)
   #pragma unroll
-          for (int i = 0; i < TM; ++i)
+          for (int j = 0; j < TN; ++j)
   #pragma unroll
-            for (int j = 0; j < TN; ++j)
-              acc[i][j] = mfma_32x32x16(wf[kk][j], af[kk][i], acc[i][j]);
+            for (int i = 0; i < TM; ++i) {
+              const int ii = (j & 1) ? TM - 1 - i : i;   // (one operand changes per product, see mfma_block below)
+              acc[ii][j] = mfma_32x32x16(wf[kk][j], af[kk][ii], acc[ii][j]);
+            }
         __builtin_amdgcn_s_setprio(DICE_PRIO_MEMORY);
         if (group == 0) copies_landed();
         phase_barrier();
@@ -1290,12 +1292,21 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
 #pragma unroll
         for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
   };
+  // The 16 products of a 16-k block, weight block by weight block with the row
+  // blocks up and down in turn: from one product to the next only one operand
+  // changes, the left one (the weights) every fourth time.  The launch is bound
+  // by the board's power limit, and the order in which the same products are
+  // issued moves it: row blocks outermost, weights changing every time, 616 us
+  // per layer call at 8192 x 1152; the same with the weight blocks down and up
+  // 607; this order 598-603 (same box, calls taking turns; same sums, bit for bit).
   auto mfma_block = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
-        acc[i][j] = mfma_32x32x16(wf[buf][j], af[buf][i], acc[i][j]);
+      for (int i = 0; i < TM; ++i) {
+        const int ii = (j & 1) ? TM - 1 - i : i;
+        acc[ii][j] = mfma_32x32x16(wf[buf][j], af[buf][ii], acc[ii][j]);
+      }
   };
 
   // ---- pipeline state ----
@@ -1499,12 +1510,14 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
 //     step), see load_quarter.
 //   * Fragments twice the size do not fit twice in the register file, so they
 //     are not double-buffered.  A step is two halves of 16 MFMAs (one per 64-k
-//     block), taken row block by row block; during a half the next half's
-//     fragments are read into the registers of operands as they die: row block
-//     i behind the four MFMAs that use it, the weight blocks one by one during
-//     the last row block, and what the half's last MFMA still holds (the last
-//     weight block and the last row block) right behind it.  Eight fragments =
-//     64 registers, as many as the bf16 kernel's double-buffered set.
+//     block), taken weight block by weight block (the row blocks up and down in
+//     turn, so that only one operand changes from one product to the next);
+//     during a half the next half's fragments are read into the registers of
+//     operands as they die: weight block j behind the four MFMAs that use it,
+//     the row blocks one by one during the last weight block, and what the
+//     half's last MFMA still holds (the last weight block and one row block)
+//     right behind it.  Eight fragments = 64 registers, as many as the bf16
+//     kernel's double-buffered set.
 //   * The workgroup barrier sits four MFMAs into the second half: by then
 //     every wave has read the step's slot for the last time (the trailing reads
 //     of the first half have had four MFMAs to land) and has finished writing
@@ -1524,10 +1537,10 @@ __device__ __forceinline__ f32x16_t mfma_f8_32x32x64(i32x8_t a, i32x8_t b, f32x1
   return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
 }
 
-// Instruction order of one half.  MFMA m (row block m / 4) is followed by the
-// fragment reads whose registers have just come free: row block 0 behind MFMAs 4
-// and 5, row block 1 behind 8 and 9, row block 2 and three weight blocks in pairs
-// behind 12..15, the last weight block and row block 3 behind the half; and by
+// Instruction order of one half.  MFMA m (weight block m / 4) is followed by the
+// fragment reads whose registers have just come free: weight block 0 behind MFMAs
+// 4 and 5, weight block 1 behind 8 and 9, weight block 2 and three row blocks in
+// pairs behind 12..15, the last row block and weight block 3 behind the half; and by
 // the LDS writes of a register stage alternating with the global loads that
 // refill it, from MFMA FIRST on (the second half of a step starts them behind its
 // barrier: 16 of them over 12 MFMAs).
@@ -1820,13 +1833,17 @@ __device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) 
   // and A, while the fragments of block RKB of slot RSLOT replace them, quarters
   // WQ and WQ + 1 of their register stage go to LDS slot WSLOT and are loaded
   // again for the step the load side stands at.  BARRIER: the workgroup barrier of the step
-  // sits behind the first row block; everything but MFMAs follows it.
+  // sits behind the first weight block; everything but MFMAs follows it.
   auto half = [&](auto rslot_c, auto rkb_c, auto wslot_c, auto wq_c, auto barrier_c) {
     constexpr int WQ = decltype(wq_c)::value;
     constexpr bool BARRIER = decltype(barrier_c)::value != 0;
+    static_assert(TM == TN, "the half below treats row blocks and weight blocks alike");
+    // Weight block by weight block, the row blocks up and down in turn: from one
+    // product to the next only one operand changes, the left one (the weights)
+    // every fourth time.
     if constexpr (BARRIER) {
 #pragma unroll
-      for (int j = 0; j < TN; ++j) acc[0][j] = mfma_f8_32x32x64(W[j], A[0], acc[0][j]);
+      for (int i = 0; i < TM; ++i) acc[i][0] = mfma_f8_32x32x64(W[0], A[i], acc[i][0]);
       // This wave has read the step's slot for the last time and has finished
       // writing the other slot; after the barrier both hold for every wave.
       __builtin_amdgcn_sched_barrier(0);
@@ -1834,29 +1851,32 @@ __device__ __forceinline__ void gemm_persist_f8_body(const PersistBatch &batch) 
       phase_barrier();
     }
     // (program order = the order in which the registers come free)
-    const i32x8_t na0 = read_a(rslot_c, rkb_c, 0);
-    const i32x8_t na1 = read_a(rslot_c, rkb_c, 1);
-    const i32x8_t na2 = read_a(rslot_c, rkb_c, 2);
-    i32x8_t nw[TN];
+    const i32x8_t nw0 = read_w(rslot_c, rkb_c, 0);
+    const i32x8_t nw1 = read_w(rslot_c, rkb_c, 1);
+    const i32x8_t nw2 = read_w(rslot_c, rkb_c, 2);
+    i32x8_t na[TM];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) nw[j] = read_w(rslot_c, rkb_c, j);
-    const i32x8_t na3 = read_a(rslot_c, rkb_c, 3);
+    for (int i = 0; i < TM; ++i) na[i] = read_a(rslot_c, rkb_c, i);   // (the last column runs the row blocks 3..0)
+    const i32x8_t nw3 = read_w(rslot_c, rkb_c, 3);
     write_quarter(wslot_c, template_int<WQ>{});
     load_quarter(wslot_c, template_int<WQ>{});
     write_quarter(wslot_c, template_int<WQ + 1>{});
     load_quarter(wslot_c, template_int<WQ + 1>{});
 #pragma unroll
-    for (int i = BARRIER ? 1 : 0; i < TM; ++i)
+    for (int j = BARRIER ? 1 : 0; j < TN; ++j)
 #pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = mfma_f8_32x32x64(W[j], A[i], acc[i][j]);
+      for (int i = 0; i < TM; ++i) {
+        const int ii = (j & 1) ? TM - 1 - i : i;
+        acc[ii][j] = mfma_f8_32x32x64(W[j], A[ii], acc[ii][j]);
+      }
     f8_sched_half<0, BARRIER ? 4 : 0>();
     __builtin_amdgcn_sched_barrier(0);
-    A[0] = na0;
-    A[1] = na1;
-    A[2] = na2;
-    A[3] = na3;
+    W[0] = nw0;
+    W[1] = nw1;
+    W[2] = nw2;
+    W[3] = nw3;
 #pragma unroll
-    for (int j = 0; j < TN; ++j) W[j] = nw[j];
+    for (int i = 0; i < TM; ++i) A[i] = na[i];
   };
 
   while (true) {  // one tile per iteration
