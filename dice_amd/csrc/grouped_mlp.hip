@@ -364,6 +364,27 @@ namespace {
 // this call's routing (NULL: it lives in the workspace), `work` names the entry
 // whose routed experts run now and `emit` the entry that is combined into y
 // (NULL: the entry one stage earlier in put -> work -> emit).
+// Small batches: all fc2 tiles of the routed and the shared expert together fill
+// less than half of the compute units, the launch lasts as long as its longest
+// tile, and a launch with two problems does not cut tiles along k.  The shared
+// expert's fc2 then gets a launch of its own, so that both launches cut theirs
+// (one piece per idle workgroup).  Measured at DiT-XL width, joint / separate, us
+// per layer call: SwiGLU experts (shared k = 2304) 132 / 124 at 64 tokens, 146 /
+// 142 at 512, 155 / 156 at 768, 164 / 167 at 1024; GELU experts with a shared
+// expert of 2 x the routed width (k = 9216: twice the routed tiles' length) 166 /
+// 116 at 64, 174 / 134 at 512, 216 / 190 at 1024, 241 / 242 at 1536.  The bound
+// on the tile count is the host's (row counts live on the device).
+bool shared_fc2_alone(const dice_moe_layer_t *L, int64_t n_tokens, int64_t max_rows) {
+  const int choice = shared_fc2_launch_choice();
+  if (choice != 0) return choice > 0;
+  // (tiles of fewer than 64 steps: a second launch costs what the cut saves - DiT-B width, 48 and 24
+  // steps: 95 / 89 us at 64 tokens, but 114 / 119 at 1024 and 121 / 129 at 1536)
+  if (!persist_split_allowed() || (L->inter < 4096 && L->shared_inter < 4096)) return false;
+  const int64_t m_tiles = max_rows / 256 + L->n_experts + n_tokens / 256 + 1;
+  const int64_t tiles = m_tiles * ((L->hidden + 255) / 256);
+  return tiles * 16 <= (int64_t)persist_cu_count() * (L->shared_inter > L->inter ? 7 : 6);
+}
+
 int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_layer_t *LE, const void *x,
                  int64_t n_tokens, bool drop_skipped, const uint8_t *skip_mask,
                  dice_moe_lag_entry_t *put, const dice_moe_lag_entry_t *work_in,
@@ -569,6 +590,11 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
         s1.prob[0] = p1;
         s2.prob[0] = p2;
         s1.n_problems = s2.n_problems = 1;
+      } else if (shared_fc2_alone(L, n_tokens, max_rows)) {
+        f1.prob[1] = p1;
+        f1.n_problems = 2;
+        s2.prob[0] = p2;
+        s2.n_problems = 1;
       } else {
         f1.prob[1] = p1;
         f2.prob[1] = p2;
@@ -576,8 +602,8 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
       }
     }
     f2.split_ws = s2.split_ws = persist_split_allowed() ? w.split_ws : nullptr;
-    const bool shared_ok =
-        s1.n_problems == 0 || (persist_supported(s1, m1) && persist_supported(s2, kFc2));
+    const bool shared_ok = (s1.n_problems == 0 || persist_supported(s1, m1)) &&
+                           (s2.n_problems == 0 || persist_supported(s2, kFc2));
     // Where the kernel can address the activation rows through the permutation
     // itself, the gathered copy is skipped.
     PersistBatch f1g = f1;

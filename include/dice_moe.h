@@ -406,6 +406,8 @@ int dice_profile_read(float *ms_out, int n);
  * bands of b m-tiles; fc1_cfg = 50 has dice_moe_forward_modulated launch the
  * router on its own behind the prologue kernel instead of inside it (same
  * results); fc2_cfg = 50 has the layer calls multiply every fc2 tile whole;
+ * fc2_cfg = 51 / 52 have them launch the shared expert's fc2 on its own always /
+ * never (by default for small batches only);
  * any value from 20 on (21 does nothing else) keeps a dice_grouped_mlp stage
  * whose groups average at most 128 rows on the persistent kernels, which by
  * default leave it to the 64-row tiles of the permutation-addressed ones.  (By default a single-problem fc2 launch - fp8 routed weights, or no

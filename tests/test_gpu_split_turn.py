@@ -126,3 +126,40 @@ def test_cut_turn_is_deterministic_and_leaves_the_stage_calls_alone(dev):
     assert torch.equal(put, a)
     skip = blk.run(x, lib.MODE_SKIP, mask, cache, None)
     assert rel_l2(skip, a) < 4e-3   # (half the rows: another tile count, another cut)
+
+
+@pytest.mark.parametrize("variant,n_shared,N", [
+    ("swiglu", 2, 256),       # the reference's shared expert (k = 2304) beside routed tiles of 72 steps
+    ("swiglu", 2, 700),       # ragged groups, the largest batch that still takes the separate launch
+    ("gelu_tanh", 8, 512),    # config-literal shared expert: its fc2 tiles are twice as long as the routed ones
+    ("gelu_tanh", 8, 64),
+])
+def test_small_batch_shared_fc2_in_its_own_launch(dev, variant, n_shared, N):
+    """Small batches at DiT-XL width: the shared expert's fc2 leaves the routed
+    experts' launch so that both launches cut their tiles along k.  Against the
+    oracle, against the joint launch (tuning hook fc2 = 52) and against the
+    forced separate launch (51: must be what the default already does)."""
+    from dice_amd import lib
+    D, E = 1152, 8
+    p = O.make_block_params(D, E, 2, 4, n_shared, seed=41, dtype=torch.bfloat16, variant=variant)
+    if variant == "gelu_tanh":
+        _bias_params(p, 42)
+    x = torch.randn(1, N, D, generator=_gen(43)).bfloat16()
+    blk = block_from_params(p, D, variant, torch.bfloat16, dev)
+    xd = x.to(dev)
+    by_rule = blk(xd).cpu()
+    assert torch.equal(blk(xd).cpu(), by_rule), "two runs differ"
+    outs = {}
+    for hook in (51, 52):
+        lib.load().dice_set_gemm_config(0, hook)
+        try:
+            outs[hook] = blk(xd).cpu()
+        finally:
+            lib.load().dice_set_gemm_config(0, 0)
+    assert torch.equal(by_rule, outs[51]), "the default did not launch the shared expert's fc2 on its own"
+    assert not torch.equal(by_rule, outs[52])
+    want, _, _, logits = O.sparse_moe_block_forward(p, x)
+    ok = ~O.gate_tie_rows(logits, 2).view(-1)
+    check_rows(by_rule.view(-1, D)[ok], want.view(-1, D)[ok], BF16_TOL, "separate launches vs oracle")
+    check_rows(outs[52].view(-1, D)[ok], want.view(-1, D)[ok], BF16_TOL, "joint launch vs oracle")
+    check_rows(by_rule.view(-1, D), outs[52].view(-1, D), BF16_TOL / 2, "separate vs joint launch")
