@@ -332,17 +332,19 @@ def time_caller(cfg, blk, x, steps, warmup, hook=(0, 0)):
         ops.ln_modulate(xs, shift, scale)
 
     from dice_amd import lib
-    # "fused": prologue and router in one launch; "fused_router_own_launch": the same call with
-    # the router behind the prologue kernel as a launch of its own (tuning hook).  The legs take
-    # turns in short rounds, so that a drift of the board's clocks falls on all of them alike.
+    # "fused": the library's call (prologue and router in one launch); "fused_router_own_launch":
+    # the same call with the router as a launch of its own (tuning hook).  The legs take turns in
+    # short rounds and every round starts with another leg: the board's clocks drift with the
+    # load of the last few milliseconds (a leg that follows the light prologue-only leg ran
+    # 1-2 % slower than the same leg elsewhere in the round), so each leg gets each place once.
     legs = (("fused", fused), ("fused_router_own_launch", fused), ("eager_caller", eager),
             ("ln_modulate_kernel", prologue))
-    rounds = 5
+    rounds = len(legs)
     per_round = max(1, steps // rounds)
     total = {name: 0.0 for name, _ in legs}
     reps = {name: 20 if name == "ln_modulate_kernel" else 1 for name, _ in legs}   # (a 10 us kernel: more calls per wait)
     for r in range(rounds):
-        for name, fn in legs:
+        for name, fn in legs[r:] + legs[:r]:
             if name == "fused_router_own_launch":
                 lib.load().dice_set_gemm_config(50, hook[1])
             try:
