@@ -44,7 +44,41 @@ template <> struct Pack<f16_t> {
 
 constexpr int kMaxTopK = 8;
 
+// What one routing slot of a token contributes: its weight and where its row
+// comes from (the cache, the slot rows, or nowhere: a zero row).
 template <typename T>
+struct SlotSource {
+  float w;
+  const Pack<T> *row;   // nullptr: a zero row
+  bool put;             // the row also goes to cache_out
+};
+template <typename T>
+__device__ __forceinline__ SlotSource<T> slot_source(
+    int64_t s, int64_t chunk_of_token, int c, int vec_per_row, const Pack<T> *__restrict__ slot_out,
+    const int32_t *__restrict__ inv_perm, const float *__restrict__ topk_weight,
+    const uint8_t *__restrict__ skip_mask, const Pack<T> *__restrict__ cache_in, bool have_cache_out) {
+  SlotSource<T> r;
+  r.w = topk_weight[s];
+  const bool skipped = skip_mask && skip_mask[s];
+  if (skipped && cache_in) {
+    r.row = cache_in + chunk_of_token;
+    r.put = false;
+  } else {
+    // A slot the dispatch left out (masked, or an expert id outside the
+    // table: inv_perm = -1) contributes a zero row, as the zero-initialised
+    // buffer of the reference's _local_combine does (ep_fwd.py:350-354).
+    const int64_t src = inv_perm ? (int64_t)inv_perm[s] : s;
+    r.row = src >= 0 ? slot_out + src * vec_per_row + c : nullptr;
+    r.put = skipped && have_cache_out;
+  }
+  return r;
+}
+
+// K > 0: top_k known at compile time - the routing tables of all K slots are read
+// first, then all K rows are requested, then they are added in slot order (two
+// memory round trips per thread instead of two per slot; same arithmetic).
+// K = 0: any top_k, slot by slot.
+template <typename T, int K>
 __global__ __launch_bounds__(256) void combine_kernel(
     const Pack<T> *__restrict__ slot_out, const int32_t *__restrict__ inv_perm,
     const float *__restrict__ topk_weight, const Pack<T> *__restrict__ shared_out,
@@ -67,23 +101,34 @@ __global__ __launch_bounds__(256) void combine_kernel(
     res = resid[i];
     gt = gate[(t / tokens_per_sample) * vec_per_row + c];
   }
-  for (int j = 0; j < top_k; ++j) {
-    const int64_t s = t * top_k + j;
-    const float w = topk_weight[s];
-    const bool skipped = skip_mask && skip_mask[s];
-    Pack<T> row{};
-    if (skipped && cache_in) {
-      row = cache_in[t * vec_per_row + c];
-    } else {
-      // A slot the dispatch left out (masked, or an expert id outside the
-      // table: inv_perm = -1) contributes a zero row, as the zero-initialised
-      // buffer of the reference's _local_combine does (ep_fwd.py:350-354).
-      const int64_t src = inv_perm ? (int64_t)inv_perm[s] : s;
-      if (src >= 0) row = slot_out[src * vec_per_row + c];
-      if (skipped && cache_out) cache_out[t * vec_per_row + c] = row;
+  if constexpr (K > 0) {
+    SlotSource<T> src[K];
+#pragma unroll
+    for (int j = 0; j < K; ++j)
+      src[j] = slot_source<T>(t * K + j, i, c, vec_per_row, slot_out, inv_perm, topk_weight, skip_mask, cache_in,
+                              cache_out != nullptr);
+    Pack<T> row[K];
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      row[j] = Pack<T>{};
+      if (src[j].row) row[j] = *src[j].row;
     }
 #pragma unroll
-    for (int e = 0; e < Pack<T>::kN; ++e) acc[e] = fmaf(w, row.get(e), acc[e]);
+    for (int j = 0; j < K; ++j) {
+      if (src[j].put) cache_out[i] = row[j];
+#pragma unroll
+      for (int e = 0; e < Pack<T>::kN; ++e) acc[e] = fmaf(src[j].w, row[j].get(e), acc[e]);
+    }
+  } else {
+    for (int j = 0; j < top_k; ++j) {
+      const SlotSource<T> src = slot_source<T>(t * top_k + j, i, c, vec_per_row, slot_out, inv_perm, topk_weight,
+                                               skip_mask, cache_in, cache_out != nullptr);
+      Pack<T> row{};
+      if (src.row) row = *src.row;
+      if (src.put) cache_out[i] = row;
+#pragma unroll
+      for (int e = 0; e < Pack<T>::kN; ++e) acc[e] = fmaf(src.w, row.get(e), acc[e]);
+    }
   }
   if (shared_out) {
 #pragma unroll
@@ -107,10 +152,18 @@ int launch_combine(const void *slot_out, const int32_t *inv_perm, const float *w
   const int vec_per_row = hidden / Pack<T>::kN;
   const int64_t total = n_tokens * vec_per_row;
   const int64_t blocks = (total + 255) / 256;
-  hipLaunchKernelGGL(combine_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s,
-                     (const Pack<T> *)slot_out, inv_perm, w, (const Pack<T> *)shared_out, skip,
-                     (const Pack<T> *)cache_in, (Pack<T> *)cache_out, (Pack<T> *)y, n_tokens, top_k,
-                     vec_per_row, (const Pack<T> *)resid, (const Pack<T> *)gate, tokens_per_sample);
+#define DICE_COMBINE_LAUNCH(K)                                                                      \
+  hipLaunchKernelGGL((combine_kernel<T, K>), dim3((unsigned)blocks), dim3(256), 0, s,               \
+                     (const Pack<T> *)slot_out, inv_perm, w, (const Pack<T> *)shared_out, skip,     \
+                     (const Pack<T> *)cache_in, (Pack<T> *)cache_out, (Pack<T> *)y, n_tokens, top_k, \
+                     vec_per_row, (const Pack<T> *)resid, (const Pack<T> *)gate, tokens_per_sample)
+  switch (top_k) {
+    case 1: DICE_COMBINE_LAUNCH(1); break;
+    case 2: DICE_COMBINE_LAUNCH(2); break;
+    case 4: DICE_COMBINE_LAUNCH(4); break;
+    default: DICE_COMBINE_LAUNCH(0); break;
+  }
+#undef DICE_COMBINE_LAUNCH
   return launch_status("dice_combine");
 }
 
