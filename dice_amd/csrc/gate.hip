@@ -270,7 +270,10 @@ int launch_gate(const void *x, const void *w, const float *bias, int64_t n_token
 // left operand (rows past n_experts repeat the last one and are ignored), the
 // tokens the 32 columns of the right one, so lane l supplies 16 bytes of token
 // l % 32 per step - straight from memory, no LDS staging.  The hidden dimension
-// is cut into 2 x WPB contiguous segments, one per (wave, lane half): a wave
+// is cut into WPB contiguous segments, one per wave, of which the two lane
+// halves take alternate 16-byte chunks (a load then touches 32 bytes of 32
+// lines; with a segment per lane half it was 16 bytes of 64 lines and the
+// launch 0.8 us longer): a wave
 // requests its whole share (at most kRouterMaxSteps x 2 loads of 1 KB) before
 // the first product, the WPB partial logit tiles are added in wave order
 // through LDS, and the first wave finishes softmax and top-k with all of a
@@ -380,15 +383,18 @@ __device__ __forceinline__ void gate_topk_mfma_body(
   const int64_t tok = (int64_t)blockIdx.x * 32 + col;
   const int64_t tok_c = tok < n_tokens ? tok : n_tokens - 1;   // (columns past the end repeat the last token)
   const int steps = hidden / 16 / WPB;                         // per wave; at most kRouterMaxSteps
-  const int seg = (wave * 2 + half) * steps * 8;               // this lane's segment of the hidden dimension
+  // A wave's segment of the hidden dimension is 2 x steps chunks of 16 bytes; the
+  // two lane halves take alternate chunks, so that a load instruction touches 32
+  // bytes of each of its 32 rows' lines, not 16 bytes of 64 lines.
+  const int seg = (wave * 2 * steps + half) * 8;
   const T *xp = x + tok_c * hidden + seg;
   const T *wp = w + (size_t)(col < n_experts ? col : n_experts - 1) * hidden + seg;
   Vec8<T> xv[kRouterMaxSteps], wv[kRouterMaxSteps];
 #pragma unroll
   for (int s = 0; s < kRouterMaxSteps; ++s) {
     const int at = s < steps ? s : 0;   // (no branch around a load: steps past the end re-read the first chunk)
-    xv[s] = load8(xp + at * 8);
-    wv[s] = load8(wp + at * 8);
+    xv[s] = load8(xp + at * 16);
+    wv[s] = load8(wp + at * 16);
   }
   f32x16_t acc;
 #pragma unroll
@@ -496,12 +502,12 @@ __device__ __forceinline__ void ln_modulate_route_body(
   // covers both, in issue order).
   const int col = lane & 31, half = lane >> 5;
   const int steps = chunks_per_row / 2 / wpb;                   // per wave; at most kRouterMaxSteps
-  const int seg = (wave * 2 + half) * steps;                    // this lane's segment, in chunks
+  const int seg = wave * 2 * steps + half;                      // this lane's first chunk; it takes every other one
   Vec8<T> wv[kRouterMaxSteps];
   if (wave < wpb) {
     const T *wp = w + ((size_t)(col < n_experts ? col : n_experts - 1) * chunks_per_row + seg) * 8;
 #pragma unroll
-    for (int s = 0; s < kRouterMaxSteps; ++s) wv[s] = load8(wp + (s < steps ? s : 0) * 8);
+    for (int s = 0; s < kRouterMaxSteps; ++s) wv[s] = load8(wp + (s < steps ? s : 0) * 16);
   }
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -531,7 +537,7 @@ __device__ __forceinline__ void ln_modulate_route_body(
     for (int s0 = 0; s0 < kRouterMaxSteps; s0 += kReads) {
       Chunk<T> xb[kReads];
 #pragma unroll
-      for (int i = 0; i < kReads; ++i) xb[i] = xp[s0 + i < steps ? s0 + i : 0];
+      for (int i = 0; i < kReads; ++i) xb[i] = xp[s0 + i < steps ? 2 * (s0 + i) : 0];
 #pragma unroll
       for (int i = 0; i < kReads; ++i)
         if (s0 + i < steps) acc = RouterMfma<T>::mul(wv[s0 + i].v, xb[i].v, acc);
