@@ -333,34 +333,40 @@ def time_caller(cfg, blk, x, steps, warmup, hook=(0, 0)):
 
     from dice_amd import lib
     # "fused": the library's call (prologue and router in one launch); "fused_router_own_launch":
-    # the same call with the router as a launch of its own (tuning hook).  The legs take turns in
-    # short rounds and every round starts with another leg: the board's clocks drift with the
-    # load of the last few milliseconds (a leg that follows the light prologue-only leg ran
-    # 1-2 % slower than the same leg elsewhere in the round), so each leg gets each place once.
-    legs = (("fused", fused), ("fused_router_own_launch", fused), ("eager_caller", eager),
-            ("ln_modulate_kernel", prologue))
-    rounds = len(legs)
-    per_round = max(1, steps // rounds)
-    total = {name: 0.0 for name, _ in legs}
-    reps = {name: 20 if name == "ln_modulate_kernel" else 1 for name, _ in legs}   # (a 10 us kernel: more calls per wait)
-    for r in range(rounds):
-        for name, fn in legs[r:] + legs[:r]:
+    # the same call with the router as a launch of its own (tuning hook).  The board's clocks
+    # drift with the load of the last few milliseconds (a leg that follows a light one ran 1-2 %
+    # slower than the same leg elsewhere), so the three layer-call legs take turns in short
+    # rounds, one round per order of the three, and the prologue-only leg runs after them.
+    import itertools
+    legs = {"fused": fused, "fused_router_own_launch": fused, "eager_caller": eager}
+    orders = list(itertools.permutations(legs))
+    per_round = max(1, steps // len(orders))
+    total = {name: 0.0 for name in legs}
+    for r, order in enumerate(orders):
+        for name in order:
             if name == "fused_router_own_launch":
                 lib.load().dice_set_gemm_config(50, hook[1])
             try:
                 for _ in range(warmup if r == 0 else 2):
-                    fn()
-                n = per_round * reps[name]
+                    legs[name]()
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
-                for _ in range(n):
-                    fn()
+                for _ in range(per_round):
+                    legs[name]()
                 torch.cuda.synchronize()
                 total[name] += time.perf_counter() - t0
             finally:
                 if name == "fused_router_own_launch":
                     lib.load().dice_set_gemm_config(*hook)
-    res = {name: total[name] / (rounds * per_round * reps[name]) * 1e3 for name, _ in legs}
+    res = {name: total[name] / (len(orders) * per_round) * 1e3 for name in legs}
+    for _ in range(warmup):
+        prologue()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(20 * steps):   # (a 10 us kernel: many calls per wait)
+        prologue()
+    torch.cuda.synchronize()
+    res["ln_modulate_kernel"] = (time.perf_counter() - t0) / (20 * steps) * 1e3
     res["ln_modulate_frac_of_hbm_peak"] = (2 * cfg["tokens"] * D * x.element_size()
                                            / (res["ln_modulate_kernel"] * 1e-3) / 1e9 / PEAK_HBM_GBS)
     return res
