@@ -520,6 +520,78 @@ def measure(cfg_name, variant, activations, dev, steps, warmup, stages=True):
     return cfg, blk, x, res
 
 
+def ab_hooks(cfg_name, variant, activations, dev, hook_a, hook_b, lib_b=None, call="layer", groups=12, seg=20):
+    """Two settings of the tuning hook (or two builds of the library: `lib_b` names the other
+    .so) on the same block in one process, in an A B B A sequence of `groups` x 4 segments of
+    `seg` back-to-back calls each; us per call as mean and standard error over the segments.
+    The board's clocks drift with the load of the last milliseconds, so that timing one
+    setting after the other compares their places in the run rather than the settings."""
+    import ctypes
+    import statistics
+    from dice_amd import lib
+    from dice_amd.lib import CallerDesc, ptr, stream_ptr
+    cfg = dict(CONFIGS[cfg_name])
+    blk = make_block(cfg, variant, dev, activations=activations)
+    x = make_input(cfg, dev)
+    y = torch.empty_like(x)
+    blk.run(x, y=y)                                   # packs the weights, sizes the workspace
+    desc = blk._ensure(x)
+    ws = blk._workspace(desc, x.shape[0], x.device)
+    libs = [lib.load(), lib.load()]
+    if lib_b:
+        other = ctypes.CDLL(os.path.abspath(lib_b))
+        for name in ("dice_moe_forward", "dice_moe_forward_modulated", "dice_set_gemm_config"):
+            getattr(other, name).restype = getattr(libs[0], name).restype
+            getattr(other, name).argtypes = getattr(libs[0], name).argtypes
+        libs[1] = other
+    caller = None
+    if call == "modulated":
+        B = cfg["samples"]
+        g = torch.Generator().manual_seed(1)
+        keep = [(torch.randn(B, cfg["D"], generator=g) * 0.3).to(x.dtype).to(dev) for _ in range(3)]
+        caller = CallerDesc()
+        caller.shift, caller.scale, caller.gate = (ptr(t) for t in keep)
+        caller.tokens_per_sample = cfg["tokens"] // B
+        caller.ln_eps = 1e-6
+
+    def run(L, n):
+        for _ in range(n):
+            if caller is None:
+                rc = L.dice_moe_forward(ctypes.byref(desc), ptr(x), x.shape[0], 0, None, None, None, ptr(y), None,
+                                        None, ptr(ws), ws.numel(), stream_ptr())
+            else:
+                rc = L.dice_moe_forward_modulated(ctypes.byref(desc), ctypes.byref(caller), ptr(x), x.shape[0], 0,
+                                                  None, None, None, ptr(y), None, None, ptr(ws), ws.numel(),
+                                                  stream_ptr())
+            if rc:
+                raise RuntimeError(f"layer call failed with code {rc}")
+        torch.cuda.synchronize()
+
+    hooks = (hook_a, hook_b)
+    outs = []
+    for i in (0, 1):
+        libs[i].dice_set_gemm_config(*hooks[i])
+        run(libs[i], 10)
+        outs.append(y.clone())
+    times = ([], [])
+    try:
+        for i in [0, 1, 1, 0] * groups:
+            libs[i].dice_set_gemm_config(*hooks[i])
+            run(libs[i], 2)
+            t0 = time.perf_counter()
+            run(libs[i], seg)
+            times[i].append((time.perf_counter() - t0) / seg * 1e6)
+    finally:
+        for L in libs:
+            L.dice_set_gemm_config(0, 0)
+    mean = [statistics.mean(t) for t in times]
+    sem = [statistics.stdev(t) / len(t) ** 0.5 for t in times]
+    return {"workload": workload_text(cfg, variant, activations), "call": call, "segments": 2 * groups,
+            "calls_per_segment": seg, "a": {"hook": list(hook_a), "us_per_call": mean[0], "sem": sem[0]},
+            "b": {"hook": list(hook_b), "lib": lib_b, "us_per_call": mean[1], "sem": sem[1]},
+            "b_over_a": mean[1] / mean[0], "outputs_bit_identical": bool(torch.equal(outs[0], outs[1]))}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -543,6 +615,12 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a known-size kernel to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
+    ap.add_argument("--ab-hooks", nargs=2, metavar=("A", "B"),
+                    help="instead of the benchmark: compare two settings 'fc1,fc2' of the tuning hook on the chosen "
+                         "configuration in an A B B A sequence of short segments and print the result")
+    ap.add_argument("--ab-lib", default=None, help="with --ab-hooks: setting B runs on this other build of the library")
+    ap.add_argument("--ab-call", default="layer", choices=["layer", "modulated"],
+                    help="with --ab-hooks: dice_moe_forward or dice_moe_forward_modulated")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the layer holds every expert on one MI355X and uses no "
@@ -552,8 +630,13 @@ def main():
         print("bench.py needs an MI355X; there is no CPU path", file=sys.stderr)
         sys.exit(2)
     from dice_amd import lib
-    lib.load().dice_set_gemm_config(args.fc1_cfg, args.fc2_cfg)
     dev = torch.device("cuda:0")
+    if args.ab_hooks:
+        a, b = (tuple(int(v) for v in h.split(",")) for h in args.ab_hooks)
+        acts = args.activations if CONFIGS[args.config].get("fp8") else "bf16"
+        print(json.dumps({"ab": ab_hooks(args.config, args.variant, acts, dev, a, b, args.ab_lib, args.ab_call)}))
+        return
+    lib.load().dice_set_gemm_config(args.fc1_cfg, args.fc2_cfg)
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
