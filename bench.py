@@ -11,6 +11,13 @@ other configurations (c1 DiT-S fp32, c3 16384 tokens with a Zipf-loaded router,
 c4 the 50-step staleness loop, c5 DiT-G width with fp8 experts) run either as
 the main workload (--config) or, in the default run, as short extra legs under
 "configs".  Prints ONE JSON line.
+
+    python bench.py [--config ...] --ab-hooks A B [--ab-call modulated] [--ab-lib other.so]
+
+compares two settings "fc1,fc2" of the library's tuning hook (or two builds of the
+library) on one block in an A B B A sequence of short segments instead, and
+prints {"ab": ...}: us per call as mean and standard error, and whether the
+outputs are bit-identical.
 """
 import argparse
 import json
