@@ -582,21 +582,28 @@ def ab_hooks(cfg_name, variant, activations, dev, hook_a, hook_b, lib_b=None, ca
         outs.append(y.clone())
     times = ([], [])
     try:
-        for i in [0, 1, 1, 0] * groups:
+        # (the first two groups are not counted: the first segments after a pause run 2-6 % slow)
+        for g, i in enumerate([0, 1, 1, 0] * (groups + 2)):
             libs[i].dice_set_gemm_config(*hooks[i])
             run(libs[i], 2)
             t0 = time.perf_counter()
             run(libs[i], seg)
-            times[i].append((time.perf_counter() - t0) / seg * 1e6)
+            if g >= 8:
+                times[i].append((time.perf_counter() - t0) / seg * 1e6)
     finally:
         for L in libs:
             L.dice_set_gemm_config(0, 0)
     mean = [statistics.mean(t) for t in times]
     sem = [statistics.stdev(t) / len(t) ** 0.5 for t in times]
+    med = [statistics.median(t) for t in times]
     return {"workload": workload_text(cfg, variant, activations), "call": call, "segments": 2 * groups,
-            "calls_per_segment": seg, "a": {"hook": list(hook_a), "us_per_call": mean[0], "sem": sem[0]},
-            "b": {"hook": list(hook_b), "lib": lib_b, "us_per_call": mean[1], "sem": sem[1]},
-            "b_over_a": mean[1] / mean[0], "outputs_bit_identical": bool(torch.equal(outs[0], outs[1]))}
+            "calls_per_segment": seg,
+            "a": {"hook": list(hook_a), "us_per_call": mean[0], "sem": sem[0], "median": med[0],
+                  "segments_us": [round(t, 1) for t in times[0]]},
+            "b": {"hook": list(hook_b), "lib": lib_b, "us_per_call": mean[1], "sem": sem[1], "median": med[1],
+                  "segments_us": [round(t, 1) for t in times[1]]},
+            "b_over_a": mean[1] / mean[0], "b_over_a_medians": med[1] / med[0],
+            "outputs_bit_identical": bool(torch.equal(outs[0], outs[1]))}
 
 
 def main():

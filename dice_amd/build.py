@@ -60,21 +60,31 @@ def _compile(src: str, extra) -> str:
     return obj
 
 
-def build_library(verbose: bool = True, extra_flags=()) -> str:
+def build_library(verbose: bool = True, extra_flags=(), out: str = None) -> str:
+    """Compiles every source and links the library (to ``out`` instead of the
+    package's own path when given: a second build to compare with, e.g.
+    ``python -m dice_amd.build --out /tmp/other.so -DDICE_MFMA_ROWS_OUTERMOST=1``)."""
+    target = os.path.abspath(out) if out else LIB_PATH
     os.makedirs(BUILD_DIR, exist_ok=True)
     jobs = min(len(SOURCES), max(1, min(8, os.cpu_count() or 1)))
     with ThreadPoolExecutor(jobs) as pool:
         objs = list(pool.map(lambda s: _compile(s, list(extra_flags)), SOURCES))
-    tmp = LIB_PATH + ".tmp"
+    tmp = target + ".tmp"
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stderr}")
-    os.replace(tmp, LIB_PATH)
+    os.replace(tmp, target)
     if verbose:
-        print(f"built {LIB_PATH} ({os.path.getsize(LIB_PATH)} bytes)")
-    return LIB_PATH
+        print(f"built {target} ({os.path.getsize(target)} bytes)")
+    return target
 
 
 if __name__ == "__main__":
-    build_library(extra_flags=sys.argv[1:])
+    argv = sys.argv[1:]
+    out_path = None
+    if "--out" in argv:
+        at = argv.index("--out")
+        out_path = argv[at + 1]
+        del argv[at:at + 2]
+    build_library(extra_flags=argv, out=out_path)

@@ -268,8 +268,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N *kWave) void grouped_gemm_bf16_ker
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
           // weight block by weight block, the row blocks up and down in turn: one operand
-          // changes per product, the left one every fourth time (less switching in the
-          // matrix pipe: the persistent kernels measure 1-2 % for it at the power limit)
+          // changes per product, the left one every fourth time (same sums as any order)
           const int ii = (j & 1) ? TM - 1 - i : i;
           acc[ii][j] = DICE_MFMA_32X32X16(wf[j], af[ii], acc[ii][j], 0, 0, 0);
         }

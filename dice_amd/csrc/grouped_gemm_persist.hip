@@ -52,6 +52,9 @@
 // A third compilation (grouped_gemm_persist_f8.hip, DICE_PERSIST_F8) holds the
 // kernel whose activations are fp8 as well; it shares the tile order, the tile
 // table and the epilogue with the others and writes bf16.
+#ifndef DICE_MFMA_ROWS_OUTERMOST
+#define DICE_MFMA_ROWS_OUTERMOST 0
+#endif
 #ifndef DICE_PERSIST_F8
 #define DICE_PERSIST_F8 0
 #endif
@@ -1294,19 +1297,24 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   };
   // The 16 products of a 16-k block, weight block by weight block with the row
   // blocks up and down in turn: from one product to the next only one operand
-  // changes, the left one (the weights) every fourth time.  The launch is bound
-  // by the board's power limit, and the order in which the same products are
-  // issued moves it: row blocks outermost, weights changing every time, 616 us
-  // per layer call at 8192 x 1152; the same with the weight blocks down and up
-  // 607; this order 598-603 (same box, calls taking turns; same sums, bit for bit).
+  // changes, the left one (the weights) every fourth time.  Against the order of
+  // a plain `for i for j` loop (DICE_MFMA_ROWS_OUTERMOST = 1 builds it) the layer
+  // call's time is the same to 0.1 %, and the sums are the same bit for bit.
   auto mfma_block = [&](int buf) {
+    if constexpr (DICE_MFMA_ROWS_OUTERMOST) {
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int ii = (j & 1) ? TM - 1 - i : i;
-        acc[ii][j] = mfma_32x32x16(wf[buf][j], af[buf][ii], acc[ii][j]);
-      }
+        for (int j = 0; j < TN; ++j) acc[i][j] = mfma_32x32x16(wf[buf][j], af[buf][i], acc[i][j]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const int ii = (j & 1) ? TM - 1 - i : i;
+          acc[ii][j] = mfma_32x32x16(wf[buf][j], af[buf][ii], acc[ii][j]);
+        }
+    }
   };
 
   // ---- pipeline state ----
