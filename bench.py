@@ -527,7 +527,8 @@ def measure(cfg_name, variant, activations, dev, steps, warmup, stages=True):
     return cfg, blk, x, res
 
 
-def ab_hooks(cfg_name, variant, activations, dev, hook_a, hook_b, lib_b=None, call="layer", groups=12, seg=20):
+def ab_hooks(cfg_name, variant, activations, dev, hook_a, hook_b, lib_b=None, call="layer", tokens=None,
+             groups=12, seg=20):
     """Two settings of the tuning hook (or two builds of the library: `lib_b` names the other
     .so) on the same block in one process, in an A B B A sequence of `groups` x 4 segments of
     `seg` back-to-back calls each; us per call as mean and standard error over the segments.
@@ -538,6 +539,9 @@ def ab_hooks(cfg_name, variant, activations, dev, hook_a, hook_b, lib_b=None, ca
     from dice_amd import lib
     from dice_amd.lib import CallerDesc, ptr, stream_ptr
     cfg = dict(CONFIGS[cfg_name])
+    if tokens:                                        # another batch size of the same block
+        cfg["tokens"] = tokens
+        cfg["samples"] = max(1, tokens // 256)
     blk = make_block(cfg, variant, dev, activations=activations)
     x = make_input(cfg, dev)
     y = torch.empty_like(x)
@@ -633,6 +637,7 @@ def main():
                     help="instead of the benchmark: compare two settings 'fc1,fc2' of the tuning hook on the chosen "
                          "configuration in an A B B A sequence of short segments and print the result")
     ap.add_argument("--ab-lib", default=None, help="with --ab-hooks: setting B runs on this other build of the library")
+    ap.add_argument("--ab-tokens", type=int, default=None, help="with --ab-hooks: tokens per call (default: the configuration's)")
     ap.add_argument("--ab-call", default="layer", choices=["layer", "modulated"],
                     help="with --ab-hooks: dice_moe_forward or dice_moe_forward_modulated")
     args = ap.parse_args()
@@ -648,7 +653,7 @@ def main():
     if args.ab_hooks:
         a, b = (tuple(int(v) for v in h.split(",")) for h in args.ab_hooks)
         acts = args.activations if CONFIGS[args.config].get("fp8") else "bf16"
-        print(json.dumps({"ab": ab_hooks(args.config, args.variant, acts, dev, a, b, args.ab_lib, args.ab_call)}))
+        print(json.dumps({"ab": ab_hooks(args.config, args.variant, acts, dev, a, b, args.ab_lib, args.ab_call, args.ab_tokens)}))
         return
     lib.load().dice_set_gemm_config(args.fc1_cfg, args.fc2_cfg)
 
