@@ -2053,7 +2053,7 @@ int64_t model_makespan(const PersistProblem *prob, int n_problems, int bn_out, i
   }
   return makespan;
 }
-PersistPlan persist_plan(const PersistBatch &b, int bn_out, int grid) {
+PersistPlan persist_plan(const PersistBatch &b, int bn_out, int grid, bool fc2) {
   if (b.n_problems < 2) return PersistPlan{false, 1};
   struct Shape {
     int n_problems, bn_out, grid, rows[kMaxPersistProblems], experts[kMaxPersistProblems], n[kMaxPersistProblems],
@@ -2062,7 +2062,7 @@ PersistPlan persist_plan(const PersistBatch &b, int bn_out, int grid) {
   };
   Shape key{};
   key.n_problems = b.n_problems;
-  key.bn_out = bn_out;
+  key.bn_out = fc2 ? -bn_out : bn_out;   // (the stage is part of the shape)
   key.grid = grid;
   for (int p = 0; p < b.n_problems; ++p) {
     key.rows[p] = b.prob[p].max_rows;
@@ -2086,10 +2086,22 @@ PersistPlan persist_plan(const PersistBatch &b, int bn_out, int grid) {
   std::stable_sort(sorted, sorted + b.n_problems,
                    [](const PersistProblem &x, const PersistProblem &y) { return x.k > y.k; });
   const int wgs = grid / kNumXcd;
-  // in order of preference
-  const PersistPlan plans[4] = {{false, 0}, {true, 0}, {false, 1}, {true, 1}};
+  // In order of preference.  The model assumes evenly loaded groups, and real ones
+  // are ragged (at a multiple of 256 rows per group half of them spill into one
+  // more m-tile), so what it cannot tell apart is decided by measurement.  fc2 with
+  // the longer problem first and an eighth of every problem per XCD, against
+  // contiguous eighths of the cost, on the layer call at DiT-XL width: 4096
+  // tokens 386 -> 362 us, 3072 -1.5 %, 1024 / 8192 / 12288 / 16384 and the
+  // Zipf-loaded 16384 -0.2 ... -0.4 %, 1536 / 2048 the same, 6144 +0.7 %; the
+  // config-literal block -0.5 % at 8192 (the same split *without* the order is 6 %
+  // behind there).  fc1 keeps contiguous eighths of the cost (+0.7 % with the
+  // other split at 8192).
+  const PersistPlan fc1_plans[4] = {{false, 0}, {true, 0}, {false, 1}, {true, 1}};
+  const PersistPlan fc2_plans[4] = {{true, 1}, {false, 1}, {true, 0}, {false, 0}};
+  const PersistPlan *plans = fc2 ? fc2_plans : fc1_plans;
   PersistPlan pick = plans[0];
-  int64_t best = model_makespan(b.prob, b.n_problems, bn_out, wgs, 0);
+  int64_t best = model_makespan(plans[0].longest_first ? sorted : b.prob, b.n_problems, bn_out, wgs,
+                                plans[0].xcd_split);
   for (int i = 1; i < 4; ++i) {
     const int64_t m = model_makespan(plans[i].longest_first ? sorted : b.prob, b.n_problems, bn_out, wgs,
                                      plans[i].xcd_split);
@@ -2336,7 +2348,7 @@ int DICE_PERSIST_LAUNCH(const PersistBatch &b, int mode, hipStream_t s) {
   }
   PersistBatch launch = b;
   launch.band_tiles = persist_band_tiles(mode);
-  const PersistPlan plan = persist_plan(b, mode == kFc1Swiglu ? kPBN / 2 : narrow ? 192 : kPBN, grid);
+  const PersistPlan plan = persist_plan(b, mode == kFc1Swiglu ? kPBN / 2 : narrow ? 192 : kPBN, grid, mode == kFc2);
   if (plan.longest_first)
     std::stable_sort(launch.prob, launch.prob + launch.n_problems,
                      [](const PersistProblem &x, const PersistProblem &y) { return x.k > y.k; });
