@@ -2006,13 +2006,21 @@ bool split_may_apply(const PersistBatch &b, int grid, int bn_out) {
 struct PersistPlan {
   bool longest_first;   // sort the problems by k, longest first
   int xcd_split;
+  int64_t makespan;     // the model's longest workgroup under this arrangement, in 32-k steps
 };
 int64_t model_makespan(const PersistProblem *prob, int n_problems, int bn_out, int wgs, int split) {
   int64_t tiles[kMaxPersistProblems], steps[kMaxPersistProblems], base[kMaxPersistProblems], total_cost = 0, total = 0;
   for (int p = 0; p < n_problems; ++p) {
     const PersistProblem &pr = prob[p];
-    const int64_t per = pr.max_rows / pr.n_experts, rem = pr.max_rows % pr.n_experts;
-    const int64_t m_tiles = rem * ((per + 1 + kPBM - 1) / kPBM) + (pr.n_experts - rem) * ((per + kPBM - 1) / kPBM);
+    // Groups of a routed problem are ragged: every other one a little over, the
+    // rest as much under the mean (1.5 standard deviations of a uniform routing) -
+    // with the mean on a multiple of the tile height, as in a benchmark, half of
+    // the groups then spill into one more m-tile, as they do on the device.
+    const int64_t per = pr.max_rows / pr.n_experts;
+    const int64_t swing = pr.n_experts > 1 ? std::min<int64_t>(kPBM / 2, (int64_t)(1.5 * std::sqrt((double)per))) : 0;
+    int64_t m_tiles = 0;
+    for (int e = 0; e < pr.n_experts; ++e)
+      m_tiles += (std::max<int64_t>(0, per + ((e & 1) ? swing : -swing)) + kPBM - 1) / kPBM;
     tiles[p] = m_tiles * ((pr.n + bn_out - 1) / bn_out);
     steps[p] = pr.k / 32;
     base[p] = total;
@@ -2054,7 +2062,6 @@ int64_t model_makespan(const PersistProblem *prob, int n_problems, int bn_out, i
   return makespan;
 }
 PersistPlan persist_plan(const PersistBatch &b, int bn_out, int grid, bool fc2) {
-  if (b.n_problems < 2) return PersistPlan{false, 1};
   struct Shape {
     int n_problems, bn_out, grid, rows[kMaxPersistProblems], experts[kMaxPersistProblems], n[kMaxPersistProblems],
         k[kMaxPersistProblems];
@@ -2070,7 +2077,7 @@ PersistPlan persist_plan(const PersistBatch &b, int bn_out, int grid, bool fc2) 
     key.n[p] = b.prob[p].n;
     key.k[p] = b.prob[p].k;
   }
-  constexpr int kRemembered = 8;
+  constexpr int kRemembered = 16;
   static thread_local Shape seen[kRemembered];
   static thread_local int n_seen = 0, next = 0;
   auto same = [](const Shape &a, const Shape &c) {
@@ -2086,6 +2093,13 @@ PersistPlan persist_plan(const PersistBatch &b, int bn_out, int grid, bool fc2) 
   std::stable_sort(sorted, sorted + b.n_problems,
                    [](const PersistProblem &x, const PersistProblem &y) { return x.k > y.k; });
   const int wgs = grid / kNumXcd;
+  if (b.n_problems < 2) {
+    key.plan = PersistPlan{false, 1, model_makespan(b.prob, b.n_problems, bn_out, wgs, 1)};
+    seen[next] = key;
+    next = (next + 1) % kRemembered;
+    if (n_seen < kRemembered) ++n_seen;
+    return key.plan;
+  }
   // In order of preference.  The model assumes evenly loaded groups, and real ones
   // are ragged (at a multiple of 256 rows per group half of them spill into one
   // more m-tile), so what it cannot tell apart is decided by measurement.  fc2 with
@@ -2096,8 +2110,8 @@ PersistPlan persist_plan(const PersistBatch &b, int bn_out, int grid, bool fc2) 
   // config-literal block -0.5 % at 8192 (the same split *without* the order is 6 %
   // behind there).  fc1 keeps contiguous eighths of the cost (+0.7 % with the
   // other split at 8192).
-  const PersistPlan fc1_plans[4] = {{false, 0}, {true, 0}, {false, 1}, {true, 1}};
-  const PersistPlan fc2_plans[4] = {{true, 1}, {false, 1}, {true, 0}, {false, 0}};
+  const PersistPlan fc1_plans[4] = {{false, 0, 0}, {true, 0, 0}, {false, 1, 0}, {true, 1, 0}};
+  const PersistPlan fc2_plans[4] = {{true, 1, 0}, {false, 1, 0}, {true, 0, 0}, {false, 0, 0}};
   const PersistPlan *plans = fc2 ? fc2_plans : fc1_plans;
   PersistPlan pick = plans[0];
   int64_t best = model_makespan(plans[0].longest_first ? sorted : b.prob, b.n_problems, bn_out, wgs,
@@ -2110,6 +2124,7 @@ PersistPlan persist_plan(const PersistBatch &b, int bn_out, int grid, bool fc2) 
       pick = plans[i];
     }
   }
+  pick.makespan = best;
   key.plan = pick;
   seen[next] = key;
   next = (next + 1) % kRemembered;
@@ -2315,6 +2330,16 @@ int DICE_PERSIST_LAUNCH(const PersistBatch &b, int mode, hipStream_t s) {
   for (int i = 0; i < b.n_problems; ++i)
     narrow = narrow && b.prob[i].n % 192 == 0 && b.prob[i].n % 256 != 0;
   const bool w8 = b.prob[0].w_scale != nullptr;
+  if (narrow && waves == 4) {
+    // ... unless the 256-row tiles, padded columns and all, spare the launch a whole turn:
+    // the model's longest workgroup with them at most 0.7 of that with the narrow
+    // ones (a narrow tile's step takes about 0.8 of a wide one's).  DiT-XL width, 8
+    // experts: 4096 and 4608 tokens, 347 -> 339 us per layer call at 4096; at 8192
+    // the wide tiles cost +4.7 %.
+    const int64_t m192 = persist_plan(b, 192, grid, mode == kFc2).makespan;
+    const int64_t m256 = persist_plan(b, kPBN, grid, mode == kFc2).makespan;
+    if (m256 * 10 <= m192 * 7) narrow = false;
+  }
   if (waves == 4) {
     const bool refill = !persist_fits_table(b, mode);
     if (mode == kFc1Swiglu)
