@@ -2108,8 +2108,9 @@ PersistPlan persist_plan(const PersistBatch &b, int bn_out, int grid, bool fc2) 
   // tokens 386 -> 362 us, 3072 -1.5 %, 1024 / 8192 / 12288 / 16384 and the
   // Zipf-loaded 16384 -0.2 ... -0.4 %, 1536 / 2048 the same, 6144 +0.7 %; the
   // config-literal block -0.5 % at 8192 (the same split *without* the order is 6 %
-  // behind there).  fc1 keeps contiguous eighths of the cost (+0.7 % with the
-  // other split at 8192).
+  // behind there).  fc1 keeps contiguous eighths of the cost (the other split:
+  // +0.3 % at 8192 and at the Zipf-loaded 16384, -0.3 ... -1.1 % between 2048 and
+  // 6144 tokens).
   const PersistPlan fc1_plans[4] = {{false, 0, 0}, {true, 0, 0}, {false, 1, 0}, {true, 1, 0}};
   const PersistPlan fc2_plans[4] = {{true, 1, 0}, {false, 1, 0}, {true, 0, 0}, {false, 0, 0}};
   const PersistPlan *plans = fc2 ? fc2_plans : fc1_plans;
