@@ -51,12 +51,24 @@ def _hipcc() -> str:
     return exe
 
 
+# Translation units whose kernels keep their sums in accumulation registers that
+# the compiler does not know about: their device assembly is kept and checked
+# (check_acc_regs.py) before the library is linked.
+ACC_CHECKED = {"grouped_gemm_persist.hip", "grouped_gemm_persist_f16.hip"}
+
+
 def _compile(src: str, extra) -> str:
-    obj = os.path.join(BUILD_DIR, os.path.splitext(src)[0] + ".o")
+    stem = os.path.splitext(src)[0]
+    obj = os.path.join(BUILD_DIR, stem + ".o")
     cmd = [_hipcc(), *HIP_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+    if src in ACC_CHECKED:
+        cmd.insert(-4, "-save-temps=obj")
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stderr}")
+    if src in ACC_CHECKED:
+        from dice_amd.check_acc_regs import check
+        check(os.path.join(BUILD_DIR, stem + "-hip-amdgcn-amd-amdhsa-gfx950.s"))
     return obj
 
 

@@ -112,6 +112,79 @@ __device__ __forceinline__ void phase_barrier() {
 
 template <int V> using template_int = std::integral_constant<int, V>;
 
+// Calls f(template_int<I>{}) for I = 0 .. N - 1: a loop whose index is a
+// compile-time constant in the body (register numbers of inline assembly).
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (I < N) {
+    f(template_int<I>{});
+    static_for<N, I + 1>(f);
+  }
+}
+
+// ---- accumulators on fixed registers ----
+// The 64-k kernel keeps its sums in the accumulation registers a0 .. a255 by
+// NAME: block b (32 x 32 sums, 16 per lane) is a[16 b : 16 b + 15].  The
+// products, the reads and the writes of these registers are inline assembly,
+// so the compiler neither sees nor allocates them - it cannot move them between
+// register files where code paths join (a second copy of the k loop made it
+// spill hundreds of registers when the sums were its own values), and the order
+// of the statements in the source is the order of the instructions: a volatile
+// asm statement is a barrier to the scheduler for every memory instruction.
+// What the compiler does not know it cannot protect, so the hazards are covered
+// by hand: fixed_acc_settle() after the last product of a tile and before the
+// first read of a sum (the matrix pipe's result is not interlocked against
+// vector-ALU reads), and nothing else may touch an accumulation register - the
+// build checks the generated code for that (dice_amd/build.py).
+#if DICE_PERSIST_F16
+#define DICE_MFMA16 "v_mfma_f32_32x32x16_f16"
+#else
+#define DICE_MFMA16 "v_mfma_f32_32x32x16_bf16"
+#endif
+// sums of block BLK += w x a
+template <int BLK>
+__device__ __forceinline__ void mfma_fixed(const h16x8_t &w, const h16x8_t &a) {
+  asm volatile(DICE_MFMA16 " a[%2:%3], %0, %1, a[%2:%3]" ::"v"(w), "v"(a), "n"(BLK * 16), "n"(BLK * 16 + 15));
+}
+// sums of block BLK = w x a (the first product of a tile: nothing to clear)
+template <int BLK>
+__device__ __forceinline__ void mfma_fixed_first(const h16x8_t &w, const h16x8_t &a) {
+  asm volatile(DICE_MFMA16 " a[%2:%3], %0, %1, 0" ::"v"(w), "v"(a), "n"(BLK * 16), "n"(BLK * 16 + 15));
+}
+template <int REG>
+__device__ __forceinline__ float fixed_acc_get() {
+  float v;
+  asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(v) : "n"(REG));
+  return v;
+}
+template <int REG>
+__device__ __forceinline__ void fixed_acc_set(float v) {
+  asm volatile("v_accvgpr_write_b32 a[%1], %0" ::"v"(v), "n"(REG));
+}
+template <int BLK>
+__device__ __forceinline__ f32x16_t fixed_acc_block() {
+  f32x16_t t;
+  static_for<16>([&](auto q) { t[decltype(q)::value] = fixed_acc_get<BLK * 16 + decltype(q)::value>(); });
+  return t;
+}
+// Clears the top REGS accumulation registers, a[256 - REGS] .. a255.  A kernel
+// with fewer than sixteen blocks keeps them at the top: the registers below are
+// the ones the compiler takes first when it runs out of vector registers (it
+// parks values there instead of in scratch memory), and it must find them free.
+// The clobber names the highest register the kernel uses, which is how the
+// compiler learns how many to reserve for the wave.
+template <int REGS>
+__device__ __forceinline__ void fixed_acc_clear() {
+  static_assert(REGS == 256 || REGS == 192, "sixteen or twelve blocks");
+  if constexpr (REGS == 256)
+    asm volatile(".set dice_acc_r, 0\n.rept 256\nv_accvgpr_write_b32 a[dice_acc_r], 0\n.set dice_acc_r, dice_acc_r + 1\n.endr" ::: "a255");
+  else
+    asm volatile(".set dice_acc_r, 64\n.rept 192\nv_accvgpr_write_b32 a[dice_acc_r], 0\n.set dice_acc_r, dice_acc_r + 1\n.endr" ::: "a255");
+}
+// Wait states between a product and a vector-ALU access to its sums (19 for the
+// longest matrix instruction), and between a vector-ALU write and a product.
+__device__ __forceinline__ void fixed_acc_settle() { asm volatile("s_nop 7\ns_nop 7\ns_nop 7"); }
+
 template <int N> __device__ __forceinline__ void pwait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
@@ -612,8 +685,11 @@ __device__ __forceinline__ f32x16_t acc_block(const f32x16_t &a) {
 // BIAS_LDS: the bias of the tile's columns sits in LDS (bias_lds[c - n0]) and is
 // read four values at a time where it is added, instead of being held in
 // registers for the whole epilogue (HAS_BIAS) or folded into the accumulators.
+// ACC_BLOCK0 >= 0: the sums are not in `acc` but in the accumulation registers by
+// name (block (i, j) = a[16 (ACC_BLOCK0 + i TN + j) ..], see mfma_fixed); the
+// caller has let the last products settle.
 template <int MODE, bool HAS_BIAS, int WAVES, int TM, int TN, bool HAS_SCALE = false, int RESERVE = 0,
-          bool HAS_ROW = false, bool BIAS_LDS = false>
+          bool HAS_ROW = false, bool BIAS_LDS = false, int ACC_BLOCK0 = -1>
 __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM][TN], unsigned char *stage,
                                               int wave_row0, int wave_col0, int lane,
                                               const float *scale_lds = nullptr,
@@ -689,16 +765,21 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
     }                                                                                                      \
     wave_lds_sync(); /* the next band overwrites the staging rows */                                       \
   } while (0)
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
+  static_for<TM>([&](auto i_c) {
+    constexpr int i = decltype(i_c)::value;
     float row_scale = 1.0f;
     if (HAS_ROW) row_scale = rowscale_lds[wave_row0 + i * 32 + frag_row];
     if constexpr (BAND == 32) {
-#pragma unroll
-      for (int j = 0; j < OUT_BLOCKS; ++j) {
-        const f32x16_t blk = acc_block<WAVES == 4>(acc[i][j]);
-        f32x16_t up;
-        if (SWIGLU) up = acc_block<WAVES == 4>(acc[i][j + OUT_BLOCKS]);
+      static_for<OUT_BLOCKS>([&](auto j_c) {
+        constexpr int j = decltype(j_c)::value;
+        f32x16_t blk, up;
+        if constexpr (ACC_BLOCK0 >= 0) {
+          blk = fixed_acc_block<ACC_BLOCK0 + i * TN + j>();
+          if constexpr (SWIGLU) up = fixed_acc_block<ACC_BLOCK0 + i * TN + j + OUT_BLOCKS>();
+        } else {
+          blk = acc_block<WAVES == 4>(acc[i][j]);
+          if constexpr (SWIGLU) up = acc_block<WAVES == 4>(acc[i][j + OUT_BLOCKS]);
+        }
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int col = j * 32 + frag_half * 4 + q * 8;
@@ -712,18 +793,23 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
           }
           *reinterpret_cast<u32x2_any_t *>(stage + frag_row * PITCH + col * 2) = __builtin_bit_cast(u32x2_t, o);
         }
-      }
+      });
       DICE_EPI_STORE_BAND(i);
     } else {
       // The staging rows hold 16 rows at a time.  The activation of the whole
       // 32-row block is worked out once, with every lane at work (per band only
       // half the lanes own rows), and kept packed while its two bands go out.
       h16x4_t packed[OUT_BLOCKS][4];
-#pragma unroll
-      for (int j = 0; j < OUT_BLOCKS; ++j) {
-        const f32x16_t blk = acc_block<WAVES == 4>(acc[i][j]);
-        f32x16_t up;
-        if (SWIGLU) up = acc_block<WAVES == 4>(acc[i][j + OUT_BLOCKS]);
+      static_for<OUT_BLOCKS>([&](auto j_c) {
+        constexpr int j = decltype(j_c)::value;
+        f32x16_t blk, up;
+        if constexpr (ACC_BLOCK0 >= 0) {
+          blk = fixed_acc_block<ACC_BLOCK0 + i * TN + j>();
+          if constexpr (SWIGLU) up = fixed_acc_block<ACC_BLOCK0 + i * TN + j + OUT_BLOCKS>();
+        } else {
+          blk = acc_block<WAVES == 4>(acc[i][j]);
+          if constexpr (SWIGLU) up = acc_block<WAVES == 4>(acc[i][j + OUT_BLOCKS]);
+        }
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           DICE_EPI_SCALES(j, q)
@@ -734,7 +820,7 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
             packed[j][q][r] = (h16_t)v;
           }
         }
-      }
+      });
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         if ((frag_row >> 4) == half) {
@@ -754,7 +840,7 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
     // over this one's stores only lengthens live ranges (register spills cost far
     // more here than the lost overlap).
     __builtin_amdgcn_sched_barrier(0);
-  }
+  });
 #undef DICE_EPI_VALUE
 #undef DICE_EPI_SCALES
 #undef DICE_EPI_STORE_BAND
@@ -1032,6 +1118,27 @@ __device__ __forceinline__ int qring_off(int row, int chunk) {
   return row * 128 + ((chunk ^ qswizzle(row)) << 4);
 }
 
+// A step's loads in four quarters: the two halves of the activation rows, then
+// the two halves of the weight rows.  quarter_first(q) .. quarter_first(q + 1)
+// are quarter q's indices into the register stage.
+constexpr int quarter_first(int copies_a, int copies_b, int q) {
+  return q <= 2 ? q * (copies_a / 2) : q == 3 ? copies_a + (copies_b + 1) / 2 : copies_a + copies_b;
+}
+// Where side work goes in a block of `mf` products: item `idx` of `n` follows
+// the product with this index (`phase` quarters of an interval in: fragment
+// reads 0, LDS writes 1, global loads 3, so that the three kinds alternate).
+// For 16 products: reads behind every even one, a write behind products 1, 5, 9,
+// 13 and a load behind 3, 7, 11, 15: one instruction per gap.  The LDS takes 16 cycles per 16-byte-per-lane
+// write against 4 per read, so the writes of the four waves are spread over the
+// whole block rather than bunched.
+constexpr int side_slot(int idx, int n, int mf, int phase) { return ((4 * idx + phase) * mf) / (4 * n); }
+// The item that follows product `i` (at most one of each kind: n <= mf), or -1.
+constexpr int side_item(int i, int n, int mf, int phase) {
+  for (int idx = 0; idx < n; ++idx)
+    if (side_slot(idx, n, mf, phase) == i) return idx;
+  return -1;
+}
+
 // Instruction order of one block of MF MFMAs: RD fragment reads, 4 LDS writes
 // and 4 global loads spread evenly behind the MFMAs (reads from the first MFMA
 // on, writes and loads offset against each other).  The LDS takes 16 cycles per
@@ -1245,33 +1352,40 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
     asm volatile("" : "+v"(rd_a[kk]), "+v"(rd_b[kk]));
   }
   h16x8_t wf[2][TN], af[2][TM];
-  auto read_frags = [&](auto slot_c, auto kk_c, int buf) {
-    constexpr int SLOT = decltype(slot_c)::value, KK = decltype(kk_c)::value;
+  // Fragment R of 16-k block KK of slot SLOT into buffer BUF, in the order in which
+  // the block's products first need them (mfma_at): weight block 0, the row
+  // blocks, then the other weight blocks.
+  auto read_frag = [&](auto slot_c, auto kk_c, auto buf_c, auto r_c) {
+    constexpr int SLOT = decltype(slot_c)::value, KK = decltype(kk_c)::value, BUF = decltype(buf_c)::value;
+    constexpr int R = decltype(r_c)::value;
     const unsigned char *base = SLOT == 0 ? lds_slot0 : lds_slot1;
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      constexpr int HALF = TN / 2;
-      const int jrow = (SWIGLU && j >= HALF) ? BN / 2 + (j - HALF) * 32 : j * 32;
-      wf[buf][j] = *reinterpret_cast<const h16x8_t *>(base + rd_b[KK] + jrow * 128);
+    if constexpr (R == 0 || R > TM) {
+      constexpr int J = R == 0 ? 0 : R - TM, HALF = TN / 2;
+      constexpr int jrow = (SWIGLU && J >= HALF) ? BN / 2 + (J - HALF) * 32 : J * 32;
+      wf[BUF][J] = *reinterpret_cast<const h16x8_t *>(base + rd_b[KK] + jrow * 128);
+    } else {
+      af[BUF][R - 1] = *reinterpret_cast<const h16x8_t *>(base + rd_a[KK] + (R - 1) * 32 * 128);
     }
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-      af[buf][i] = *reinterpret_cast<const h16x8_t *>(base + rd_a[KK] + i * 32 * 128);
+  };
+  auto read_frags = [&](auto slot_c, auto kk_c, auto buf_c) {
+    static_for<TM + TN>([&](auto r_c) { read_frag(slot_c, kk_c, buf_c, r_c); });
   };
 
   const int wave_col0 = SWIGLU ? wn * (WTN / 2) : wn * WTN;
-  f32x16_t acc[TM][TN];
+  // The sums live in the accumulation registers by name: block (i, j) is
+  // a[16 (kAccBlock0 + i TN + j) ..], the TM x TN blocks at the top of the
+  // register file (see mfma_fixed, fixed_acc_clear).
+  constexpr int kAccBlock0 = 16 - TM * TN;
   // (256-wide biased tiles) the accumulators start from the bias of their columns:
   // every 32-row block of a column block gets the same 16 values per lane.
   auto init_acc = [&](const Tile &t, int buf, int sbuf) {
     if constexpr (kBiasInAcc) {
       if (uni((int)(t.bias != nullptr))) {
         const float *src = lds_bias + buf * kBiasBufFloats + wave_col0 + frag_half * 4;
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          f32x16_t b;
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
+        static_for<TN>([&](auto j_c) {
+          constexpr int j = decltype(j_c)::value;
+          static_for<4>([&](auto q_c) {
+            constexpr int q = decltype(q_c)::value;
             f32x4_t v = *reinterpret_cast<const f32x4_t *>(src + j * 32 + q * 8);
             if constexpr (W8) {  // the epilogue multiplies the sums by the scale
               const f32x4_t sc = *reinterpret_cast<const f32x4_t *>(
@@ -1279,42 +1393,28 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
 #pragma unroll
               for (int r = 0; r < 4; ++r) v[r] = v[r] / sc[r];
             }
-#pragma unroll
-            for (int r = 0; r < 4; ++r) b[q * 4 + r] = v[r];
-          }
-#pragma unroll
-          for (int i = 0; i < TM; ++i) acc[i][j] = b;
-        }
+            static_for<4>([&](auto r_c) {
+              constexpr int r = decltype(r_c)::value;
+              static_for<TM>([&](auto i_c) {
+                fixed_acc_set<(kAccBlock0 + decltype(i_c)::value * TN + j) * 16 + q * 4 + r>(v[r]);
+              });
+            });
+          });
+        });
+        fixed_acc_settle();
         return;
       }
     }
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+    fixed_acc_clear<TM * TN * 16>();
+    fixed_acc_settle();
   };
-  // The 16 products of a 16-k block, weight block by weight block with the row
-  // blocks up and down in turn: from one product to the next only one operand
-  // changes, the left one (the weights) every fourth time.  Against the order of
-  // a plain `for i for j` loop (DICE_MFMA_ROWS_OUTERMOST = 1 builds it) the layer
-  // call's time is the same to 0.1 %, and the sums are the same bit for bit.
-  auto mfma_block = [&](int buf) {
-    if constexpr (DICE_MFMA_ROWS_OUTERMOST) {
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = mfma_32x32x16(wf[buf][j], af[buf][i], acc[i][j]);
-    } else {
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          const int ii = (j & 1) ? TM - 1 - i : i;
-          acc[ii][j] = mfma_32x32x16(wf[buf][j], af[buf][ii], acc[ii][j]);
-        }
-    }
+  // Product I of a 16-k block: weight block by weight block with the row blocks
+  // up and down in turn, so that from one product to the next only one operand
+  // changes, the left one (the weights) every TM-th time.
+  auto mfma_at = [&](auto buf_c, auto i_c) {
+    constexpr int BUF = decltype(buf_c)::value, I = decltype(i_c)::value;
+    constexpr int j = I / TM, i = (j & 1) ? TM - 1 - I % TM : I % TM;
+    mfma_fixed<kAccBlock0 + i * TN + j>(wf[BUF][j], af[BUF][i]);
   };
 
   // ---- pipeline state ----
@@ -1355,56 +1455,61 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   // A step's loads in four quarters: the two halves of the activation rows, then
   // the two halves of the weight rows.  first(q) .. first(q + 1) are quarter q's
   // indices into the register stage.
-  auto quarter_first = [](int q) { return q <= 2 ? q * (kCopiesA / 2) : kCopiesA + (kCopiesB + 1) / 2; };
-  // Quarter q of the step the load side stands at, into register stage P.
-  auto load_quarter = [&](auto stage_c, auto q_c) {
-    constexpr int P = decltype(stage_c)::value, Q = decltype(q_c)::value;
-#pragma unroll
-    for (int l = quarter_first(Q); l < (Q == 3 ? kQCopies : quarter_first(Q + 1)); ++l) {
-      if (l < kCopiesA) {
-        const int i = l;
-        // (uni() costs nothing while the description sits in scalar registers and
-        // avoids a loop over lanes around the load if the compiler moved it out)
-        const __amdgpu_buffer_rsrc_t rs =
-            __builtin_amdgcn_make_buffer_rsrc((void *)uni(ld.a), 0, uni(ld.a_bytes), kRsrcFlags);
-        const uint32_t voff = GATHER ? ld_voff_rows[i] : ld_voff_a + (uint32_t)(32 * i) * uni(ld.a_pitch);
-        stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, uni(ld_kt * 128), 0);
-      } else {
-        const int i = l - kCopiesA;
-        constexpr int kStride = kRowsPerCopyB * kQWaves;  // weight rows between a lane's consecutive loads
-        const bool up_half = SWIGLU && kStride * i >= BN / 2;  // a wave's rows of one load never cross the halves
-        const int row = up_half ? kStride * i - BN / 2 : kStride * i;
-        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)uni(up_half ? ld.b1 : ld.b0), 0, uni(ld.b_bytes), kRsrcFlags);
-        stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(
-            rs, ld_voff_b + (uint32_t)row * uni(ld.b_pitch), uni(ld_kt * (W8 ? 64 : 128)), 0);
-      }
+  // Load l of the step the load side stands at, into register stage P.
+  auto load_one = [&](auto stage_c, auto l_c) {
+    constexpr int P = decltype(stage_c)::value, l = decltype(l_c)::value;
+    if constexpr (l < kCopiesA) {
+      // (uni() costs nothing while the description sits in scalar registers and
+      // avoids a loop over lanes around the load if the compiler moved it out)
+      const __amdgpu_buffer_rsrc_t rs =
+          __builtin_amdgcn_make_buffer_rsrc((void *)uni(ld.a), 0, uni(ld.a_bytes), kRsrcFlags);
+      uint32_t voff;
+      if constexpr (GATHER) voff = ld_voff_rows[l];
+      else voff = ld_voff_a + (uint32_t)(32 * l) * uni(ld.a_pitch);
+      stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, uni(ld_kt * 128), 0);
+    } else {
+      constexpr int i = l - kCopiesA;
+      constexpr int kStride = kRowsPerCopyB * kQWaves;  // weight rows between a lane's consecutive loads
+      constexpr bool up_half = SWIGLU && kStride * i >= BN / 2;  // a wave's rows of one load never cross the halves
+      constexpr int row = up_half ? kStride * i - BN / 2 : kStride * i;
+      const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+          (void *)uni(up_half ? ld.b1 : ld.b0), 0, uni(ld.b_bytes), kRsrcFlags);
+      stage_regs[P][l] = __builtin_amdgcn_raw_buffer_load_b128(
+          rs, ld_voff_b + (uint32_t)row * uni(ld.b_pitch), uni(ld_kt * (W8 ? 64 : 128)), 0);
     }
   };
-  // Quarter q of register stage P into LDS slot P.
-  auto write_quarter = [&](auto stage_c, auto q_c) {
-    constexpr int P = decltype(stage_c)::value, Q = decltype(q_c)::value;
+  // Load l of register stage P into LDS slot P.
+  auto write_one = [&](auto stage_c, auto l_c) {
+    constexpr int P = decltype(stage_c)::value, l = decltype(l_c)::value;
+    constexpr int i = l < kCopiesA ? l : l - kCopiesA;
+    if constexpr (W8 && l >= kCopiesA) {
+      unsigned char *row = (P == 0 ? lds_slot0 : lds_slot1) + kPBM * 128 + i * (kRowsPerCopyB * kQWaves) * 128;
+      const u32x4_t src = stage_regs[P][l];
+      u32x4_t lo, hi;
 #pragma unroll
-    for (int l = quarter_first(Q); l < (Q == 3 ? kQCopies : quarter_first(Q + 1)); ++l) {
-      const int i = l < kCopiesA ? l : l - kCopiesA;
-      if (W8 && l >= kCopiesA) {
-        unsigned char *row = (P == 0 ? lds_slot0 : lds_slot1) + kPBM * 128 + i * (kRowsPerCopyB * kQWaves) * 128;
-        const u32x4_t src = stage_regs[P][l];
-        u32x4_t lo, hi;
-#pragma unroll
-        for (int q = 0; q < 2; ++q) {
-          lo[2 * q] = widen_fp8_pair(src[q], false);
-          lo[2 * q + 1] = widen_fp8_pair(src[q], true);
-          hi[2 * q] = widen_fp8_pair(src[q + 2], false);
-          hi[2 * q + 1] = widen_fp8_pair(src[q + 2], true);
-        }
-        *reinterpret_cast<u32x4_any_t *>(row + wr_off_b8) = lo;
-        *reinterpret_cast<u32x4_any_t *>(row + wr_off_b8_hi) = hi;
-      } else {
-        unsigned char *dst = (P == 0 ? lds_slot0 : lds_slot1) + (l < kCopiesA ? 0 : kPBM * 128) + i * 32 * 128 + wr_off;
-        *reinterpret_cast<u32x4_any_t *>(dst) = stage_regs[P][l];
+      for (int q = 0; q < 2; ++q) {
+        lo[2 * q] = widen_fp8_pair(src[q], false);
+        lo[2 * q + 1] = widen_fp8_pair(src[q], true);
+        hi[2 * q] = widen_fp8_pair(src[q + 2], false);
+        hi[2 * q + 1] = widen_fp8_pair(src[q + 2], true);
       }
+      *reinterpret_cast<u32x4_any_t *>(row + wr_off_b8) = lo;
+      *reinterpret_cast<u32x4_any_t *>(row + wr_off_b8_hi) = hi;
+    } else {
+      unsigned char *dst = (P == 0 ? lds_slot0 : lds_slot1) + (l < kCopiesA ? 0 : kPBM * 128) + i * 32 * 128 + wr_off;
+      *reinterpret_cast<u32x4_any_t *>(dst) = stage_regs[P][l];
     }
+  };
+  // Quarter Q of a step covers loads [quarter_first(Q), quarter_first(Q + 1)).
+  auto load_quarter = [&](auto stage_c, auto q_c) {
+    constexpr int Q = decltype(q_c)::value;
+    constexpr int F = quarter_first(kCopiesA, kCopiesB, Q), N = quarter_first(kCopiesA, kCopiesB, Q + 1) - F;
+    static_for<N>([&](auto n_c) { load_one(stage_c, template_int<F + decltype(n_c)::value>{}); });
+  };
+  auto write_quarter = [&](auto stage_c, auto q_c) {
+    constexpr int Q = decltype(q_c)::value;
+    constexpr int F = quarter_first(kCopiesA, kCopiesB, Q), N = quarter_first(kCopiesA, kCopiesB, Q + 1) - F;
+    static_for<N>([&](auto n_c) { write_one(stage_c, template_int<F + decltype(n_c)::value>{}); });
   };
   auto load_step = [&](auto stage_c) {
     load_quarter(stage_c, c0); load_quarter(stage_c, c1); load_quarter(stage_c, c2); load_quarter(stage_c, c3);
@@ -1426,52 +1531,61 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   init_acc(cp, 0, 0);
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   phase_barrier();
-  read_frags(c0, c0, 0);
+  read_frags(c0, c0, c0);
   __builtin_amdgcn_sched_barrier(0);
 
   unsigned char *const stage_rows = lds_stage + wave * Epi::WAVE_BYTES;
+  f32x16_t no_acc[TM][TN];  // (the epilogue takes the sums from the accumulation registers; never read)
+
+  // One block of a step: the TM x TN products of fragment buffer MB and, threaded
+  // between them (side_slot), the reads of the fragments of 16-k block RK of slot
+  // RS into the other buffer, quarter Q of register stage WP into LDS slot WP, and
+  // quarter Q of the step the load side stands at into that stage.  The products
+  // are volatile asm statements, which no memory instruction is moved across: the
+  // order below is the order of the instructions.
+  auto block = [&](auto mb_c, auto rs_c, auto rk_c, auto wp_c, auto q_c) {
+    constexpr int MB = decltype(mb_c)::value, Q = decltype(q_c)::value;
+    constexpr int MF = TM * TN, RD = TM + TN;
+    constexpr int F = quarter_first(kCopiesA, kCopiesB, Q), N = quarter_first(kCopiesA, kCopiesB, Q + 1) - F;
+    const template_int<MB ^ 1> rb_c;
+    static_assert(RD <= MF && N <= MF, "at most one item of a kind per product");
+    static_for<MF>([&](auto i_c) {
+      constexpr int I = decltype(i_c)::value;
+      mfma_at(mb_c, i_c);
+      constexpr int R = side_item(I, RD, MF, 0), W = side_item(I, N, MF, 1), L = side_item(I, N, MF, 3);
+      // (where two share a gap the read goes first: a read queued behind a write
+      // waits for the write's 16 cycles)
+      if constexpr (R >= 0) read_frag(rs_c, rk_c, rb_c, template_int<R>{});
+      if constexpr (R >= 0 && (W >= 0 || L >= 0)) __builtin_amdgcn_sched_barrier(0);
+      if constexpr (W >= 0) write_one(wp_c, template_int<F + W>{});
+      if constexpr (W >= 0 && L >= 0) __builtin_amdgcn_sched_barrier(0);
+      if constexpr (L >= 0) load_one(wp_c, template_int<F + L>{});
+    });
+    __builtin_amdgcn_sched_barrier(0);
+  };
 
   while (true) {  // one tile per iteration
     // Every tile has an even number of steps, so a tile always starts in slot 0.
     auto step = [&](auto slot_c) {
       constexpr int S = decltype(slot_c)::value;
       const template_int<S ^ 1> other_c;
-      read_frags(slot_c, c1, 1);
-      write_quarter(other_c, c1);
-      load_quarter(other_c, c1);
-      mfma_block(0);
-      qsched_block<0, TM * TN, TM + TN>();
-      __builtin_amdgcn_sched_barrier(0);
-      read_frags(slot_c, c2, 0);
-      write_quarter(other_c, c2);
-      load_quarter(other_c, c2);
-      mfma_block(1);
-      qsched_block<0, TM * TN, TM + TN>();
-      __builtin_amdgcn_sched_barrier(0);
-      read_frags(slot_c, c3, 1);
-      write_quarter(other_c, c3);
-      load_quarter(other_c, c3);
-      mfma_block(0);
-      qsched_block<0, TM * TN, TM + TN>();
-      __builtin_amdgcn_sched_barrier(0);
+      block(c0, slot_c, c1, other_c, c1);
+      block(c1, slot_c, c2, other_c, c2);
+      block(c0, slot_c, c3, other_c, c3);
       advance_copy();
       // This wave has read slot S for the last time and has finished writing the
       // other slot; after the barrier both hold for every wave.
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       phase_barrier();
-      read_frags(other_c, c0, 0);
-      write_quarter(slot_c, c0);
-      load_quarter(slot_c, c0);
-      mfma_block(1);
-      qsched_block<0, TM * TN, TM + TN>();
-      __builtin_amdgcn_sched_barrier(0);
+      block(c1, other_c, c0, slot_c, c0);
     };
     for (int s = 0; s < cp.steps; s += 2) {
       step(c0);
       step(c1);
     }
-    tile_epilogue<MODE, HAS_BIAS && !kBiasInAcc, kQWaves, TM, TN, W8, W8 ? kEpiReserve : 0>(
-        cp, acc, stage_rows, wm * WTM, wave_col0, lane, lds_scale + scale_buf * kScaleBufFloats);
+    fixed_acc_settle();
+    tile_epilogue<MODE, HAS_BIAS && !kBiasInAcc, kQWaves, TM, TN, W8, W8 ? kEpiReserve : 0, false, false, kAccBlock0>(
+        cp, no_acc, stage_rows, wm * WTM, wave_col0, lane, lds_scale + scale_buf * kScaleBufFloats);
     // The load side is within the next tile here (every tile has at least
     // kQMinSteps steps).
     cp = ld;
@@ -1492,7 +1606,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
     init_acc(cp, bias_buf, scale_buf);
     // The last block above already fetched these fragments; reading them again
     // here keeps 32 registers free during the epilogue.
-    read_frags(c0, c0, 0);
+    read_frags(c0, c0, c0);
   }
 }
 
