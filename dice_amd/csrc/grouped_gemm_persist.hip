@@ -146,10 +146,12 @@ template <int BLK>
 __device__ __forceinline__ void mfma_fixed(const h16x8_t &w, const h16x8_t &a) {
   asm volatile(DICE_MFMA16 " a[%2:%3], %0, %1, a[%2:%3]" ::"v"(w), "v"(a), "n"(BLK * 16), "n"(BLK * 16 + 15));
 }
-// sums of block BLK = w x a (the first product of a tile: nothing to clear)
+// sums of block BLK = z x z + 0 for a fragment z of zeros: clears the block on the
+// matrix pipe, which is idle during an epilogue, instead of with sixteen
+// vector-ALU writes that the epilogue's arithmetic would have to wait for
 template <int BLK>
-__device__ __forceinline__ void mfma_fixed_first(const h16x8_t &w, const h16x8_t &a) {
-  asm volatile(DICE_MFMA16 " a[%2:%3], %0, %1, 0" ::"v"(w), "v"(a), "n"(BLK * 16), "n"(BLK * 16 + 15));
+__device__ __forceinline__ void mfma_fixed_clear(const h16x8_t &z) {
+  asm volatile(DICE_MFMA16 " a[%1:%2], %0, %0, 0" ::"v"(z), "n"(BLK * 16), "n"(BLK * 16 + 15));
 }
 template <int REG>
 __device__ __forceinline__ float fixed_acc_get() {
@@ -687,9 +689,11 @@ __device__ __forceinline__ f32x16_t acc_block(const f32x16_t &a) {
 // registers for the whole epilogue (HAS_BIAS) or folded into the accumulators.
 // ACC_BLOCK0 >= 0: the sums are not in `acc` but in the accumulation registers by
 // name (block (i, j) = a[16 (ACC_BLOCK0 + i TN + j) ..], see mfma_fixed); the
-// caller has let the last products settle.
+// caller has let the last products settle.  CLEAR_ACC: every block is cleared as
+// soon as it has been read (mfma_fixed_clear), so the next tile's products can
+// add to it at once.
 template <int MODE, bool HAS_BIAS, int WAVES, int TM, int TN, bool HAS_SCALE = false, int RESERVE = 0,
-          bool HAS_ROW = false, bool BIAS_LDS = false, int ACC_BLOCK0 = -1>
+          bool HAS_ROW = false, bool BIAS_LDS = false, int ACC_BLOCK0 = -1, bool CLEAR_ACC = false>
 __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM][TN], unsigned char *stage,
                                               int wave_row0, int wave_col0, int lane,
                                               const float *scale_lds = nullptr,
@@ -704,6 +708,15 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
   const __amdgpu_buffer_rsrc_t crs =
       __builtin_amdgcn_make_buffer_rsrc((void *)uni(cp.c), 0, uni(cp.c_bytes), kRsrcFlags);
   const int col_base = cp.n0 + wave_col0;
+  // (a fragment of zeros, made here and not ahead of the tile loop, where it
+  // would hold four registers through the k-loop)
+  h16x8_t zero_frag;
+  if constexpr (CLEAR_ACC) {
+    u32x4_t z;
+    asm volatile("v_mov_b32 %0, 0\nv_mov_b32 %1, 0\nv_mov_b32 %2, 0\nv_mov_b32 %3, 0"
+                 : "=v"(z[0]), "=v"(z[1]), "=v"(z[2]), "=v"(z[3]));
+    zero_frag = __builtin_bit_cast(h16x8_t, z);
+  }
   // Bias of this lane's columns, fetched in one batch (one wait instead of one per element).
   float bias_v[OUT_BLOCKS][16];
   if (HAS_BIAS) {
@@ -776,6 +789,10 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
         if constexpr (ACC_BLOCK0 >= 0) {
           blk = fixed_acc_block<ACC_BLOCK0 + i * TN + j>();
           if constexpr (SWIGLU) up = fixed_acc_block<ACC_BLOCK0 + i * TN + j + OUT_BLOCKS>();
+          if constexpr (CLEAR_ACC) {   // ready for the next tile's sums
+            mfma_fixed_clear<ACC_BLOCK0 + i * TN + j>(zero_frag);
+            if constexpr (SWIGLU) mfma_fixed_clear<ACC_BLOCK0 + i * TN + j + OUT_BLOCKS>(zero_frag);
+          }
         } else {
           blk = acc_block<WAVES == 4>(acc[i][j]);
           if constexpr (SWIGLU) up = acc_block<WAVES == 4>(acc[i][j + OUT_BLOCKS]);
@@ -806,6 +823,10 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
         if constexpr (ACC_BLOCK0 >= 0) {
           blk = fixed_acc_block<ACC_BLOCK0 + i * TN + j>();
           if constexpr (SWIGLU) up = fixed_acc_block<ACC_BLOCK0 + i * TN + j + OUT_BLOCKS>();
+          if constexpr (CLEAR_ACC) {   // ready for the next tile's sums
+            mfma_fixed_clear<ACC_BLOCK0 + i * TN + j>(zero_frag);
+            if constexpr (SWIGLU) mfma_fixed_clear<ACC_BLOCK0 + i * TN + j + OUT_BLOCKS>(zero_frag);
+          }
         } else {
           blk = acc_block<WAVES == 4>(acc[i][j]);
           if constexpr (SWIGLU) up = acc_block<WAVES == 4>(acc[i][j + OUT_BLOCKS]);
@@ -1584,7 +1605,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
       step(c1);
     }
     fixed_acc_settle();
-    tile_epilogue<MODE, HAS_BIAS && !kBiasInAcc, kQWaves, TM, TN, W8, W8 ? kEpiReserve : 0, false, false, kAccBlock0>(
+    tile_epilogue<MODE, HAS_BIAS && !kBiasInAcc, kQWaves, TM, TN, W8, W8 ? kEpiReserve : 0, false, false, kAccBlock0, !kBiasInAcc>(
         cp, no_acc, stage_rows, wm * WTM, wave_col0, lane, lds_scale + scale_buf * kScaleBufFloats);
     // The load side is within the next tile here (every tile has at least
     // kQMinSteps steps).
@@ -1603,7 +1624,8 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
     bias_buf ^= 1;
     scale_buf = scale_buf == 2 ? 0 : scale_buf + 1;       // the tile multiplied next
     copy_scale(nxt, scale_buf == 2 ? 0 : scale_buf + 1);  // the one after it
-    init_acc(cp, bias_buf, scale_buf);
+    // (without a bias the epilogue has cleared every block it read)
+    if constexpr (kBiasInAcc) init_acc(cp, bias_buf, scale_buf);
     // The last block above already fetched these fragments; reading them again
     // here keeps 32 registers free during the epilogue.
     read_frags(c0, c0, c0);
