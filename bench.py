@@ -282,6 +282,107 @@ def time_staleness(cfg, variant, dev, x, sample_steps=50, modes=("high", "low", 
     return out
 
 
+def time_sustained_cold(cfg, variant, dev, n_blocks=8, seconds=1.0):
+    """What the reference's sampler makes of the layer: a stack of blocks with distinct weights,
+    each with its own input, walked in order again and again (models.py:653-688 walks `depth`
+    blocks per step).  `n_blocks` blocks of this configuration (8 x 271 MB of weights at C2:
+    beyond the 256 MB memory-side cache, so every call streams its weights from HBM) are
+    called round-robin for at least `seconds`, with no host synchronisation inside a group
+    of 64 calls; the dominant launch is bracketed by the library's two HIP events per call
+    over the SAME run.  Returns whole-run throughput and that launch's mean duration."""
+    import ctypes
+    from dice_amd.lib import check
+    lib, n, names = _stage_names()
+    fc1 = names.index("moe.mlp.fc1")
+    buf = (ctypes.c_float * n)()
+    blocks = [make_block(cfg, variant, dev, layer_idx=l, total_layers=n_blocks) for l in range(n_blocks)]
+    xs = [make_input(cfg, dev, seed=100 + l) for l in range(n_blocks)]
+    ys = [torch.empty_like(x) for x in xs]
+    weight_bytes = 0
+    for b in blocks:
+        b.run(xs[0], y=ys[0])        # packs the weights, sizes the workspace
+        pk = b._packed
+        weight_bytes += sum(t.numel() * t.element_size() for t in (pk.w1, pk.w2, pk.sw1, pk.sw2) if t is not None)
+    for l, b in enumerate(blocks):   # one untimed walk
+        b.run(xs[l], y=ys[l])
+    check(lib.dice_profile_enable(2))
+    calls, fc1_ms = 0, 0.0
+    rounds_per_group = max(1, 64 // n_blocks)
+    try:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while True:
+            for _ in range(rounds_per_group):
+                for l, b in enumerate(blocks):
+                    b.run(xs[l], y=ys[l])
+            group = rounds_per_group * n_blocks
+            check(lib.dice_profile_read(buf, n))   # waits for this group's last fc1 launch only
+            fc1_ms += buf[fc1] * group
+            calls += group
+            if time.perf_counter() - t0 >= seconds:
+                break
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+    finally:
+        check(lib.dice_profile_enable(0))
+    del blocks, xs, ys
+    torch.cuda.empty_cache()
+    return {"blocks": n_blocks, "distinct_weight_bytes": weight_bytes, "calls": calls, "seconds": wall,
+            "ms_per_step": wall / calls * 1e3, "tokens_per_s": cfg["tokens"] * calls / wall,
+            "fc1_ms_per_launch": fc1_ms / calls}
+
+
+def time_staleness_layers(cfg, variant, dev, n_layers=8, sample_steps=50, mode="high"):
+    """The staleness loop as the reference runs it: `n_layers` blocks with distinct weights and
+    one skip-cache entry per layer (cache_capacity = depth, sample_ddp.py:182-192), every
+    sampler step walking all of them; layer l has its own drifting input.  Milliseconds per
+    layer call over the whole loop (host clock, no synchronisation inside) and per step kind
+    (two events per layer call)."""
+    from dice_amd import ParaMode, diep
+    n_tok, D = cfg["tokens"], cfg["D"]
+    blocks = [make_block(cfg, variant, dev, l, n_layers, ParaMode(ep=True)) for l in range(n_layers)]
+    g = torch.Generator(device=dev).manual_seed(5)
+    noise = [0.05 * torch.randn((1, n_tok, D), generator=g, device=dev, dtype=torch.float32) for _ in range(4)]
+    x0 = [make_input(cfg, dev, seed=200 + l).view(1, n_tok, D) for l in range(n_layers)]
+    try:
+        diep.ep_cache_init(cache_capacity=n_layers, noskip_step=2, skip_mode=mode)
+        diep.ep_set_rand_mask(None)
+        ev = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_layers)]
+              for _ in range(sample_steps)]
+        kinds, wall = [], 0.0
+        for rep in range(2):            # first repetition warms up
+            xt = [x.clone() for x in x0]
+            kinds = []
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for j, (i, clear) in enumerate(staleness_schedule(sample_steps)):
+                diep.ep_set_step(i)
+                if clear:
+                    diep.ep_cache_clear()
+                kinds.append("skip" if diep.ep_skip_now(0) else "full")
+                for l, b in enumerate(blocks):
+                    ev[j][l][0].record()
+                    b(xt[l])
+                    ev[j][l][1].record()
+                    xt[l] = (xt[l].float() + noise[(i + l) % 4]).to(xt[l].dtype)
+            torch.cuda.synchronize()
+            wall = time.perf_counter() - t0
+        per = {"full": [], "skip": []}
+        for j, kd in enumerate(kinds):
+            per[kd].extend(ev[j][l][0].elapsed_time(ev[j][l][1]) for l in range(n_layers))
+        cached = diep.ep_cached_tensors_size()
+    finally:
+        diep.ep_cache_init(cache_capacity=1, noskip_step=1)
+    del blocks
+    torch.cuda.empty_cache()
+    calls = sample_steps * n_layers
+    return {"layers": n_layers, "skip_mode": mode, "ms_per_layer_call": sum(sum(v) for v in per.values()) / calls,
+            "loop_wall_ms_per_layer_call_incl_drift_update": wall / calls * 1e3,
+            "full_put_step_ms_per_layer_call": statistics.mean(per["full"]),
+            "skip_step_ms_per_layer_call": statistics.mean(per["skip"]),
+            "full_steps": kinds.count("full"), "skip_steps": kinds.count("skip"), "cached_bytes_at_end": cached}
+
+
 def time_lagged(cfg, variant, dev, x, steps, warmup, pipeline):
     """ms per layer call of the step-lagged modes on the same block shape: two
     layers, a forced-sync first step, then `steps` lagged steps (displaced: each
@@ -626,6 +727,8 @@ def main():
     ap.add_argument("--no-caller", action="store_true", help="skip the fused-caller (LayerNorm/modulate + residual) pass")
     ap.add_argument("--no-staleness", action="store_true", help="skip the 50-step conditional-communication loop")
     ap.add_argument("--no-lagged", action="store_true", help="skip the step-lagged (displaced / interweaved) pass")
+    ap.add_argument("--no-sustained", action="store_true",
+                    help="skip the sustained pass over eight blocks with distinct weights")
     ap.add_argument("--no-vendor", action="store_true",
                     help="skip the vendor-GEMM reference (torch.matmul on the routed fc1 shape with the same operands)")
     ap.add_argument("--no-configs", action="store_true",
@@ -713,6 +816,19 @@ def main():
     if not args.no_staleness and main_cfg == "c2":
         # configs[3] on the same block shape (not part of `value`)
         out["staleness_loop_50_steps"] = time_staleness(CONFIGS["c4"], args.variant, dev, x)
+    if not args.no_sustained and cfg["dtype"] == "bf16":
+        # The reference walks a stack of blocks with distinct weights (not part of `value`): eight blocks of this
+        # configuration round-robin for at least a second, the dominant launch timed over that same run.
+        sus = time_sustained_cold(cfg, args.variant, dev)
+        out["tokens_per_s_sustained_cold"] = sus["tokens_per_s"]
+        if "roofline" in out and sus["fc1_ms_per_launch"] > 0:
+            ach = out["roofline"]["flop_per_launch"] / (sus["fc1_ms_per_launch"] * 1e-3) / 1e12
+            sus["fc1_achieved_tflops"] = ach
+            sus["fc1_frac_of_peak"] = ach / out["roofline"]["peak"]
+        out["sustained_cold_layers"] = sus
+    if not args.no_staleness and main_cfg == "c2":
+        # configs[3] with one cache entry per layer over a stack of eight distinct blocks (not part of `value`)
+        out["staleness_loop_50_steps_8_layers"] = time_staleness_layers(CONFIGS["c4"], args.variant, dev)
     if not args.no_lagged and main_cfg == "c2":
         # the same layer under the reference's step-lagged schedules (not part of `value`)
         out["step_lag_ms_per_layer_call"] = {

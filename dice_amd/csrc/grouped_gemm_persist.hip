@@ -2197,6 +2197,51 @@ int64_t model_makespan(const PersistProblem *prob, int n_problems, int bn_out, i
   }
   return makespan;
 }
+// The most turns any workgroup walks when every problem has its tallest
+// possible groups (the row bound plus a ragged tile per expert), under one way
+// of sharing the tiles out over the XCDs: the device's arithmetic, counted in
+// tiles instead of steps.
+int64_t worst_case_turns(const PersistProblem *prob, int n_problems, int bn_out_fc1, bool fc2, int wgs, int split) {
+  int64_t tiles[kMaxPersistProblems], steps[kMaxPersistProblems], base[kMaxPersistProblems], total_cost = 0, total = 0;
+  for (int p = 0; p < n_problems; ++p) {
+    const PersistProblem &pr = prob[p];
+    const int bn_out = !fc2 ? bn_out_fc1 : (pr.n % 192 == 0 && pr.n % 256 != 0 ? 192 : kPBN);
+    const int64_t m_tiles = ((int64_t)pr.max_rows + kPBM - 1) / kPBM + pr.n_experts;
+    tiles[p] = m_tiles * ((pr.n + bn_out - 1) / bn_out);
+    steps[p] = pr.k / 32;
+    base[p] = total;
+    total += tiles[p];
+    total_cost += tiles[p] * steps[p];
+  }
+  auto boundary = [&](int x) -> int64_t {
+    if (x >= kNumXcd) return total;
+    const int64_t target = total_cost * x / kNumXcd;
+    int64_t cbase = 0;
+    for (int p = 0; p < n_problems; ++p) {
+      const int64_t c = tiles[p] * steps[p];
+      if (c > 0 && target >= cbase && target < cbase + c) return base[p] + (target - cbase + steps[p] / 2) / steps[p];
+      cbase += c;
+    }
+    return total;
+  };
+  int64_t worst = 0;
+  for (int x = 0; x < kNumXcd; ++x) {
+    int64_t run = 0;
+    for (int p = 0; p < n_problems; ++p) {
+      int64_t lo, hi;
+      if (split == 0) {
+        lo = std::max(boundary(x), base[p]);
+        hi = std::min(boundary(x + 1), base[p] + tiles[p]);
+      } else {
+        lo = base[p] + tiles[p] * x / kNumXcd;
+        hi = base[p] + tiles[p] * (x + 1) / kNumXcd;
+      }
+      run += std::max<int64_t>(0, hi - lo);
+    }
+    worst = std::max(worst, (run + wgs - 1) / wgs);
+  }
+  return worst;
+}
 PersistPlan persist_plan(const PersistBatch &b, int bn_out, int grid, bool fc2) {
   struct Shape {
     int n_problems, bn_out, grid, rows[kMaxPersistProblems], experts[kMaxPersistProblems], n[kMaxPersistProblems],
@@ -2389,19 +2434,28 @@ bool persist_common_ok(const PersistBatch &b, int mode) {
 
 // Whether every workgroup's turns fit the LDS tile table of the 64-k kernel
 // (the last entry stays an invalid tile), bounded from the host-side row
-// bounds: an XCD gets an eighth of every problem's tiles.  Launches that do not
-// fit take the table-rewriting kernels.
-bool persist64_fits_table(const PersistBatch &b, int mode) {
-  int64_t tiles_per_xcd = 0;
+// bounds for either way of sharing the tiles out over the XCDs (the launcher
+// picks one later): an eighth of every problem's tiles, or an eighth of the
+// total cost - which, for an XCD that gets only the shortest tiles, is that
+// cost divided by the shortest tile's.  Launches that do not fit take the
+// table-rewriting kernels.
+int64_t persist64_turn_bound(const PersistBatch &b, int mode, int wgs_per_xcd) {
+  int64_t tiles_per_xcd = 0, total_cost = 0, min_k32 = 1 << 30;
   for (int i = 0; i < b.n_problems; ++i) {
     const PersistProblem &p = b.prob[i];
     const int bn_out = mode == kFc1Swiglu ? kPBN / 2 : (p.n % 192 == 0 && p.n % 256 != 0 ? 192 : kPBN);
     const int64_t m_tiles = ((int64_t)p.max_rows + kPBM - 1) / kPBM + p.n_experts;
     const int64_t n_tiles = (p.n + bn_out - 1) / bn_out;
     tiles_per_xcd += m_tiles * n_tiles / kNumXcd + 1;
+    total_cost += m_tiles * n_tiles * (p.k / 32);
+    min_k32 = std::min<int64_t>(min_k32, std::max(1, p.k / 32));
   }
-  const int wgs_per_xcd = cu_count() / kNumXcd;
-  return (tiles_per_xcd + wgs_per_xcd - 1) / wgs_per_xcd + 2 <= kTableTurns;
+  const int64_t by_cost = total_cost / kNumXcd / min_k32 + 2;
+  const int64_t run = std::max(tiles_per_xcd, by_cost);
+  return (run + wgs_per_xcd - 1) / wgs_per_xcd + 2;
+}
+bool persist64_fits_table(const PersistBatch &b, int mode) {
+  return persist64_turn_bound(b, mode, cu_count() / kNumXcd) <= kTableTurns;
 }
 
 // 64-k kernel: long enough tiles.
@@ -2436,6 +2490,28 @@ int persist_variant(const PersistBatch &b, int mode) {
 
 bool persist_supported(const PersistBatch &b, int mode) { return persist_variant(b, mode) != 0; }
 size_t persist_split_ws_bytes() { return (size_t)kPersistSplitSlots * kPBM * kPBN * 2; }
+}  // namespace dice
+extern "C" int dice_debug_persist_turns(int n_problems, const int64_t *max_rows, const int32_t *n_experts,
+                                        const int32_t *n, const int32_t *k, int fc2, int wgs_per_xcd,
+                                        int xcd_split, int64_t *bound_out, int64_t *turns_out) {
+  using namespace dice;
+  if (n_problems < 1 || n_problems > kMaxPersistProblems || !max_rows || !n_experts || !n || !k || !bound_out ||
+      !turns_out || wgs_per_xcd < 1)
+    return fail(DICE_ERR_BAD_ARG, "dice_debug_persist_turns: bad argument");
+  PersistBatch b{};
+  b.n_problems = n_problems;
+  for (int i = 0; i < n_problems; ++i) {
+    b.prob[i].max_rows = (int)max_rows[i];
+    b.prob[i].n_experts = n_experts[i];
+    b.prob[i].n = n[i];
+    b.prob[i].k = k[i];
+  }
+  const int mode = fc2 ? kFc2 : kFc1Swiglu;
+  *bound_out = persist64_turn_bound(b, mode, wgs_per_xcd);
+  *turns_out = worst_case_turns(b.prob, n_problems, kPBN / 2, fc2 != 0, wgs_per_xcd, xcd_split);
+  return DICE_OK;
+}
+namespace dice {
 #endif  // !DICE_PERSIST_F16
 
 namespace {

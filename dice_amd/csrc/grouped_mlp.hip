@@ -43,6 +43,24 @@ struct LayerWorkspace {
   size_t total;
 };
 
+// Widths the fp8 x fp8 expert path takes: whole 256-k pairs of steps, at least six
+// steps per tile, rows the quantiser holds in registers.
+bool act_quant_widths_ok(int hidden, int inter) {
+  auto ok = [](int w) { return w % 256 == 0 && w >= 768 && w <= 8192; };
+  return ok(hidden) && ok(inter);
+}
+
+// Whether a layer call can launch a single-problem fc2 (the only launches that
+// cut a short last turn along k and need the partial-tile slots): routed experts
+// with fp8 weights (their bf16 shared expert rides alone), no shared expert, or
+// the small batches whose shared fc2 gets a launch of its own.
+bool shared_fc2_alone(const dice_moe_layer_t *L, int64_t n_tokens, int64_t max_rows);
+bool layer_may_split_fc2(const dice_moe_layer_t *L, int64_t n_tokens) {
+  if (!is_16bit(L->act_dtype) || L->batch_invariant) return false;
+  if (L->w_dtype == DICE_FP8_E4M3 || L->shared_inter == 0) return true;
+  return shared_fc2_alone(L, n_tokens, 0);   // (fewer routed rows, as on a skip step, only make it likelier)
+}
+
 LayerWorkspace carve_layer(const dice_moe_layer_t *L, int64_t n_tokens, void *ws) {
   LayerWorkspace w;
   Carve c{(unsigned char *)ws, 0};
@@ -66,7 +84,7 @@ LayerWorkspace carve_layer(const dice_moe_layer_t *L, int64_t n_tokens, void *ws
     w.shared_h = w.shared_out = nullptr;
   }
   w.modulated = c.take_bytes((size_t)n_tokens * L->hidden * es);  // layer input when the caller's prologue runs here
-  w.split_ws = is_16bit(L->act_dtype) ? c.take_bytes(persist_split_ws_bytes()) : nullptr;
+  w.split_ws = layer_may_split_fc2(L, n_tokens) ? c.take_bytes(persist_split_ws_bytes()) : nullptr;
   w.q_rows = nullptr;
   w.q_scale = nullptr;
   if (L->act_quant) {
@@ -377,6 +395,7 @@ namespace {
 bool shared_fc2_alone(const dice_moe_layer_t *L, int64_t n_tokens, int64_t max_rows) {
   const int choice = shared_fc2_launch_choice();
   if (choice != 0) return choice > 0;
+  if (L->batch_invariant) return false;   // (the second launch only pays where both cut their tiles)
   // (tiles of fewer than 64 steps: a second launch costs what the cut saves - DiT-B width, 48 and 24
   // steps: 95 / 89 us at 64 tokens, but 114 / 119 at 1024 and 121 / 129 at 1536)
   if (!persist_split_allowed() || (L->inter < 4096 && L->shared_inter < 4096)) return false;
@@ -412,11 +431,16 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
     DICE_REQUIRE(L->shared_w1 && L->shared_w2 && L->shared_inter % 64 == 0, DICE_ERR_BAD_ARG,
                  "%s: shared expert weights / shared_inter %d", who, L->shared_inter);
   }
-  if (L->act_quant || LE->act_quant)
+  if (L->act_quant || LE->act_quant) {
     DICE_REQUIRE(L->act_quant == 1 && LE->act_quant == 1 && L->act_dtype == DICE_BF16 &&
                      LE->w_dtype == DICE_FP8_E4M3 && LE->w1_scale && LE->w2_scale,
                  DICE_ERR_UNSUPPORTED,
                  "%s: act_quant (0 or 1) needs bf16 activations and fp8 expert weights with scales, in both layers", who);
+    // (what the fp8 kernels and the row quantiser take, checked before anything is launched)
+    DICE_REQUIRE(act_quant_widths_ok(L->hidden, L->inter), DICE_ERR_UNSUPPORTED,
+                 "%s: act_quant needs hidden %d and inter %d to be multiples of 256 between 768 and 8192", who,
+                 L->hidden, L->inter);
+  }
   if (combine_mode == 1)
     DICE_REQUIRE(skip_mask && cache_out, DICE_ERR_BAD_ARG, "%s: a put step needs skip_mask and cache_out", who);
   if (combine_mode == 2)
@@ -544,7 +568,7 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
                                   swiglu ? nullptr : L->shared_b2, w.shared_out, L->hidden, L->hidden, si, (int)n_tokens};
       s1.n_problems = s2.n_problems = 1;
     }
-    f2.split_ws = s2.split_ws = persist_split_allowed() ? w.split_ws : nullptr;
+    f2.split_ws = s2.split_ws = persist_split_allowed() && !L->batch_invariant ? w.split_ws : nullptr;
     const bool shared_persist = s1.n_problems && persist_supported(s1, m1) && persist_supported(s2, kFc2);
     rc = mlp_a8_run(
         3, work.x, work.perm, L->top_k, work.offsets, L->n_experts, max_rows, L->hidden, L->inter, f1, f2, swiglu,
@@ -601,7 +625,7 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
         f1.n_problems = f2.n_problems = 2;
       }
     }
-    f2.split_ws = s2.split_ws = persist_split_allowed() ? w.split_ws : nullptr;
+    f2.split_ws = s2.split_ws = persist_split_allowed() && !L->batch_invariant ? w.split_ws : nullptr;
     const bool shared_ok = (s1.n_problems == 0 || persist_supported(s1, m1)) &&
                            (s2.n_problems == 0 || persist_supported(s2, kFc2));
     // Where the kernel can address the activation rows through the permutation

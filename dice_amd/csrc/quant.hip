@@ -70,6 +70,7 @@ __global__ __launch_bounds__(256) void quantize_act_rows_kernel(const T *__restr
   const int n_chunks = cols / 8;  // 16-byte pieces of a row
   u32x4_t v[CHUNKS];
   float m = 0.f;
+  bool finite = true;
 #pragma unroll
   for (int c = 0; c < CHUNKS; ++c) {
     const int i = c * kWave + lane;
@@ -77,11 +78,19 @@ __global__ __launch_bounds__(256) void quantize_act_rows_kernel(const T *__restr
     if (i < n_chunks) v[c] = row[i];
     const T *e = reinterpret_cast<const T *>(&v[c]);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(to_f32(e[j])));
+    for (int j = 0; j < 8; ++j) {
+      const float a = fabsf(to_f32(e[j]));
+      finite = finite && a < __builtin_inff();   // (false for NaN as well; fmaxf would drop a NaN)
+      m = fmaxf(m, a);
+    }
   }
   m = wave_max(m);
-  const float inv = m > 0.f ? 448.0f / m : 1.0f;
-  if (lane == 0) scale[r] = m > 0.f ? m / 448.0f : 1.0f;
+  // A row with a NaN or an infinity stays visible: its scale is NaN, which the
+  // GEMM's epilogue multiplies into every output of the row (a 16-bit row would
+  // carry it through the products likewise); its bytes are zeros.
+  const bool row_finite = __ballot(!finite) == 0;
+  const float inv = !row_finite ? 0.f : m > 0.f ? 448.0f / m : 1.0f;
+  if (lane == 0) scale[r] = !row_finite ? __builtin_nanf("") : m > 0.f ? m / 448.0f : 1.0f;
   u32x2_t *qrow = reinterpret_cast<u32x2_t *>(q + r * cols);
 #pragma unroll
   for (int c = 0; c < CHUNKS; ++c) {
@@ -89,7 +98,7 @@ __global__ __launch_bounds__(256) void quantize_act_rows_kernel(const T *__restr
     const T *e = reinterpret_cast<const T *>(&v[c]);
     float f[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) f[j] = fminf(fmaxf(to_f32(e[j]) * inv, -448.f), 448.f);
+    for (int j = 0; j < 8; ++j) f[j] = row_finite ? fminf(fmaxf(to_f32(e[j]) * inv, -448.f), 448.f) : 0.f;
     u32x2_t o;
     int w = 0;
     w = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], w, false);

@@ -80,12 +80,8 @@ def moe_infer_ep(inp, experts, flat_expert_indices, flat_expert_weights, num_exp
     else:
         work = emit = new
     owner = work.owner if work.owner is not None else blk
-    if owner._packed is None:
-        owner.pack_weights(owner._fp8)
-    q = owner._packed
-    work.rows = ops.grouped_mlp(work.x, work.perm, k, work.offsets, work.max_rows, q.w1, q.w2, owner.variant,
-                                q.b1, q.b2, q.w1_scale, q.w2_scale, scatter_to_slots=False,
-                                n_out_rows=max(work.max_rows, 1), out=work.rows)
+    # (the block's own arithmetic: the fp8 matrix pipe when it quantises its activations)
+    work.rows = owner.routed_experts(work.x, work.perm, work.offsets, work.max_rows, out=work.rows)
     if emit.rows is None:
         raise DiceError("moe_infer_ep: the cached step to return has never been through the experts")
     cache_in = cache_out = None

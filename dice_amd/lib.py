@@ -38,6 +38,7 @@ EXPORTS = [
     "dice_grouped_mlp",
     "dice_grouped_mlp_stage",
     "dice_set_gemm_config",
+    "dice_debug_persist_turns",
     "dice_profile_enable",
     "dice_profile_stage_count",
     "dice_profile_stage_name",
@@ -71,7 +72,7 @@ class MoeLayerDesc(Structure):
         ("b1", c_void_p), ("b2", c_void_p), ("w1_scale", c_void_p), ("w2_scale", c_void_p),
         ("shared_w1", c_void_p), ("shared_w2", c_void_p),
         ("shared_b1", c_void_p), ("shared_b2", c_void_p),
-        ("act_quant", c_int32),
+        ("act_quant", c_int32), ("batch_invariant", c_int32),
     ]
 
 
@@ -170,6 +171,9 @@ def load() -> ctypes.CDLL:
     lib.dice_profile_read.argtypes = [POINTER(c_float), c_int]
     lib.dice_set_gemm_config.restype = c_int
     lib.dice_set_gemm_config.argtypes = [c_int, c_int]
+    lib.dice_debug_persist_turns.restype = c_int
+    lib.dice_debug_persist_turns.argtypes = [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                             c_void_p, c_void_p]
     if lib.dice_abi_version() != 2:
         raise DiceError(f"ABI version {lib.dice_abi_version()} != 2")
     _lib = lib

@@ -197,6 +197,9 @@ class SparseMoeBlock(nn.Module):
         self._packed: Optional[_Packed] = None
         self._fp8 = False
         self._act_quant = False      # fp8 experts: activations quantised per row too (fp8 matrix pipe)
+        # True: a token's result never depends on what else is in the call (no fc2 tile is cut along k; see
+        # dice_moe_layer_t.batch_invariant).  Set it before the first call, or clear ``_desc`` after changing it.
+        self.batch_invariant = False
         self._desc = None
         self._ws = None
         self._spare_cache = None     # a skip-cache tensor a skip step has consumed: the next full step writes into it
@@ -266,10 +269,37 @@ class SparseMoeBlock(nn.Module):
         ``activations=True`` also quantises the routed experts' input rows (per
         token, dynamically, in front of each GEMM), so that the products run on
         the fp8 matrix pipe; bf16 blocks whose widths are multiples of 256."""
+        if activations:
+            # what the fp8 matrix-pipe kernels and the row quantiser take; refused here, not at the first forward
+            for name, width in (("hidden", self.embed_dim), ("expert", self.inter)):
+                if width % 256 != 0 or not 768 <= width <= 8192:
+                    raise DiceError(f"quantize_fp8(activations=True): {name} width {width} is not a multiple of 256 "
+                                    f"between 768 and 8192; use quantize_fp8() (e4m3 weights, 16-bit activations)")
+            if next(self.experts.parameters()).dtype != torch.bfloat16:
+                raise DiceError("quantize_fp8(activations=True): act_quant (the fp8 matrix-pipe path) takes bf16 "
+                                "blocks; use quantize_fp8() (e4m3 weights, 16-bit activations)")
         self.pack_weights(fp8=True)
         self._act_quant = bool(activations)
         self._desc = None
         return self
+
+    def routed_experts(self, x, perm, offsets, max_rows, out=None):
+        """The routed experts' two GEMMs on grouped rows (reference models.py:368-377)
+        in the arithmetic this block's layer call uses: e4m3 rows on the fp8 matrix
+        pipe when the block quantises its activations, else 16-bit rows.  Returns
+        the unweighted expert outputs ``[max_rows, D]`` in grouped order."""
+        if self._packed is None:
+            self.pack_weights(self._fp8)
+        p = self._packed
+        k = self.num_experts_per_tok
+        if self._act_quant and self._fp8:
+            if out is None:
+                out = torch.zeros((max(max_rows, 1), self.embed_dim), dtype=x.dtype, device=x.device)
+            rows, _ = ops.grouped_mlp_a8(x, perm, k, offsets, max_rows, p.w1, p.w2, p.w1_scale, p.w2_scale,
+                                         self.variant, p.b1, p.b2, out=out)
+            return rows
+        return ops.grouped_mlp(x, perm, k, offsets, max_rows, p.w1, p.w2, self.variant, p.b1, p.b2,
+                               p.w1_scale, p.w2_scale, scatter_to_slots=False, n_out_rows=max(max_rows, 1), out=out)
 
     def _ensure(self, x: torch.Tensor):
         if self._packed is None:
@@ -293,6 +323,7 @@ class SparseMoeBlock(nn.Module):
             d.shared_w1, d.shared_w2 = ptr(p.sw1), ptr(p.sw2)
             d.shared_b1, d.shared_b2 = ptr(p.sb1), ptr(p.sb2)
             d.act_quant = int(self._act_quant and self._fp8)
+            d.batch_invariant = int(self.batch_invariant)
             self._desc = d
         return self._desc
 
@@ -505,9 +536,6 @@ class SparseMoeBlock(nn.Module):
     @torch.no_grad()
     def moe_infer(self, x, flat_expert_indices, flat_expert_weights):
         """Routed experts only, from given routing (reference models.py:361-382)."""
-        if self._packed is None:
-            self.pack_weights(self._fp8)
-        p = self._packed
         k = self.num_experts_per_tok
         n = x.shape[0]
         if flat_expert_indices.numel() != n * k or flat_expert_weights.numel() != n * k:
@@ -515,7 +543,6 @@ class SparseMoeBlock(nn.Module):
                             f"weights for {n} tokens x {k}")
         idx = flat_expert_indices.reshape(-1).to(torch.int32).contiguous()
         _, offsets, perm, inv_perm = ops.dispatch(idx, len(self.experts))
-        rows = ops.grouped_mlp(x.contiguous(), perm, k, offsets, n * k, p.w1, p.w2, self.variant,
-                               p.b1, p.b2, p.w1_scale, p.w2_scale, scatter_to_slots=False)
+        rows = self.routed_experts(x.contiguous(), perm, offsets, n * k)
         w = flat_expert_weights.reshape(n, k).float().contiguous()
         return ops.combine(rows, w, n, k, inv_perm=inv_perm)

@@ -265,7 +265,18 @@ typedef struct dice_moe_layer {
                            * on the way into each GEMM (dice_quantize_fp8_act)
                            * and multiplied on the fp8 matrix pipe: needs
                            * act_dtype BF16, w_dtype FP8_E4M3, hidden and inter
-                           * multiples of 256 */
+                           * multiples of 256 between 768 and 8192 */
+  int32_t batch_invariant; /* 1: a token's result does not depend on what else is in
+                           * the call.  By default an fc2 launch that carries one
+                           * problem (fp8 routed weights, no shared expert, or a
+                           * small batch whose shared expert gets its own launch)
+                           * and whose tiles leave most workgroups idle in their
+                           * last turn cuts that turn's tiles along k and adds the
+                           * 16-bit pieces in fp32 in a fixed order: deterministic,
+                           * but a token's last bit can then depend on the number
+                           * of tokens (or dropped slots) in the call, and a skip
+                           * step fed its own cache need not reproduce the full
+                           * step bit for bit.  1 multiplies every tile whole. */
 } dice_moe_layer_t;
 
 /* mode: 0 = plain step; 1 = full step that also writes cache_out ("put");
@@ -399,25 +410,37 @@ const char *dice_profile_stage_name(int i);
 int dice_profile_read(float *ms_out, int n);
 
 /*
- * Tuning hook, no counterpart in the reference: selects the kernel of the
- * bf16/fp8 expert GEMMs per stage (0 = library default).  1..4 force a tiling
- * of the permutation-addressed kernels; 20 restricts the persistent launches to
- * the 32-k pipeline; 30 + b (b = 1..16) walks the persistent launches' tiles in
- * bands of b m-tiles; fc1_cfg = 50 has dice_moe_forward_modulated launch the
- * router on its own behind the prologue kernel instead of inside it (same
- * results); fc2_cfg = 50 has the layer calls multiply every fc2 tile whole;
- * fc2_cfg = 51 / 52 have them launch the shared expert's fc2 on its own always /
- * never (by default for small batches only);
- * any value from 20 on (21 does nothing else) keeps a dice_grouped_mlp stage
- * whose groups average at most 128 rows on the persistent kernels, which by
- * default leave it to the 64-row tiles of the permutation-addressed ones.  (By default a single-problem fc2 launch - fp8 routed weights, or no
- * shared expert - whose tiles leave most workgroups idle in their last turn
- * cuts that turn's tiles along k, one piece per workgroup, and adds the 16-bit
- * pieces in fp32 in a fixed order: results are deterministic, but a token's last
- * bit can then depend on the number of tokens in the call.)  Process-wide;
- * meant for benchmarks and tests that compare kernels, not for the drop-in path.
+ * Tuning hook, no counterpart in the reference: one code per GEMM stage of the
+ * bf16/fp8 expert MLPs (0 = library default).  Process-wide; meant for benchmarks
+ * and tests that compare kernels, not for the drop-in path (a caller who needs
+ * results that do not depend on the batch sets dice_moe_layer_t.batch_invariant).
+ * Any code from DICE_GEMM_CFG_PIPE32 on also keeps a dice_grouped_mlp stage whose
+ * groups average at most 128 rows on the persistent kernels, which by default
+ * leave it to the 64-row tiles of the permutation-addressed ones.
  */
+#define DICE_GEMM_CFG_DEFAULT 0
+/* 1..4: force a tiling of the permutation-addressed kernels (either stage) */
+#define DICE_GEMM_CFG_PIPE32 20          /* persistent launches on the 32-k pipeline only */
+#define DICE_GEMM_CFG_PERSISTENT 21      /* nothing but the small-group rule above */
+#define DICE_GEMM_CFG_BANDS(b) (30 + (b)) /* b = 1..16: tiles of the persistent launches in bands of b m-tiles */
+#define DICE_GEMM_CFG_FC1_ROUTER_OWN_LAUNCH 50 /* fc1: dice_moe_forward_modulated launches the router behind the prologue
+                                                * kernel instead of inside it (same results) */
+#define DICE_GEMM_CFG_FC2_WHOLE_TILES 50 /* fc2: no last turn is cut along k (as batch_invariant, for every layer) */
+#define DICE_GEMM_CFG_FC2_SHARED_ALONE 51 /* fc2: the shared expert's fc2 always in a launch of its own */
+#define DICE_GEMM_CFG_FC2_SHARED_JOINT 52 /* fc2: ... never (by default: small batches only) */
 int dice_set_gemm_config(int fc1_cfg, int fc2_cfg);
+
+/*
+ * Test hook, no counterpart in the reference: the host-side bound on the turns
+ * a workgroup of a persistent expert-GEMM launch may walk (which decides whether
+ * the launch takes the kernel that rewrites its tile table) and, for the same
+ * shapes with every group as tall as the bound allows, the most turns any
+ * workgroup gets when the tiles are shared out over the XCDs by cost
+ * (xcd_split 0) or per problem (1).  Arrays of n_problems entries.
+ */
+int dice_debug_persist_turns(int n_problems, const int64_t *max_rows, const int32_t *n_experts,
+                             const int32_t *n, const int32_t *k, int fc2, int wgs_per_xcd,
+                             int xcd_split, int64_t *bound_out, int64_t *turns_out);
 
 #ifdef __cplusplus
 }

@@ -40,8 +40,12 @@ Pinning status (what independently fixes each function's result):
                           previous step, computed with its own experts), by the
                           forced-sync step being exact, and by the latest- vs
                           stale-weight switch changing only the scale factors.
-                          Its combination with the skip cache is exercised only
-                          as a state machine: "parity unpinned".
+                          Step lag together with the skip cache (displaced and
+                          interweaved, cached and latest weights): a float64
+                          per-token closed form with a different input, routing
+                          and weights at every step (which entry is emitted,
+                          whether it blends with or refills the cache, which
+                          weights scale it).
 * ``norm_modulate`` /    - float64 numpy definition of LayerNorm (biased variance
   ``dit_block_moe_half``  around the mean, eps inside the root) and of the two
                           affine maps on small inputs; constant rows give
@@ -781,8 +785,9 @@ def quantize_fp8_act(x: torch.Tensor):
     """Per-row (per-token) dynamic quantisation of activations to OCP e4m3fn,
     as the fp8 expert GEMMs take them: ``amax = max|row|``,
     ``q = rne(row * (448 / amax))``, ``scale = amax / 448`` (1.0 and zeros for
-    an all-zero row).  The quotient ``448 / amax`` and the product are each
-    rounded once in fp32 (IEEE division, not reciprocal times 448).  Returns (q float8_e4m3fn [rows, cols], scale fp32 [rows])."""
+    an all-zero row; NaN and zeros for a row that holds a NaN or an infinity).
+    The quotient ``448 / amax`` and the product are each rounded once in fp32
+    (IEEE division, not reciprocal times 448).  Returns (q float8_e4m3fn [rows, cols], scale fp32 [rows])."""
     xf = x.float()
     amax = xf.abs().amax(dim=-1)
     nz = amax > 0
@@ -792,6 +797,12 @@ def quantize_fp8_act(x: torch.Tensor):
     inv = torch.where(nz, torch.full_like(amax, E4M3_MAX) / amax, one)
     scale = torch.where(nz, amax / E4M3_MAX, one)
     q = (xf * inv[:, None]).clamp(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn)
+    # a row with a NaN or an infinity: zeros and a NaN scale, so that every output
+    # of the row is NaN, as the 16-bit path would give (build-defined)
+    bad = ~torch.isfinite(xf).all(dim=-1)
+    if bad.any():
+        q = torch.where(bad[:, None], torch.zeros_like(xf), q.float()).to(torch.float8_e4m3fn)
+        scale = torch.where(bad, torch.full_like(scale, float("nan")), scale)
     return q, scale
 
 

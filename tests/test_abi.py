@@ -300,3 +300,39 @@ int main(void) {
     run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
     assert run.returncode == 0, (run.returncode, run.stderr)
     assert "null pointer" in run.stdout
+
+
+@pytest.mark.parametrize("split", [0, 1])
+@pytest.mark.parametrize("tokens", [64, 1024, 8192, 16384, 65536, 140000, 300000])
+@pytest.mark.parametrize("shape", ["swiglu_fc1", "swiglu_fc2", "literal_fc2", "fp8_fc2"])
+def test_tile_table_bound_covers_every_xcd_split(shape, tokens, split):
+    """The host decides from a bound on a workgroup's turns whether a persistent
+    expert-GEMM launch may take the kernel whose LDS tile table holds 64 turns.
+    The bound has to cover both ways of sharing the tiles out over the XCDs: with
+    contiguous eighths of the cost, an XCD that gets only the short tiles of a
+    launch whose problems differ in k walks more tiles than an eighth of every
+    problem's.  Here: the bound against the device's arithmetic restated on the
+    host, with every group as tall as the row bound allows."""
+    import numpy as np
+    from dice_amd import lib
+    cdll = ctypes.CDLL(lib.LIB_PATH)
+    D, I, E = 1152, 4608, 8
+    if shape == "swiglu_fc1":     # routed + shared fc1, k = D for both
+        rows, experts, n, k, fc2 = [2 * tokens, tokens], [E, 1], [I, I // 2], [D, D], 0
+    elif shape == "swiglu_fc2":   # routed k = I, shared k = I / 2
+        rows, experts, n, k, fc2 = [2 * tokens, tokens], [E, 1], [D, D], [I, I // 2], 1
+    elif shape == "literal_fc2":  # shared expert of twice the routed width: k = 2 I
+        rows, experts, n, k, fc2 = [2 * tokens, tokens], [E, 1], [D, D], [I, 2 * I], 1
+    else:                         # fp8 routed experts: one problem
+        rows, experts, n, k, fc2 = [2 * tokens], [16], [2048], [8192], 1
+    a = lambda v, t: np.asarray(v, dtype=t)
+    rows_a, exp_a, n_a, k_a = a(rows, np.int64), a(experts, np.int32), a(n, np.int32), a(k, np.int32)
+    bound, turns = ctypes.c_int64(), ctypes.c_int64()
+    cdll.dice_debug_persist_turns.argtypes = [ctypes.c_int] + [ctypes.c_void_p] * 4 + [ctypes.c_int] * 3 + \
+        [ctypes.POINTER(ctypes.c_int64)] * 2
+    rc = cdll.dice_debug_persist_turns(len(rows), rows_a.ctypes.data, exp_a.ctypes.data, n_a.ctypes.data,
+                                       k_a.ctypes.data, fc2, 32, split, ctypes.byref(bound), ctypes.byref(turns))
+    assert rc == 0
+    # (one table entry stays an invalid tile, which ends the workgroup's walk)
+    assert turns.value + 1 <= bound.value, f"{shape} {tokens} tokens, split {split}: {turns.value} turns, bound {bound.value}"
+    assert bound.value <= 2 * turns.value + 4, "the bound should not send small launches to the rewriting kernel"

@@ -70,6 +70,33 @@ def test_act_quantiser_bit_exact(dev, dtype, cols):
     assert not q.cpu().view(torch.uint8)[33:].any() and not s.cpu()[33:].any()   # untouched
 
 
+def test_act_quantiser_keeps_non_finite_rows_visible(dev):
+    """A row with a NaN or an infinity gets a NaN scale (and zero bytes), so that
+    every output of that row is NaN, as the 16-bit path would give; its
+    neighbours are untouched.  Pinned in the oracle alike (build-defined)."""
+    from dice_amd import ops
+    x = torch.randn(6, 1024, generator=_gen(77)).bfloat16()
+    x[1, 5] = float("nan")
+    x[3, 1000] = float("inf")
+    x[4, 17] = float("-inf")
+    q, s = ops.quantize_fp8_act(x.to(dev))
+    wq, ws = O.quantize_fp8_act(x)
+    assert torch.equal(torch.isnan(s.cpu()), torch.tensor([False, True, False, True, True, False]))
+    assert torch.equal(torch.isnan(ws), torch.isnan(s.cpu()))
+    good = ~torch.isnan(ws)
+    assert torch.equal(s.cpu()[good], ws[good])
+    assert torch.equal(q.cpu().view(torch.uint8), wq.view(torch.uint8))
+    # through the expert GEMMs: NaN rows out, finite neighbours
+    D, E = 1024, 4
+    p = O.make_block_params(D, E, 2, 2, None, seed=5, dtype=torch.bfloat16)
+    blk = block_from_params(p, D, "swiglu", torch.bfloat16, dev)
+    blk.quantize_fp8(activations=True)
+    idx = torch.tensor([0, 1] * 6)
+    w = torch.full((12, 1), 0.5).bfloat16()
+    y = blk.moe_infer(x.to(dev), idx.to(dev), w.to(dev)).cpu().float()
+    assert torch.isnan(y[[1, 3, 4]]).all() and torch.isfinite(y[[0, 2, 5]]).all()
+
+
 def _packed(p, variant, dev):
     if variant == "swiglu":
         w1 = torch.stack([torch.cat([e.gate_proj, e.up_proj], 0) for e in p.experts])
@@ -217,9 +244,42 @@ def test_act_quant_needs_fp8_weights_and_bf16(dev):
     D, E = 1024, 8
     p = O.make_block_params(D, E, 2, 4, 2, seed=1, dtype=torch.float16)
     blk = block_from_params(p, D, "swiglu", torch.float16, dev)
+    with pytest.raises(DiceError, match="act_quant"):      # refused when asked for, not at the first forward
+        blk.quantize_fp8(activations=True)
+    # widths the fp8 matrix-pipe kernels do not take (DiT-XL: 1152 = 4.5 x 256) are refused up front as well
+    p = O.make_block_params(1152, E, 2, 4, 2, seed=1, dtype=torch.bfloat16)
+    blk = block_from_params(p, 1152, "swiglu", torch.bfloat16, dev)
+    with pytest.raises(DiceError, match="multiple of 256"):
+        blk.quantize_fp8(activations=True)
+    blk.quantize_fp8()                                      # e4m3 weights with 16-bit activations still apply
+    assert blk(torch.zeros(1, 64, 1152, dtype=torch.bfloat16, device=dev)).shape == (1, 64, 1152)
+
+
+def test_block_a8_one_arithmetic_behind_every_entry_point(dev):
+    """A block that quantises its activations computes its routed experts on the
+    fp8 matrix pipe whichever way it is entered: SparseMoeBlock.moe_infer
+    (models.py:361-382) and moe_infer_ep (expertpara/ep_fwd.py:19) with the
+    caller's own routing give the oracle's Fp8ActExpert result, the same rows
+    bit for bit, and not the result of the 16-bit-activation path."""
+    from dice_amd import ParaMode, diep
+    from dice_amd.ep_fwd import moe_infer_ep
+    D, E, N, k = 1024, 8, 600, 2
+    g = _gen(31)
+    p = O.make_block_params(D, E, k, 4, None, seed=30, dtype=torch.bfloat16)
+    x = torch.randn(N, D, generator=g).bfloat16()
+    idx = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(N)]).view(-1)
+    w = torch.rand(N * k, 1, generator=g).bfloat16()
+    blk = block_from_params(p, D, "swiglu", torch.bfloat16, dev, para_mode=ParaMode(ep=True))
     blk.quantize_fp8(activations=True)
-    with pytest.raises(DiceError, match="act_quant"):
-        blk(torch.zeros(1, 64, D, dtype=torch.float16, device=dev))
+    want = O.moe_infer(x, _a8_oracle(p).experts, idx, w, k)
+    y = blk.moe_infer(x.to(dev), idx.to(dev), w.to(dev)).cpu()
+    check_rows(y, want, SAME_QUANT_TOL, "moe_infer on the fp8 matrix pipe vs same quantisation")
+    diep.ep_cache_init(cache_capacity=1, noskip_step=1)
+    y_ep = moe_infer_ep(x.to(dev), blk.experts, idx.to(dev), w.to(dev), k, False).cpu()
+    assert torch.equal(y_ep, y)
+    blk.quantize_fp8(activations=False)
+    y16 = blk.moe_infer(x.to(dev), idx.to(dev), w.to(dev)).cpu()
+    assert not torch.equal(y16, y)
 
 
 def test_block_a8_step_lag_and_fused_caller(dev):

@@ -35,7 +35,7 @@ def _reset(diep):
 
 
 def _drive(dev, dtype, L, strategy, pipeline, latest, steps, D=256, E=8, N=384, noskip=1, skip_mode=None,
-           tol=FP32_TOL, forced_at=(0,)):
+           tol=FP32_TOL, forced_at=(0,), drift=0.05):
     """Runs ``steps`` sampler steps over a stack of ``L`` blocks (layer l+1
     reads layer l's output plus a per-step drift, so every layer sees different
     inputs every step) on the GPU and in the oracle, comparing every output."""
@@ -77,7 +77,7 @@ def _drive(dev, dtype, L, strategy, pipeline, latest, steps, D=256, E=8, N=384, 
             if forced:
                 diep.diep_cancel_sync()
                 state.cancel_sync()
-            x0 = x0 + 0.05 * torch.randn(1, N, D, generator=g)
+            x0 = (x0 if drift < 1.0 else 0.0) + drift * torch.randn(1, N, D, generator=g)
         assert diep.ep_cached_tensors_size() > 0
     finally:
         _reset(diep)
@@ -110,14 +110,19 @@ def test_interweaved_bf16_persistent_path(dev):
            tol=BF16_TOL)
 
 
+@pytest.mark.parametrize("latest", [False, True])
 @pytest.mark.parametrize("pipeline", [False, True])
 @pytest.mark.parametrize("mode", ["high", "low"])
-def test_lag_with_conditional_communication(dev, pipeline, mode):
+def test_lag_with_conditional_communication(dev, pipeline, mode, latest):
     """Step lag together with the skip cache at interval 2: whether a call
     blends with the cache or refills it follows the entry it returns, not the
-    current step."""
-    _drive(dev, torch.float32, L=2, strategy="all", pipeline=pipeline, latest=True, steps=7, noskip=2,
-           skip_mode=mode)
+    current step.  Every step draws a fresh input (no two steps alike, so the
+    wrong entry, a stale cache row or the wrong routing weights cannot pass),
+    with the cached and with the latest routing weights; the oracle's side of
+    this sequence is pinned by the float64 closed form of
+    tests/test_oracle.py::test_lag_with_skip_cache_closed_form."""
+    _drive(dev, torch.float32, L=2, strategy="all", pipeline=pipeline, latest=latest, steps=9, noskip=2,
+           skip_mode=mode, drift=1.0)
 
 
 def test_lagged_equals_earlier_synchronous_result(dev):

@@ -128,6 +128,32 @@ def test_cut_turn_is_deterministic_and_leaves_the_stage_calls_alone(dev):
     assert rel_l2(skip, a) < 4e-3   # (half the rows: another tile count, another cut)
 
 
+def test_batch_invariant_layer_multiplies_every_tile_whole(dev):
+    """``dice_moe_layer_t.batch_invariant`` (``SparseMoeBlock.batch_invariant``) is the
+    supported switch for callers who need a token's result not to depend on
+    what else is in the call: the layer then equals the whole-tile schedule of the
+    process-wide tuning hook bit for bit, a skip step fed its own cache reproduces
+    the full step exactly, and a token gives the same bits in a smaller batch."""
+    from dice_amd import lib
+    D, E, N = 768, 4, 1024
+    p = O.make_block_params(D, E, 2, 2, 0, seed=41, dtype=torch.bfloat16)
+    x = torch.randn(N, D, generator=_gen(42)).bfloat16().to(dev)
+    cutting = block_from_params(p, D, "swiglu", torch.bfloat16, dev)
+    whole, cut = _whole_and_cut(cutting, x.view(1, N, D))
+    assert not torch.equal(whole, cut)
+    blk = block_from_params(p, D, "swiglu", torch.bfloat16, dev)
+    blk.batch_invariant = True
+    a = blk.run(x).clone()
+    assert torch.equal(a.cpu(), whole.view(N, D))
+    mask = O.skip_mask(2 * N, "high").to(dev)
+    cache = torch.empty_like(x)
+    put = blk.run(x, lib.MODE_PUT, mask, None, cache).clone()
+    skip = blk.run(x, lib.MODE_SKIP, mask, cache, None)
+    assert torch.equal(put, a) and torch.equal(skip, a)
+    part = blk.run(x[:300].contiguous())
+    assert torch.equal(part, a[:300])
+
+
 @pytest.mark.parametrize("variant,n_shared,N", [
     ("swiglu", 2, 256),       # the reference's shared expert (k = 2304) beside routed tiles of 72 steps
     ("swiglu", 2, 700),       # ragged groups, the largest batch that still takes the separate launch

@@ -417,34 +417,87 @@ def test_interweaved_lag_closed_form(strategy, latest):
             state.cancel_sync()
 
 
-def test_displaced_with_skip_cache_state_machine():
-    """Displaced lag together with conditional communication, interval 2, on
-    the reference schedule: the sizes that flow through the caches stay
-    consistent (every call returns [N, D]) and, because the lag of two steps
-    preserves the full/skip parity, a skip-step entry always meets a skip cache
-    entry.  Values: with identical inputs every step the lagged result equals
-    the synchronous full result."""
-    n, d, E = 16, 8, 4
-    gen = torch.Generator().manual_seed(5)
-    experts = _rand_linear_experts(gen, E, d)
-    x = torch.randn(n, d, generator=gen)
-    idx = torch.stack([torch.randperm(E, generator=gen)[:2] for _ in range(n)]).reshape(-1)
-    w = torch.rand(2 * n, 1, generator=gen)
-    want = _per_token(x, experts, idx, w)
-    state = O.DiepState(1, noskip_step=2, skip_mode="low")
-    mask = O.skip_mask(2 * n, "low")
-    for i in range(10, 0, -1):
+def _expert_row(experts, e, x64_row):
+    ex = experts[int(e)]
+    return ex.w.double().numpy() @ x64_row + ex.b.double().numpy()
+
+
+@pytest.mark.parametrize("skip_mode", ["low", "high"])
+@pytest.mark.parametrize("latest", [False, True])
+@pytest.mark.parametrize("pipeline", [False, True])
+def test_lag_with_skip_cache_closed_form(pipeline, latest, skip_mode):
+    """Step lag together with conditional communication (interval 2) on the
+    reference's countdown schedule, with a different input, routing and routing
+    weights at every step and in every layer, against a float64 per-token
+    definition that shares no code with the oracle (expertpara/ep_fwd.py:49-66,
+    176-193; expertpara/diep.py:196-289; expertpara/ep_cache.py:215-220).
+
+    What a call returns is fixed by three things.  (1) Which earlier call's
+    routing and rows it emits: displaced mode emits step 0 at steps 0 and 1 and
+    step t - 2 from then on; interweaved mode emits the layer's own step t - 1
+    (step 0 at step 0).  (2) What kind of entry that was: a call made while
+    ``ep_skip_now`` held dispatched only its unmasked slot, so its emission takes
+    the masked slot's row from the skip cache (which ``get`` empties); a full
+    entry's emission refills the cache with its masked slots' unweighted rows.
+    (3) The routing weights: the emitting call's own when
+    ``use_latest_expert_weights``, else those of the emitted entry.  A wrong lag
+    (1 for 2), put and work swapped, a stale cache row or the wrong weights
+    each change the result, because no two steps share an input here."""
+    L, n, d, E, steps = (3 if pipeline else 1), 12, 8, 4, 9
+    gen = torch.Generator().manual_seed(17 + int(pipeline))
+    layers = [_rand_linear_experts(gen, E, d) for _ in range(L)]
+    state = O.DiepState(L, noskip_step=2, skip_mode=skip_mode, async_pipeline=pipeline,
+                        selective_async_strategy="all" if pipeline else None, use_latest_expert_weights=latest)
+    mask = O.skip_mask(2 * n, skip_mode)
+    m = 0 if skip_mode == "high" else 1          # the masked slot of every token; r = the other
+    r = 1 - m
+    hist = []                                    # per step, per layer: (x, idx, w, kind)
+    cache_rows = [None] * L                      # the skip cache as this test keeps it: float64 rows [n, d] or None
+    for t in range(steps):
+        i = steps - t                            # the sampler counts down (rectified_flow.py:83-128)
         state.step = i
-        forced = i == 10
+        forced = t == 0
         if forced:
             state.force_sync()
             state.cache_clear()
-        now = O.skip_now(True, state.skip, 0, i, 2)
-        got = O.moe_infer_ep_async(state, x, experts, idx, w, 2, True, mask, now, 0)
+            cache_rows = [None] * L
+        cur = []
+        for l in range(L):
+            x = torch.randn(n, d, generator=gen)
+            idx = torch.stack([torch.randperm(E, generator=gen)[:2] for _ in range(n)]).reshape(-1)
+            w = torch.rand(2 * n, 1, generator=gen)
+            now = O.skip_now(True, state.skip, l, i, 2)
+            # the test's own view of the policy (diep.py:61-68): enabled, an entry in the cache, an odd step
+            assert now == (cache_rows[l] is not None and i % 2 != 0)
+            cur.append((x, idx, w, "skip" if now else "full"))
+            got = O.moe_infer_ep_async(state, x, layers[l], idx, w, 2, True, mask, now, l)
+            if forced:
+                ex, eidx, ew, kind = cur[l]
+            elif pipeline:
+                ex, eidx, ew, kind = hist[t - 1][l]
+            else:
+                ex, eidx, ew, kind = hist[max(t - 2, 0)][l]
+            wt = (w if latest else ew).double().numpy().reshape(n, 2)
+            x64 = ex.double().numpy()
+            want = np.zeros((n, d))
+            if kind == "full":
+                rows_m = np.stack([_expert_row(layers[l], eidx[2 * tok + m], x64[tok]) for tok in range(n)])
+                rows_r = np.stack([_expert_row(layers[l], eidx[2 * tok + r], x64[tok]) for tok in range(n)])
+                cache_rows[l] = rows_m           # the put of a full emission: unweighted rows of the masked slots
+            else:
+                assert cache_rows[l] is not None, "a skip entry is emitted against an empty cache"
+                rows_m = cache_rows[l]           # whatever expert the masked slot names now: the cached row stands
+                rows_r = np.stack([_expert_row(layers[l], eidx[2 * tok + r], x64[tok]) for tok in range(n)])
+                cache_rows[l] = None             # get empties the entry
+            for tok in range(n):
+                want[tok] = wt[tok, m] * rows_m[tok] + wt[tok, r] * rows_r[tok]
+            assert got.shape == x.shape
+            assert torch.allclose(got.double(), torch.from_numpy(want), atol=1e-4, rtol=1e-5), (t, l, kind)
+        hist.append(cur)
         if forced:
             state.cancel_sync()
-        assert got.shape == x.shape
-        assert torch.allclose(got, want, atol=1e-5, rtol=1e-5), i
+    kinds = [h[0][3] for h in hist]
+    assert "skip" in kinds[1:] and "full" in kinds[1:], kinds
 
 
 # --------------------------------------------------------------------------- #
@@ -493,3 +546,19 @@ def test_block_caller_identities():
     # fp32: one rounding or four, same result
     out_s, *_ = O.dit_block_moe_half(p, x, shift, scale, gate, single_rounding=True)
     assert torch.allclose(out_s, out, atol=1e-5)
+
+
+def test_fp8_act_quantiser_non_finite_rows():
+    """Build-defined: a row holding a NaN or an infinity quantises to zero bytes
+    with a NaN scale (so every product of the row is NaN, as a 16-bit row would
+    give); finite rows beside it are quantised as if it were not there."""
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(4, 64, generator=g)
+    clean_q, clean_s = O.quantize_fp8_act(x)
+    x[1, 3] = float("inf")
+    x[2, 9] = float("nan")
+    q, s = O.quantize_fp8_act(x)
+    assert torch.isnan(s[1]) and torch.isnan(s[2]) and torch.isfinite(s[[0, 3]]).all()
+    assert (q[1].float() == 0).all() and (q[2].float() == 0).all()
+    assert torch.equal(q[[0, 3]].view(torch.uint8), clean_q[[0, 3]].view(torch.uint8))
+    assert torch.equal(s[[0, 3]], clean_s[[0, 3]])
