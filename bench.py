@@ -656,6 +656,12 @@ def ab_hooks(cfg_name, variant, activations, dev, hook_a, hook_b, lib_b=None, ca
             getattr(other, name).restype = getattr(libs[0], name).restype
             getattr(other, name).argtypes = getattr(libs[0], name).argtypes
         libs[1] = other
+        # (the other build may size its workspace differently: take the larger of the two)
+        other.dice_moe_workspace_bytes.restype = libs[0].dice_moe_workspace_bytes.restype
+        other.dice_moe_workspace_bytes.argtypes = libs[0].dice_moe_workspace_bytes.argtypes
+        need = int(other.dice_moe_workspace_bytes(ctypes.byref(desc), x.shape[0]))
+        if need > ws.numel() * ws.element_size():
+            ws = torch.empty(need, dtype=torch.uint8, device=x.device)
     caller = None
     if call == "modulated":
         B = cfg["samples"]

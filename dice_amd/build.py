@@ -57,10 +57,24 @@ def _hipcc() -> str:
 ACC_CHECKED = {"grouped_gemm_persist.hip", "grouped_gemm_persist_f16.hip"}
 
 
+def _generate_sources() -> None:
+    """Writes the generated k-loop of the expert GEMM (csrc/gen_persist64_asm.py) into the
+    build directory, which is on the include path of every translation unit."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("gen_persist64_asm", os.path.join(CSRC, "gen_persist64_asm.py"))
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)
+    text = gen.generate()
+    path = os.path.join(BUILD_DIR, "persist64_asm.inc")
+    if not os.path.exists(path) or open(path).read() != text:
+        with open(path, "w") as f:
+            f.write(text)
+
+
 def _compile(src: str, extra) -> str:
     stem = os.path.splitext(src)[0]
     obj = os.path.join(BUILD_DIR, stem + ".o")
-    cmd = [_hipcc(), *HIP_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [_hipcc(), *HIP_FLAGS, "-I", BUILD_DIR, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     if src in ACC_CHECKED:
         cmd.insert(-4, "-save-temps=obj")
     r = subprocess.run(cmd, capture_output=True, text=True)
@@ -78,6 +92,7 @@ def build_library(verbose: bool = True, extra_flags=(), out: str = None) -> str:
     ``python -m dice_amd.build --out /tmp/other.so -DDICE_MFMA_ROWS_OUTERMOST=1``)."""
     target = os.path.abspath(out) if out else LIB_PATH
     os.makedirs(BUILD_DIR, exist_ok=True)
+    _generate_sources()
     jobs = min(len(SOURCES), max(1, min(8, os.cpu_count() or 1)))
     with ThreadPoolExecutor(jobs) as pool:
         objs = list(pool.map(lambda s: _compile(s, list(extra_flags)), SOURCES))

@@ -183,6 +183,9 @@ __device__ __forceinline__ void fixed_acc_clear() {
   else
     asm volatile(".set dice_acc_r, 64\n.rept 192\nv_accvgpr_write_b32 a[dice_acc_r], 0\n.set dice_acc_r, dice_acc_r + 1\n.endr" ::: "a255");
 }
+// Tells the compiler that the kernel uses accumulation registers up to a255 (it
+// sizes the wave's register file from the registers it sees named).
+__device__ __forceinline__ void fixed_acc_declare() { asm volatile("" ::: "a255", "v255"); }
 // Wait states between a product and a vector-ALU access to its sums (19 for the
 // longest matrix instruction), and between a vector-ALU write and a product.
 __device__ __forceinline__ void fixed_acc_settle() { asm volatile("s_nop 7\ns_nop 7\ns_nop 7"); }
@@ -692,13 +695,19 @@ __device__ __forceinline__ f32x16_t acc_block(const f32x16_t &a) {
 // caller has let the last products settle.  CLEAR_ACC: every block is cleared as
 // soon as it has been read (mfma_fixed_clear), so the next tile's products can
 // add to it at once.
+// ROW_STRIDE: tile rows between a wave's consecutive 32-row blocks (32: the wave
+// owns a solid band of the tile; 64: the two waves that share a tile's columns
+// take alternate 32-row blocks).  live_blocks (wave-uniform): only the wave's
+// first live_blocks row blocks hold rows of the group (a group's last tile);
+// the others were not multiplied and are not touched.
 template <int MODE, bool HAS_BIAS, int WAVES, int TM, int TN, bool HAS_SCALE = false, int RESERVE = 0,
-          bool HAS_ROW = false, bool BIAS_LDS = false, int ACC_BLOCK0 = -1, bool CLEAR_ACC = false>
+          bool HAS_ROW = false, bool BIAS_LDS = false, int ACC_BLOCK0 = -1, bool CLEAR_ACC = false,
+          int ROW_STRIDE = 32>
 __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM][TN], unsigned char *stage,
                                               int wave_row0, int wave_col0, int lane,
                                               const float *scale_lds = nullptr,
                                               const float *rowscale_lds = nullptr,
-                                              const float *bias_lds = nullptr) {
+                                              const float *bias_lds = nullptr, int live_blocks = TM) {
   static_assert(!(HAS_BIAS && BIAS_LDS), "one source of the bias");
   using G = EpiGeom<MODE, WAVES, TM, TN, RESERVE>;
   constexpr bool SWIGLU = G::SWIGLU;
@@ -760,7 +769,7 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
       if (MODE == kFc1Gelu) v = gelu_tanh_fast(v);          \
     }                                                       \
   } while (0)
-#define DICE_EPI_STORE_BAND(band)                                                                          \
+#define DICE_EPI_STORE_BAND(row_off)                                                                        \
   do {                                                                                                     \
     wave_lds_sync();                                                                                       \
     _Pragma("unroll") for (int ps = 0; ps < G::PASSES; ++ps) {                                             \
@@ -771,7 +780,7 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
         r = live ? r : 0;                                                                                  \
       }                                                                                                    \
       const u32x4_t v = *reinterpret_cast<const u32x4_any_t *>(stage + r * PITCH + rd_chunk * 16);         \
-      const int m = wave_row0 + (band) * BAND + r;                                                         \
+      const int m = wave_row0 + (row_off) + r;                                                             \
       const int n = col_base + rd_chunk * 8;                                                               \
       const uint32_t voff = (live && n < cp.n) ? (uint32_t)m * cp.c_pitch + (uint32_t)n * 2 : kOutOfRange; \
       __builtin_amdgcn_raw_buffer_store_b128(v, crs, voff, 0, 0);                                          \
@@ -780,8 +789,9 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
   } while (0)
   static_for<TM>([&](auto i_c) {
     constexpr int i = decltype(i_c)::value;
+    if (i >= live_blocks) return;
     float row_scale = 1.0f;
-    if (HAS_ROW) row_scale = rowscale_lds[wave_row0 + i * 32 + frag_row];
+    if (HAS_ROW) row_scale = rowscale_lds[wave_row0 + i * ROW_STRIDE + frag_row];
     if constexpr (BAND == 32) {
       static_for<OUT_BLOCKS>([&](auto j_c) {
         constexpr int j = decltype(j_c)::value;
@@ -811,7 +821,7 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
           *reinterpret_cast<u32x2_any_t *>(stage + frag_row * PITCH + col * 2) = __builtin_bit_cast(u32x2_t, o);
         }
       });
-      DICE_EPI_STORE_BAND(i);
+      DICE_EPI_STORE_BAND(i * ROW_STRIDE);
     } else {
       // The staging rows hold 16 rows at a time.  The activation of the whole
       // 32-row block is worked out once, with every lane at work (per band only
@@ -854,7 +864,7 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
                   __builtin_bit_cast(u32x2_t, packed[j][q]);
             }
         }
-        DICE_EPI_STORE_BAND(2 * i + half);
+        DICE_EPI_STORE_BAND(i * ROW_STRIDE + half * 16);
       }
     }
     // Keeps the 32-row blocks apart: hoisting the next block's accumulator reads
@@ -1632,6 +1642,301 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// The same 64-k pipeline with its k-loop in assembly (persist64_asm.inc, written by
+// gen_persist64_asm.py: register plan, order of the pieces and wait counts are
+// described there).  Every memory instruction of the loop, its registers and its
+// waits are spelled out; the compiler's share between the statements is scalar
+// bookkeeping (the load side's position, the tile switch) and the epilogue.
+// What this buys over the loop the compiler schedules (gemm_persist64_body):
+//   * a group's last tile multiplies only its live 64-row blocks (the two waves
+//     that share a tile's columns take alternate 32-row blocks, so both have
+//     work in every live block): one loop variant per number of live blocks;
+//   * the first products of a tile start the sums (no clearing);
+// neither of which the compiler-scheduled loop survives: a second copy of the
+// loop or a branch inside it sends its register allocator through the
+// accumulation registers and its wait-count pass to lgkmcnt(0) at every join
+// (in-block branches: bit-identical results, 62 % longer layer call).
+// Taken for 16-bit weights and bias-free tiles of the two shapes generated:
+// KIND 0 = SwiGLU fc1 with gathered rows (256 weight rows), KIND 1 = fc2 with
+// 192 weight rows.
+struct P64Addr {
+  uint32_t wr[2];       // LDS address of this lane's chunk in slot 0 / 1 (writes)
+  uint32_t ra[2][4];    // LDS address of this lane's activation fragment of 16-k block kk in slot 0 / 1
+  uint32_t rb[2][4];    // ... of its weight fragment
+  uint32_t va[8];       // byte offsets of this lane's eight activation rows in the tile being loaded
+  uint32_t vb;          // ... of its first weight row (the others: scalar offsets, P64_PARAMS)
+};
+#define P64_PARAMS                                                                                        \
+  f32x32_t &f0, f32x32_t &f1, const P64Addr &ad, u32x4_t dA, u32x4_t dB0, u32x4_t dB1, uint32_t koff,       \
+      const uint32_t (&sb)[8]
+#define P64_ARGS f0, f1, ad, dA, dB0, dB1, koff, sb
+#define P64_CONSTRAINTS                                                                                         \
+  : "+{v[0:31]}"(f0), "+{v[32:63]}"(f1)                                                                         \
+  : [wr0] "v"(ad.wr[0]), [wr1] "v"(ad.wr[1]), [ra00] "v"(ad.ra[0][0]), [ra01] "v"(ad.ra[0][1]),                 \
+    [ra02] "v"(ad.ra[0][2]), [ra03] "v"(ad.ra[0][3]), [ra10] "v"(ad.ra[1][0]), [ra11] "v"(ad.ra[1][1]),         \
+    [ra12] "v"(ad.ra[1][2]), [ra13] "v"(ad.ra[1][3]), [rb00] "v"(ad.rb[0][0]), [rb01] "v"(ad.rb[0][1]),         \
+    [rb02] "v"(ad.rb[0][2]), [rb03] "v"(ad.rb[0][3]), [rb10] "v"(ad.rb[1][0]), [rb11] "v"(ad.rb[1][1]),         \
+    [rb12] "v"(ad.rb[1][2]), [rb13] "v"(ad.rb[1][3]), [va0] "v"(ad.va[0]), [va1] "v"(ad.va[1]),                 \
+    [va2] "v"(ad.va[2]), [va3] "v"(ad.va[3]), [va4] "v"(ad.va[4]), [va5] "v"(ad.va[5]), [va6] "v"(ad.va[6]),    \
+    [va7] "v"(ad.va[7]), [vb] "v"(ad.vb), [dA] "s"(dA), [dB0] "s"(dB0), [dB1] "s"(dB1), [koff] "s"(koff),       \
+    [sb0] "s"(sb[0]), [sb1] "s"(sb[1]), [sb2] "s"(sb[2]), [sb3] "s"(sb[3]), [sb4] "s"(sb[4]), [sb5] "s"(sb[5]), \
+    [sb6] "s"(sb[6]), [sb7] "s"(sb[7])                                                                          \
+  : "memory"
+typedef float f32x32_t __attribute__((ext_vector_type(32)));
+#include "persist64_asm.inc"
+
+template <int MODE, bool HAS_BIAS, int BN, bool GATHER, bool W8>
+constexpr bool persist64_asm_applies() {
+  return !W8 && !HAS_BIAS && ((MODE == kFc1Swiglu && BN == 256 && GATHER) || (MODE == kFc2 && BN == 192));
+}
+
+template <int MODE, int BN, bool GATHER, bool REFILL>
+__device__ __forceinline__ void gemm_persist64_asm_body(const PersistBatch &batch) {
+  constexpr bool SWIGLU = MODE == kFc1Swiglu;
+  constexpr int KIND = SWIGLU ? 0 : 1;
+  constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
+  constexpr int WTN = BN / 2, TM = 4, TN = WTN / 32;
+  constexpr int kCopiesA = kPBM / 8 / kQWaves, kCopiesB = BN / 8 / kQWaves;
+  constexpr int kAccBlock0 = 16 - TM * TN;
+  using Epi = EpiGeom<MODE, kQWaves, TM, TN, 0>;
+  typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
+
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_slot0[kQSlotBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_slot1[kQSlotBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_stage[kPStageArea];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  fixed_acc_declare();
+
+  constexpr int kTableBytes = kTableTurns * kTileWords * 4, kRowSlotBytes = kPBM * 4;
+  static_assert(kQWaves * Epi::WAVE_BYTES + kTableBytes + (GATHER ? kRowSlotBytes : 0) <= kPStageArea,
+                "no room for the tile table");
+  uint32_t *const tile_table = reinterpret_cast<uint32_t *>(lds_stage + kPStageArea - kTableBytes);
+  int32_t *const lds_row_slots = reinterpret_cast<int32_t *>(lds_stage + kPStageArea - kTableBytes - kRowSlotBytes);
+  if (wave == 0) {
+    TileWalker<BN_OUT> walk(batch, lane);
+    walk.build_table(batch, lane, kQBK, tile_table, false);
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  phase_barrier();
+  auto fetch_tile = [&](int turn) {
+    if constexpr (REFILL) {
+      if (turn != 0 && (turn & (kTableTurns - 1)) == 0) {
+        phase_barrier();
+        if (wave == 0) {
+          TileWalker<BN_OUT> walk(batch, lane);
+          walk.build_table(batch, lane, kQBK, tile_table, false, turn);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        phase_barrier();
+      }
+    }
+    int lane_c = lane;   // (opaque: worked out at the tile switch, not held through the k-loop)
+    asm volatile("" : "+v"(lane_c));
+    return PackedTile{tile_table[(turn & (kTableTurns - 1)) * kTileWords + (lane_c < kTileWords ? lane_c : 0)]};
+  };
+
+  // ---- addresses the assembly takes (see P64Addr) ----
+  const int cp_row0 = wave * 8 + (lane >> 3), cp_chunk = lane & 7;
+  const int b_row0 = SWIGLU ? wn * (WTN / 2) : wn * WTN;
+  const uint32_t slot_base[2] = {(uint32_t)(size_t)(lds_byte_t *)lds_slot0, (uint32_t)(size_t)(lds_byte_t *)lds_slot1};
+  P64Addr ad;
+  // Three of the LDS addresses are kept; the other fifteen follow from them at
+  // the start of every tile (one integer instruction each: 16-k block kk of a
+  // fragment row is the chunk index xor 2 kk, slot 1 lies a constant behind slot
+  // 0), so that they do not hold registers through the epilogue.
+  uint32_t wr0 = slot_base[0] + qring_off(cp_row0, cp_chunk);
+  uint32_t ra0 = slot_base[0] + qring_off(wm * 32 + (lane & 31), lane >> 5);
+  uint32_t rb0 = slot_base[0] + kPBM * 128 + qring_off(b_row0 + (lane & 31), lane >> 5);
+  static_assert((kQSlotBytes & 1023) == 0, "the xor below must stay inside the chunk field");
+  auto set_lds_addresses = [&]() {
+    asm volatile("" : "+v"(wr0), "+v"(ra0), "+v"(rb0));
+    const uint32_t slot1 = slot_base[1] - slot_base[0];
+    ad.wr[0] = wr0;
+    ad.wr[1] = wr0 + slot1;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      // (row block i of wave row wm = tile rows 64 i + 32 wm ..: the assembly adds i x 64 rows)
+      ad.ra[0][kk] = ra0 ^ (uint32_t)(kk << 5);
+      ad.rb[0][kk] = rb0 ^ (uint32_t)(kk << 5);
+      ad.ra[1][kk] = ad.ra[0][kk] + slot1;
+      ad.rb[1][kk] = ad.rb[0][kk] + slot1;
+    }
+  };
+  set_lds_addresses();
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ad.va[i] = 0;
+  ad.vb = 0;
+  uint32_t sb_row[8] = {}, sb[8] = {};   // scalar offsets of the weight loads: row part, and with the step's k offset
+  auto copy_row_slots = [&](const PackedTile &pk) {
+    if constexpr (GATHER) {
+      const uint64_t ptr = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane(pk.words, 21) << 32) |
+                           (uint32_t)__builtin_amdgcn_readlane(pk.words, 20);
+      const int rows = __builtin_amdgcn_readlane(pk.words, 23);
+      if (wave == 0 && ptr != 0) {
+        // Global memory -> LDS without a register in between, as text: a load the
+        // compiler knows of would have it wait for "its only load" with vmcnt(0)
+        // before the next LDS access of its own - which drains the 32 operand
+        // loads the assembly keeps in flight, once per tile.  Rows past the
+        // group's end read as slot 0 (a legal row; their products are never
+        // stored).  M0 holds the LDS address for the instruction and is put back.
+        const u32x4_t rs = {uni((uint32_t)ptr), uni((uint32_t)(ptr >> 32) & 0xffffu), uni((uint32_t)rows * 4u),
+                            kRsrcFlags};
+        const uint32_t dst = uni((uint32_t)(size_t)(lds_byte_t *)lds_row_slots);
+        int lane_c = lane;
+        asm volatile("" : "+v"(lane_c));
+        const uint32_t voff = (uint32_t)lane_c * 16u;
+        uint32_t keep_m0;
+        asm volatile("s_mov_b32 %[keep], m0\n\t"
+                     "s_mov_b32 m0, %[dst]\n\t"
+                     "s_nop 0\n\t"
+                     "buffer_load_dwordx4 %[voff], %[rs], 0 offen lds\n\t"
+                     "s_mov_b32 m0, %[keep]"
+                     : [keep] "=&s"(keep_m0)
+                     : [dst] "s"(dst), [voff] "v"(voff), [rs] "s"(rs)
+                     : "memory");
+      }
+    }
+  };
+  // Descriptors of the tile being loaded, as plain register values (base, extent, flags).
+  u32x4_t dA, dB0, dB1;
+  auto set_copy_offsets = [&](const Tile &t) {
+    auto desc = [](const unsigned char *base, uint32_t bytes) {
+      const uint64_t p = (uint64_t)base;
+      return u32x4_t{uni((uint32_t)p), uni((uint32_t)(p >> 32) & 0xffffu), uni(bytes), kRsrcFlags};
+    };
+    dA = desc(t.a, t.a_bytes);
+    dB0 = desc(t.b0, t.b_bytes);
+    dB1 = desc(t.b1, t.b_bytes);
+    int row0 = cp_row0;   // (opaque, as the lane above)
+    asm volatile("" : "+v"(row0));
+    const uint32_t voff_a = (uint32_t)row0 * t.a_pitch + cp_chunk * 16;
+    const uint32_t voff_b = (uint32_t)row0 * t.b_pitch + cp_chunk * 16;
+#pragma unroll
+    for (int i = 0; i < kCopiesA; ++i) {
+      const int r = row0 + 32 * i;
+      uint32_t off = voff_a + (uint32_t)(32 * i) * t.a_pitch;
+      if constexpr (GATHER) {
+        if (t.a_rows) {
+          const uint32_t slot = (uint32_t)lds_row_slots[r];
+          const uint32_t src_row = t.a_magic ? __umulhi(slot, t.a_magic) : slot;
+          off = r < t.rows ? src_row * t.a_pitch + cp_chunk * 16 : kOutOfRange;
+        }
+      }
+      ad.va[i] = off;
+    }
+    ad.vb = voff_b;
+#pragma unroll
+    for (int i = 0; i < kCopiesB; ++i) {
+      const int row = (SWIGLU && 32 * i >= BN / 2) ? 32 * i - BN / 2 : 32 * i;   // (the up half has its own descriptor)
+      sb_row[i] = uni((uint32_t)row * t.b_pitch);
+    }
+  };
+
+  // ---- pipeline state (as gemm_persist64_body) ----
+  int next_turn = 0;
+  PackedTile nxt = fetch_tile(next_turn++);
+  Tile ld = unpack_tile(nxt);
+  if (!ld.valid) return;
+  if constexpr (GATHER) {
+    copy_row_slots(nxt);
+    pwait_vmcnt<0>();
+    phase_barrier();
+  }
+  Tile cp = ld;
+  int ld_kt = 0;
+  set_copy_offsets(ld);
+  nxt = fetch_tile(next_turn++);
+  if constexpr (GATHER) {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    phase_barrier();
+    copy_row_slots(nxt);
+  }
+  uint32_t koff = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) sb[i] = sb_row[i];
+  auto advance_copy = [&]() {
+    if (++ld_kt == ld.steps) {
+      ld = unpack_tile(nxt);
+      set_copy_offsets(ld);
+      ld_kt = 0;
+    }
+    koff = uni((uint32_t)ld_kt * 128u);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sb[i] = uni(sb_row[i] + koff);
+  };
+  // The two register stages (v128..v255) carry loads in flight from one tile
+  // into the next, across the epilogue: the assembly names them, and the kernel
+  // is compiled with a budget of 128 vector registers (gemm_persist_kernel4a), so
+  // the compiler's own values never sit there.
+  {
+    // (the prologue reads and writes no fragments; the buffers are values of a tile's
+    // k-loop only, so that their registers are free for the epilogue)
+    f32x32_t f0, f1;
+    asm volatile("" : "={v[0:31]}"(f0), "={v[32:63]}"(f1));
+
+  // Prologue: steps 0 and 1 through the stages into the slots (of step 1 only the
+  // first quarter), steps 2 and 3 (first quarter) into the stages behind them.
+  p64_load_step0<KIND, 4>(P64_ARGS);
+  advance_copy();
+  p64_load_step1<KIND, 4>(P64_ARGS);
+  advance_copy();
+  p64_write_step0<KIND, 4>(P64_ARGS);
+  p64_load_step0<KIND, 4>(P64_ARGS);
+  advance_copy();
+  p64_write_q0_stage1<KIND, 4>(P64_ARGS);
+  p64_load_q0_stage1<KIND, 4>(P64_ARGS);
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  phase_barrier();
+
+  unsigned char *const stage_rows = lds_stage + wave * Epi::WAVE_BYTES;
+  f32x16_t no_acc[TM][TN];
+  const int wave_col0 = SWIGLU ? wn * (WTN / 2) : wn * WTN;
+
+  // The steps of a tile whose rows fill its first LIVE 64-row blocks.
+  auto run_tile = [&](auto live_c) {
+    constexpr int LIVE = decltype(live_c)::value;
+    f32x32_t f0, f1;   // the fragment buffers: live inside the tile's k-loop only
+    asm volatile("" : "={v[0:31]}"(f0), "={v[32:63]}"(f1));
+    set_lds_addresses();
+    p64_read_first<KIND, LIVE>(P64_ARGS);
+    p64_abc_s0_v1<KIND, LIVE>(P64_ARGS);   // the first 16-k block's products start the sums
+    advance_copy();
+    p64_d_s0<KIND, LIVE>(P64_ARGS);
+    p64_abc_s1_v0<KIND, LIVE>(P64_ARGS);
+    advance_copy();
+    p64_d_s1<KIND, LIVE>(P64_ARGS);
+    for (int s = 2; s < cp.steps; s += 2) {
+      p64_abc_s0_v0<KIND, LIVE>(P64_ARGS);
+      advance_copy();
+      p64_d_s0<KIND, LIVE>(P64_ARGS);
+      p64_abc_s1_v0<KIND, LIVE>(P64_ARGS);
+      advance_copy();
+      p64_d_s1<KIND, LIVE>(P64_ARGS);
+    }
+  };
+
+  while (true) {  // one tile per iteration
+    const int live = uni((cp.rows + 63) >> 6);   // 64-row blocks of the tile that hold rows of its group
+    if (live >= 4) run_tile(template_int<4>{});
+    else if (live == 3) run_tile(template_int<3>{});
+    else if (live == 2) run_tile(template_int<2>{});
+    else run_tile(template_int<1>{});
+    fixed_acc_settle();
+    int lane_e = lane;   // (opaque: the epilogue's addresses are worked out here, not held through the k-loop)
+    asm volatile("" : "+v"(lane_e));
+    tile_epilogue<MODE, false, kQWaves, TM, TN, false, 0, false, false, kAccBlock0, false, 64>(
+        cp, no_acc, stage_rows, wm * 32, wave_col0, lane_e, nullptr, nullptr, nullptr, live);
+    cp = ld;
+    if (!cp.valid) break;
+    nxt = fetch_tile(next_turn++);
+    copy_row_slots(nxt);
+  }
+}
+
 #if DICE_PERSIST_F8
 // ---------------------------------------------------------------------------
 // fp8 x fp8 pipeline, four waves: e4m3 activations (one fp32 scale per row) times
@@ -2333,6 +2638,14 @@ template <int MODE, bool HAS_BIAS, int BN, bool GATHER, bool W8 = false, bool RE
 __global__ __launch_bounds__(4 * kWave, 1) void gemm_persist_kernel4(PersistBatch batch) {
   gemm_persist64_body<MODE, HAS_BIAS, BN, GATHER, W8, REFILL>(batch);
 }
+// The same with the k-loop in assembly (gemm_persist64_asm_body).  The compiler
+// allocates from v0..v127 only; v128..v255 and every accumulation register
+// belong to the assembly text.
+template <int MODE, int BN, bool GATHER, bool REFILL = false>
+__global__ __launch_bounds__(4 * kWave, 1) __attribute__((amdgpu_num_vgpr(128)))
+void gemm_persist_kernel4a(PersistBatch batch) {
+  gemm_persist64_asm_body<MODE, BN, GATHER, REFILL>(batch);
+}
 
 #if DICE_PERSIST_F8
 // fp8 activations and weights (see gemm_persist_f8_body).
@@ -2523,6 +2836,9 @@ PersistKernel pick64(bool w8, bool refill) {
   if (w8)
     return refill ? gemm_persist_kernel4<MODE, HAS_BIAS, BN, GATHER, true, true>
                   : gemm_persist_kernel4<MODE, HAS_BIAS, BN, GATHER, true, false>;
+  if constexpr (persist64_asm_applies<MODE, HAS_BIAS, BN, GATHER, false>())
+    return refill ? gemm_persist_kernel4a<MODE, BN, GATHER, true> : gemm_persist_kernel4a<MODE, BN, GATHER, false>;
+  else
   return refill ? gemm_persist_kernel4<MODE, HAS_BIAS, BN, GATHER, false, true>
                 : gemm_persist_kernel4<MODE, HAS_BIAS, BN, GATHER, false, false>;
 }
