@@ -49,7 +49,9 @@ CONFIGS = {
 }
 TORCH_DTYPE = {"bf16": torch.bfloat16, "f32": torch.float32}
 # rocprofv3 --pmc summaries of the dominant launch (bytes past the L2 per launch), keyed by (config, variant)
-TRAFFIC_PROFILES = {("c2", "swiglu"): "profiles/layer_c2_bf16_hbm_traffic.txt"}
+TRAFFIC_PROFILES = {("c2", "swiglu"): "profiles/layer_c2_bf16_hbm_traffic.txt",
+                    ("c3", "swiglu"): "profiles/layer_c3_bf16_zipf_kernel_trace_and_mfma.txt",
+                    ("c5", "swiglu"): "profiles/layer_c5_fp8_kernel_trace_and_counters.txt"}
 
 
 def make_block(cfg, variant, dev, layer_idx=0, total_layers=1, para_mode=None, activations="bf16"):
