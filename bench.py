@@ -139,6 +139,23 @@ def time_layer(blk, x, steps, warmup):
     return sec, fc1_ms / steps
 
 
+def time_after_idle(blk, x, calls=64, idle_s=2.0):
+    """Duration (ms) of each of the first `calls` layer calls after `idle_s` seconds without GPU work, from
+    one event per call on torch's current stream.  A run of 20 timed steps behind 5 warm-ups falls into the
+    transient this shows (the board's power management answering a step from idle to full load), a longer run
+    averages over it."""
+    y = torch.empty_like(x)
+    torch.cuda.synchronize()
+    time.sleep(idle_s)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(calls + 1)]
+    ev[0].record()
+    for i in range(calls):
+        blk.run(x, y=y)
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    return [round(ev[i].elapsed_time(ev[i + 1]), 4) for i in range(calls)]
+
+
 def time_stages(blk, x, steps):
     """Mean duration of every launch of the layer in ms, from the library's own
     stage timers: HIP events recorded between the launches of dice_moe_forward
@@ -735,6 +752,8 @@ def main():
     ap.add_argument("--no-caller", action="store_true", help="skip the fused-caller (LayerNorm/modulate + residual) pass")
     ap.add_argument("--no-staleness", action="store_true", help="skip the 50-step conditional-communication loop")
     ap.add_argument("--no-lagged", action="store_true", help="skip the step-lagged (displaced / interweaved) pass")
+    ap.add_argument("--no-after-idle", action="store_true",
+                    help="skip the per-call durations of the first 64 calls after a two-second pause")
     ap.add_argument("--no-sustained", action="store_true",
                     help="skip the sustained pass over eight blocks with distinct weights")
     ap.add_argument("--no-vendor", action="store_true",
@@ -819,6 +838,9 @@ def main():
                 "fp8_launch_frac_of_fp8_peak", "quantiser_gbs"):
         if key in res:
             out[key] = res[key]
+    if not args.no_after_idle and main_cfg == "c2":
+        # (not part of `value`) the first calls after a pause, one duration per call
+        out["ms_per_call_after_2s_idle"] = time_after_idle(blk, x)
     if not args.no_caller:
         out["block_moe_half_ms"] = time_caller(cfg, blk, x, args.steps, args.warmup, (args.fc1_cfg, args.fc2_cfg))
     if not args.no_staleness and main_cfg == "c2":
