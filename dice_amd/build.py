@@ -54,7 +54,7 @@ def _hipcc() -> str:
 # Translation units whose kernels keep their sums in accumulation registers that
 # the compiler does not know about: their device assembly is kept and checked
 # (check_acc_regs.py) before the library is linked.
-ACC_CHECKED = {"grouped_gemm_persist.hip", "grouped_gemm_persist_f16.hip"}
+ACC_CHECKED = {"grouped_gemm_persist.hip", "grouped_gemm_persist_f16.hip", "grouped_gemm_persist_f8.hip"}
 
 
 def _generate_sources() -> None:

@@ -6,7 +6,7 @@ of vector registers it parks values in accumulation registers of its own
 choice, lowest numbers first; a kernel of sixteen blocks owns all 256 and must
 see none of that, a kernel of twelve blocks keeps its sums in a64 .. a255 and
 leaves a0 .. a63 to the compiler.  A kernel whose k-loop is assembly text
-(gemm_persist_kernel4a) also names its register stages, v128 .. v255, in that
+(gemm_persist_kernel4a, gemm_persist_kernel_f8a) also names its register stages, v128 .. v255, in that
 text only: it is compiled with a budget of 128 vector registers and must see
 the compiler neither above v127 nor in any accumulation register.  This script
 reads the device assembly the compiler wrote for a translation unit and fails
@@ -18,14 +18,14 @@ from __future__ import annotations
 import re
 import sys
 
-_KERNEL = re.compile(r"^(_ZN4dice\S*gemm_persist_kernel4a?I\S+):")
+_KERNEL = re.compile(r"^(_ZN4dice\S*gemm_persist_kernel(?:4a?|_f8a)I\S+):")
 _ANY_FN = re.compile(r"^(\S+):\s*(;.*)?$")
 _REG = re.compile(r"\b([av])(\d+)\b|\b([av])\[(\d+):(\d+)\]")
 
 
 def _owned_from(mangled: str):
     """(first accumulation register, first vector register) the assembly owns."""
-    if "gemm_persist_kernel4aI" in mangled:
+    if "gemm_persist_kernel4aI" in mangled or "gemm_persist_kernel_f8aI" in mangled:
         return 0, 128
     # gemm_persist_kernel4<MODE, HAS_BIAS, BN, ...>: ILi<mode>ELb<bias>ELi<BN>E...
     m = re.search(r"gemm_persist_kernel4ILi\d+ELb[01]ELi(\d+)E", mangled)
@@ -72,7 +72,7 @@ def check(asm_path: str) -> int:
             "the compiler placed values of its own in registers that belong to the kernel's assembly "
             f"({len(problems)} instructions), e.g.\n  " + "\n  ".join(problems[:8]))
     if not checked:
-        raise RuntimeError(f"{asm_path}: no gemm_persist_kernel4 instantiation found")
+        raise RuntimeError(f"{asm_path}: no checked kernel found")
     return len(checked)
 
 

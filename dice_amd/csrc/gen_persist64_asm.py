@@ -41,6 +41,9 @@ KINDS = {
     # kind: (TN, copies of B per step, B frag row offsets (rows), acc block 0, B loads that use the second descriptor)
     0: dict(name="fc1 SwiGLU, 256 weight rows", TN=4, CB=8, brow=[0, 32, 128, 160], acc0=0, up_from=4),
     1: dict(name="fc2, 192 weight rows", TN=3, CB=6, brow=[0, 32, 64], acc0=4, up_from=99),
+    # fp8 activations and weights (grouped_gemm_persist_f8.hip): a step is 128 k in two halves of 64 k
+    2: dict(name="fp8 SwiGLU fc1, 256 weight rows", TN=4, CB=8, brow=[0, 32, 128, 160], acc0=0, up_from=4, f8=True),
+    3: dict(name="fp8 GELU fc1 / fc2, 256 weight rows", TN=4, CB=8, brow=[0, 32, 64, 96], acc0=0, up_from=99, f8=True),
 }
 CA = 8            # loads of activation rows per wave per step
 TM = 4
@@ -153,6 +156,96 @@ class Stream:
         c = "0" if first else f"a[{acc}:{acc + 15}]"
         self.emit(f"MFMA a[{acc}:{acc + 15}], v[{w}:{w + 3}], v[{a}:{a + 3}], {c}")
 
+    # ---- fp8 kinds: fragments of 32 bytes per lane (two LDS reads), one set of eight, replaced in place ----
+    def frag_reg8(self, which, idx):
+        return 8 * idx if which == "w" else 32 + 8 * idx
+
+    def read_half8(self, slot, kb, which, idx, t):
+        """16-byte half t of fragment (which, idx) of k-block kb of slot `slot`."""
+        reg = self.frag_reg8(which, idx) + 4 * t
+        if which == "w":
+            off = self.k["brow"][idx] * 128
+            addr = f"%[rb{slot}{kb * 2 + t}]"
+        else:
+            off = idx * 64 * 128
+            addr = f"%[ra{slot}{kb * 2 + t}]"
+        self.emit(f"ds_read_b128 v[{reg}:{reg + 3}], {addr} offset:{off}")
+        self.frag_op[reg] = self.lds_issued
+        self.lds_issued += 1
+
+    def mfma8(self, i, j, first):
+        w, a = self.frag_reg8("w", j), self.frag_reg8("a", i)
+        need = max(self.frag_op.get(r, -1) for r in (w, w + 4, a, a + 4)) + 1
+        self.wait("lgkm", need)
+        acc = 16 * (self.k["acc0"] + i * self.k["TN"] + j)
+        c = "0" if first else f"a[{acc}:{acc + 15}]"
+        self.emit(f"MFMA8 a[{acc}:{acc + 15}], v[{w}:{w + 7}], v[{a}:{a + 7}], {c}")
+
+    def column(self, j, up):
+        rows = range(self.live) if up else range(self.live - 1, -1, -1)
+        return [(i, j) for i in rows]
+
+    def run8(self, prods, first_n, n_block, rslot, rkb, carried, wstage, quarters):
+        """The products `prods` in order, the first first_n of them starting the sums.  The first n_block of them
+        are one k-block; behind the last product of that block that uses a fragment come the two reads that
+        replace it by the fragment of k-block rkb of slot rslot (`carried` = fragments already free when the
+        statement starts); products past n_block use the new fragments.  The quarters' LDS writes and refills
+        are spread over all gaps."""
+        cb = self.k["CB"]
+        mf = len(prods)
+        gaps = [[] for _ in range(mf)]
+        last_w, last_a = {}, {}
+        for m, (i, j) in enumerate(prods[:n_block]):
+            last_w[j] = m
+            last_a[i] = m
+        frees = [(0, f) for f in carried]
+        frees += [(m, ("w", j)) for j, m in last_w.items()]
+        frees += [(m, ("a", i)) for i, m in last_a.items()]
+        for g, (which, idx) in sorted(frees):
+            # (both halves before the first product past the block, which may be the fragment's next user)
+            gaps[min(g, n_block - 1)].append(("r", (which, idx, 0)))
+            gaps[min(g + 1, n_block - 1)].append(("r", (which, idx, 1)))
+        items = [l for q in quarters for l in range(quarter_first(cb, q), quarter_first(cb, q + 1))]
+        for n, l in enumerate(items):
+            gaps[side_slot(n, len(items), mf, 1)].append(("w", l))
+        for n, l in enumerate(items):
+            gaps[side_slot(n, len(items), mf, 3)].append(("l", l))
+        for g in range(mf):
+            i, j = prods[g]
+            self.mfma8(i, j, g < first_n)
+            for kind in ("r", "w", "l"):
+                for k2, x in gaps[g]:
+                    if k2 != kind:
+                        continue
+                    if kind == "r":
+                        self.read_half8(rslot, rkb, x[0], x[1], x[2])
+                    elif kind == "w":
+                        self.write(wstage, x)
+                    else:
+                        self.load(wstage, x)
+
+    def frags8(self):
+        return [("w", j) for j in range(self.k["TN"])] + [("a", i) for i in range(self.live)]
+
+    def abc8(self, slot, var):
+        """First statement of an fp8 step: the 64-k block kb = 0 (weight block by weight block, the row blocks up
+        and down in turn), its fragments replaced in place by those of kb = 1 as they die; then the first weight
+        block of kb = 1 (the rows downwards: the order in which their fragments arrived).  Quarters 1..3 of the
+        next step go from register stage slot^1 to LDS slot slot^1 and are refilled."""
+        first = 4 * self.live if var == 1 else 0
+        half0 = [p for j in range(4) for p in self.column(j, j % 2 == 0)]
+        self.run8(half0 + self.column(0, False), first, len(half0), slot, 1, [], slot ^ 1, (1, 2, 3))
+
+    def d8(self, slot):
+        """Second statement: the barrier, then weight blocks 1..3 of kb = 1, the fragments replaced by those of the
+        next step's kb = 0 (other slot); quarter 0 of the step after next goes to this slot and is refilled."""
+        self.needed.add((self.key, self.site))
+        self.wait("lgkm", self.lds_issued)
+        self.emit("s_barrier")
+        prods = [p for j in (1, 2, 3) for p in self.column(j, j % 2 == 1)]
+        # weight block 0 of kb = 1 had its last product in the first statement
+        self.run8(prods, 0, len(prods), slot ^ 1, 0, [("w", 0)], slot, (0,))
+
     # ---- the pieces ----
     def frag_order(self):
         tn = self.k["TN"]
@@ -193,11 +286,15 @@ class Stream:
                         self.load(wstage, x)
 
     def abc(self, slot, var):
+        if self.k.get("f8"):
+            return self.abc8(slot, var)
         self.block(0, slot, 1, slot ^ 1, 1, var)
         self.block(1, slot, 2, slot ^ 1, 2, 0 if var == 1 else var)
         self.block(0, slot, 3, slot ^ 1, 3, 0 if var == 1 else var)
 
     def d(self, slot, var):
+        if self.k.get("f8"):
+            return self.d8(slot)
         # This wave has read slot `slot` for the last time and finished writing the other one;
         # after the barrier both hold for every wave.  (The barrier opens this statement rather
         # than closing the one before: the scalar bookkeeping between the two then runs while the
@@ -221,6 +318,11 @@ class Stream:
             (self.write if what == "w" else self.load)(stage, l)
 
     def read_first(self):
+        if self.k.get("f8"):
+            for which, idx in self.frags8():
+                for t in (0, 1):
+                    self.read_half8(0, 0, which, idx, t)
+            return
         for which, idx in self.frag_order():
             self.read_frag(0, 0, 0, which, idx)
 
@@ -295,7 +397,7 @@ def generate() -> str:
         out.append(f"template <int KIND, int LIVE>\n__device__ __forceinline__ void p64_{name}(P64_PARAMS) {{")
         first = True
         for (kind, live), pcs in table.items():
-            text = [ln.replace("MFMA", '" DICE_MFMA16 "') for ln in pcs[name]]
+            text = [ln.replace("MFMA8", '" DICE_MFMA8 "').replace("MFMA ", '" DICE_MFMA16 " ') for ln in pcs[name]]
             cond = f"KIND == {kind} && LIVE == {live}"
             out.append(f"  {'if' if first else 'else if'} constexpr ({cond})")
             out.append("    asm volatile(")

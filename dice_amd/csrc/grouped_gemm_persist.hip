@@ -776,31 +776,6 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
 // Taken for 16-bit weights and bias-free tiles of the two shapes generated:
 // KIND 0 = SwiGLU fc1 with gathered rows (256 weight rows), KIND 1 = fc2 with
 // 192 weight rows.
-struct P64Addr {
-  uint32_t wr[2];       // LDS address of this lane's chunk in slot 0 / 1 (writes)
-  uint32_t ra[2][4];    // LDS address of this lane's activation fragment of 16-k block kk in slot 0 / 1
-  uint32_t rb[2][4];    // ... of its weight fragment
-  uint32_t va[8];       // byte offsets of this lane's eight activation rows in the tile being loaded
-  uint32_t vb;          // ... of its first weight row (the others: scalar offsets, P64_PARAMS)
-};
-#define P64_PARAMS                                                                                        \
-  f32x32_t &f0, f32x32_t &f1, const P64Addr &ad, u32x4_t dA, u32x4_t dB0, u32x4_t dB1, uint32_t koff,       \
-      const uint32_t (&sb)[8]
-#define P64_ARGS f0, f1, ad, dA, dB0, dB1, koff, sb
-#define P64_CONSTRAINTS                                                                                         \
-  : "+{v[0:31]}"(f0), "+{v[32:63]}"(f1)                                                                         \
-  : [wr0] "v"(ad.wr[0]), [wr1] "v"(ad.wr[1]), [ra00] "v"(ad.ra[0][0]), [ra01] "v"(ad.ra[0][1]),                 \
-    [ra02] "v"(ad.ra[0][2]), [ra03] "v"(ad.ra[0][3]), [ra10] "v"(ad.ra[1][0]), [ra11] "v"(ad.ra[1][1]),         \
-    [ra12] "v"(ad.ra[1][2]), [ra13] "v"(ad.ra[1][3]), [rb00] "v"(ad.rb[0][0]), [rb01] "v"(ad.rb[0][1]),         \
-    [rb02] "v"(ad.rb[0][2]), [rb03] "v"(ad.rb[0][3]), [rb10] "v"(ad.rb[1][0]), [rb11] "v"(ad.rb[1][1]),         \
-    [rb12] "v"(ad.rb[1][2]), [rb13] "v"(ad.rb[1][3]), [va0] "v"(ad.va[0]), [va1] "v"(ad.va[1]),                 \
-    [va2] "v"(ad.va[2]), [va3] "v"(ad.va[3]), [va4] "v"(ad.va[4]), [va5] "v"(ad.va[5]), [va6] "v"(ad.va[6]),    \
-    [va7] "v"(ad.va[7]), [vb] "v"(ad.vb), [dA] "s"(dA), [dB0] "s"(dB0), [dB1] "s"(dB1), [koff] "s"(koff),       \
-    [sb0] "s"(sb[0]), [sb1] "s"(sb[1]), [sb2] "s"(sb[2]), [sb3] "s"(sb[3]), [sb4] "s"(sb[4]), [sb5] "s"(sb[5]), \
-    [sb6] "s"(sb[6]), [sb7] "s"(sb[7])                                                                          \
-  : "memory"
-typedef float f32x32_t __attribute__((ext_vector_type(32)));
-#include "persist64_asm.inc"
 
 template <int MODE, bool HAS_BIAS, int BN, bool GATHER, bool W8>
 constexpr bool persist64_asm_applies() {
@@ -892,27 +867,13 @@ __device__ __forceinline__ void gemm_persist64_asm_body(const PersistBatch &batc
                            (uint32_t)__builtin_amdgcn_readlane(pk.words, 20);
       const int rows = __builtin_amdgcn_readlane(pk.words, 23);
       if (wave == 0 && ptr != 0) {
-        // Global memory -> LDS without a register in between, as text: a load the
-        // compiler knows of would have it wait for "its only load" with vmcnt(0)
-        // before the next LDS access of its own - which drains the 32 operand
-        // loads the assembly keeps in flight, once per tile.  Rows past the
-        // group's end read as slot 0 (a legal row; their products are never
-        // stored).  M0 holds the LDS address for the instruction and is put back.
+        // (as text, see lds_dma_x4_text; rows past the group's end read as slot 0, a
+        // legal row: their products are never stored)
         const u32x4_t rs = {uni((uint32_t)ptr), uni((uint32_t)(ptr >> 32) & 0xffffu), uni((uint32_t)rows * 4u),
                             kRsrcFlags};
-        const uint32_t dst = uni((uint32_t)(size_t)(lds_byte_t *)lds_row_slots);
         int lane_c = lane;
         asm volatile("" : "+v"(lane_c));
-        const uint32_t voff = (uint32_t)lane_c * 16u;
-        uint32_t keep_m0;
-        asm volatile("s_mov_b32 %[keep], m0\n\t"
-                     "s_mov_b32 m0, %[dst]\n\t"
-                     "s_nop 0\n\t"
-                     "buffer_load_dwordx4 %[voff], %[rs], 0 offen lds\n\t"
-                     "s_mov_b32 m0, %[keep]"
-                     : [keep] "=&s"(keep_m0)
-                     : [dst] "s"(dst), [voff] "v"(voff), [rs] "s"(rs)
-                     : "memory");
+        lds_dma_x4_text(rs, (uint32_t)(size_t)(lds_byte_t *)lds_row_slots, (uint32_t)lane_c * 16u);
       }
     }
   };

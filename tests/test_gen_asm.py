@@ -3,9 +3,11 @@ generator must guarantee whatever its schedule, checked on the text it writes (n
 
 An independent replay of every statement sequence the kernel runs (prologue, then tiles of
 steps) with in-order LDS and vector-memory queues: every MFMA reads fragments whose LDS reads
-have completed under the waits in the text, every LDS write sends a stage register whose load
-has completed, no load refills a stage register before the LDS write that reads it was issued,
-and every register stays inside the plan the build-time checker assumes.
+have completed under the waits in the text AND that hold the k-block, slot and row / weight
+block its accumulator calls for (fragments replaced in place included), every LDS write sends a
+stage register whose load has completed, no load refills a stage register before the LDS write
+that reads it was issued, and every register stays inside the plan the build-time checker
+assumes.
 """
 import importlib.util
 import os
@@ -33,13 +35,29 @@ def _regs(tok):
 class Replay:
     """In-order queues; `done` counts completed operations of each queue."""
 
-    def __init__(self):
+    def __init__(self, kind_desc):
+        self.k = kind_desc
+        self.f8 = bool(kind_desc.get("f8"))
         self.lds_issued = self.lds_done = 0
         self.vm_issued = self.vm_done = 0
-        self.frag_ready = {}      # first register of a fragment -> index of the LDS read filling it
+        self.frag_ready = {}      # first register of a 16-byte fragment part -> index of the LDS read filling it
+        self.frag_tag = {}        # ... -> (operand, slot, address index, byte offset) it was read from
         self.stage_ready = {}     # first register of a stage entry -> index of the load filling it
         self.stage_sent = {}      # first register of a stage entry -> True once its LDS write was issued
         self.mfma = 0
+        self.blocks = []          # (slot, k-block) of every MFMA, in order
+
+    def _operand(self, first_reg, n_parts, operand, block_offset):
+        """The (slot, address indices) the parts of a fragment were read from; checks readiness and offsets."""
+        tags = []
+        for part in range(n_parts):
+            r = first_reg + 4 * part
+            assert r in self.frag_ready, f"fragment v{r} never read"
+            assert self.frag_ready[r] < self.lds_done, f"fragment v{r} still in flight"
+            op, slot, kk, off = self.frag_tag[r]
+            assert op == operand and off == block_offset, (r, self.frag_tag[r], operand, block_offset)
+            tags.append((slot, kk))
+        return tags
 
     def run(self, lines):
         for ln in lines:
@@ -54,19 +72,32 @@ class Replay:
                     self.vm_done = max(self.vm_done, self.vm_issued - int(m.group(2)))
             elif op == "s_barrier":
                 assert self.lds_done == self.lds_issued, "barrier with LDS operations in flight"
-            elif op == "MFMA":
+            elif op in ("MFMA", "MFMA8"):
+                assert (op == "MFMA8") == self.f8
+                parts = 2 if self.f8 else 1
                 (fa, a0, a1), (_, w0, w1), (_, r0, r1) = _regs(args[0]), _regs(args[1]), _regs(args[2])
                 assert fa == "a" and a1 - a0 == 15 and a0 % 16 == 0 and a1 < 256
-                assert w1 - w0 == 3 and r1 - r0 == 3 and w1 < 64 and r1 < 64
+                assert w1 - w0 == 4 * parts - 1 and r1 - r0 == 4 * parts - 1 and w1 < 64 and r1 < 64
                 assert args[3] in ("0", args[0])
-                for f in (w0, r0):
-                    assert f in self.frag_ready, f"fragment v{f} never read"
-                    assert self.frag_ready[f] < self.lds_done, f"{ln}: fragment v{f} still in flight"
+                blk = a0 // 16 - self.k["acc0"]
+                i, j = divmod(blk, self.k["TN"])
+                assert 0 <= i < 4 and 0 <= j < self.k["TN"]
+                tw = self._operand(w0, parts, "b", self.k["brow"][j] * 128)
+                ta = self._operand(r0, parts, "a", i * 64 * 128)
+                assert tw == ta, f"{ln}: operands of different k-blocks {tw} {ta}"
+                if self.f8:      # address index kk = 2 kb + t
+                    assert tw[0][0] == tw[1][0] and tw[0][1] % 2 == 0 and tw[1][1] == tw[0][1] + 1, tw
+                    self.blocks.append((tw[0][0], tw[0][1] // 2))
+                else:
+                    self.blocks.append(tw[0])
                 self.mfma += 1
             elif op == "ds_read_b128":
                 _, d0, d1 = _regs(args[0])
                 assert d1 - d0 == 3 and d1 < 64
+                m = re.fullmatch(r"%\[r([ab])(\d)(\d)\] offset:(\d+)", args[1])
+                assert m, ln
                 self.frag_ready[d0] = self.lds_issued
+                self.frag_tag[d0] = (m.group(1), int(m.group(2)), int(m.group(3)), int(m.group(4)))
                 self.lds_issued += 1
             elif op == "ds_write_b128":
                 _, d0, d1 = _regs(args[1].split(" ")[0])
@@ -86,7 +117,7 @@ class Replay:
                 raise AssertionError(f"unexpected instruction {ln}")
 
 
-@pytest.mark.parametrize("kind", [0, 1])
+@pytest.mark.parametrize("kind", [0, 1, 2, 3])
 @pytest.mark.parametrize("live", [1, 2, 3, 4])
 def test_generated_loop_waits_cover_every_dependence(kind, live):
     gen = _load()
@@ -94,24 +125,34 @@ def test_generated_loop_waits_cover_every_dependence(kind, live):
     tn = gen.KINDS[kind]["TN"]
     assert sorted(pcs) == ["abc_s0_v0", "abc_s0_v1", "abc_s1_v0", "d_s0", "d_s1", "load_q0_stage1",
                            "load_step0", "load_step1", "read_first", "write_q0_stage1", "write_step0"]
-    r = Replay()
+    r = Replay(gen.KINDS[kind])
+    f8 = bool(gen.KINDS[kind].get("f8"))
+    per_step = (2 if f8 else 4) * live * tn    # products per step: two k-blocks of 64 (fp8) or four of 16
     for name in ("load_step0", "load_step1", "write_step0", "load_step0", "write_q0_stage1", "load_q0_stage1"):
         r.run(pcs[name])
     r.lds_done = r.lds_issued                      # s_waitcnt lgkmcnt(0) + barrier in the kernel's own code
     for tile_steps in (6, 18, 8):                  # (even step counts of at least six, as the launcher admits)
         r.run(pcs["read_first"])
         before = r.mfma
+        r.blocks = []
         for s in range(tile_steps):
             slot = s & 1
             r.run(pcs[f"abc_s{slot}_v{1 if s == 0 else 0}"])
             r.run(pcs[f"d_s{slot}"])
-        assert r.mfma - before == tile_steps * 4 * live * tn
+        assert r.mfma - before == tile_steps * per_step
+        # the k-blocks in order: every step its slot, its blocks one after the other, each live * tn products
+        n_kb = 2 if f8 else 4
+        want = [(s & 1, kb) for s in range(tile_steps) for kb in range(n_kb) for _ in range(live * tn)]
+        assert r.blocks == want
         r.lds_done = r.lds_issued                  # the epilogue drains the LDS queue; vector loads stay in flight
         r.vm_issued += 24                          # ... and issues stores of its own: waits only get stricter
     # the first step of a tile starts the sums, every later one adds to them
     first = [ln for ln in pcs["abc_s0_v1"] if ln.startswith("MFMA")]
     assert all(ln.endswith(", 0") for ln in first[:live * tn])
     assert not any(ln.endswith(", 0") for ln in first[live * tn:])
+    # every block of sums is started exactly once per tile
+    started = sorted(ln.split(",")[0] for ln in first[:live * tn])
+    assert len(set(started)) == live * tn
     assert not any(ln.endswith(", 0") for ln in pcs["abc_s0_v0"] if ln.startswith("MFMA"))
 
 
