@@ -163,5 +163,8 @@ def test_generated_text_names_only_planned_registers():
     for m in re.finditer(r"\bv\[(\d+):(\d+)\]", text):
         lo, hi = int(m.group(1)), int(m.group(2))
         assert hi < 64 or lo >= 128, m.group(0)     # fragments or stages, never the compiler's v64..v127
-    for word in ("s_store", "s_buffer_store", "s_atomic", "s_dcache", "v_pk_"):
-        assert word not in text
+    # every instruction of the text is one of these (the replay above refuses anything else, too)
+    allowed = {"s_waitcnt", "s_barrier", "ds_read_b128", "ds_write_b128", "buffer_load_dwordx4", "DICE_MFMA16",
+               "DICE_MFMA8"}
+    for m in re.finditer(r'^\s*"(?:" )?([A-Za-z_0-9]+)', text, re.M):
+        assert m.group(1) in allowed, m.group(0)
