@@ -41,6 +41,7 @@ KINDS = {
     # kind: (TN, copies of B per step, B frag row offsets (rows), acc block 0, B loads that use the second descriptor)
     0: dict(name="fc1 SwiGLU, 256 weight rows", TN=4, CB=8, brow=[0, 32, 128, 160], acc0=0, up_from=4),
     1: dict(name="fc2, 192 weight rows", TN=3, CB=6, brow=[0, 32, 64], acc0=4, up_from=99),
+    4: dict(name="fc2, 128 weight rows", TN=2, CB=4, brow=[0, 32], acc0=8, up_from=99),
     # fp8 activations and weights (grouped_gemm_persist_f8.hip): a step is 128 k in two halves of 64 k
     2: dict(name="fp8 SwiGLU fc1, 256 weight rows", TN=4, CB=8, brow=[0, 32, 128, 160], acc0=0, up_from=4, f8=True),
     3: dict(name="fp8 GELU fc1 / fc2, 256 weight rows", TN=4, CB=8, brow=[0, 32, 64, 96], acc0=0, up_from=99, f8=True),

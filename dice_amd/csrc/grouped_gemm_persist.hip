@@ -779,18 +779,28 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
 
 template <int MODE, bool HAS_BIAS, int BN, bool GATHER, bool W8>
 constexpr bool persist64_asm_applies() {
-  return !W8 && !HAS_BIAS && ((MODE == kFc1Swiglu && BN == 256 && GATHER) || (MODE == kFc2 && BN == 192));
+  return !W8 && ((!HAS_BIAS && MODE == kFc1Swiglu && BN == 256 && GATHER) || (!HAS_BIAS && MODE == kFc2 && BN == 192) ||
+                 (MODE == kFc2 && BN == 128));
 }
 
-template <int MODE, int BN, bool GATHER, bool REFILL>
+// HAS_BIAS (128-row weight tiles only: the wider tiles' staging rows leave no room): the
+// tile's bias is staged in LDS a tile ahead, as the fp8 kernel does, and added in the epilogue.
+template <int MODE, int BN, bool GATHER, bool REFILL, bool HAS_BIAS = false>
 __device__ __forceinline__ void gemm_persist64_asm_body(const PersistBatch &batch) {
   constexpr bool SWIGLU = MODE == kFc1Swiglu;
-  constexpr int KIND = SWIGLU ? 0 : 1;
+  constexpr int KIND = SWIGLU ? 0 : BN == 192 ? 1 : 4;
+  static_assert(SWIGLU ? BN == 256 : (BN == 192 || BN == 128), "the shapes the generator writes");
   constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
   constexpr int WTN = BN / 2, TM = 4, TN = WTN / 32;
   constexpr int kCopiesA = kPBM / 8 / kQWaves, kCopiesB = BN / 8 / kQWaves;
   constexpr int kAccBlock0 = 16 - TM * TN;
-  using Epi = EpiGeom<MODE, kQWaves, TM, TN, 0>;
+  static_assert(!HAS_BIAS || (BN == 128 && !GATHER), "no LDS for a staged bias beside wider tiles' staging rows");
+  constexpr int kTableBytes = kTableTurns * kTileWords * 4, kRowSlotBytes = kPBM * 4;
+  // (three bias buffers: the epilogue of a tile reads its bias while the first wave, a little ahead, may already
+  // stage that of the tile after the next)
+  constexpr int kBiasBufFloats = 256, kBiasBytes = HAS_BIAS ? 3 * kBiasBufFloats * 4 : 0;
+  constexpr int kEpiReserve = kTableBytes + (GATHER ? kRowSlotBytes : 0) + kBiasBytes;
+  using Epi = EpiGeom<MODE, kQWaves, TM, TN, HAS_BIAS ? kEpiReserve : 0>;
   typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
 
   __shared__ __attribute__((aligned(1024))) unsigned char lds_slot0[kQSlotBytes];
@@ -801,11 +811,10 @@ __device__ __forceinline__ void gemm_persist64_asm_body(const PersistBatch &batc
   const int wm = wave >> 1, wn = wave & 1;
   fixed_acc_declare();
 
-  constexpr int kTableBytes = kTableTurns * kTileWords * 4, kRowSlotBytes = kPBM * 4;
-  static_assert(kQWaves * Epi::WAVE_BYTES + kTableBytes + (GATHER ? kRowSlotBytes : 0) <= kPStageArea,
-                "no room for the tile table");
+  static_assert(kQWaves * Epi::WAVE_BYTES + kEpiReserve <= kPStageArea, "no room for the tile table");
   uint32_t *const tile_table = reinterpret_cast<uint32_t *>(lds_stage + kPStageArea - kTableBytes);
   int32_t *const lds_row_slots = reinterpret_cast<int32_t *>(lds_stage + kPStageArea - kTableBytes - kRowSlotBytes);
+  float *const lds_bias = reinterpret_cast<float *>(lds_stage + kPStageArea - kEpiReserve);
   if (wave == 0) {
     TileWalker<BN_OUT> walk(batch, lane);
     walk.build_table(batch, lane, kQBK, tile_table, false);
@@ -877,6 +886,22 @@ __device__ __forceinline__ void gemm_persist64_asm_body(const PersistBatch &batc
       }
     }
   };
+  auto copy_bias = [&](const PackedTile &pk, int buf) {
+    if constexpr (HAS_BIAS) {
+      const uint64_t ptr = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane(pk.words, 9) << 32) |
+                           (uint32_t)__builtin_amdgcn_readlane(pk.words, 8);
+      const int n0 = __builtin_amdgcn_readlane(pk.words, 16), n = __builtin_amdgcn_readlane(pk.words, 17);
+      if (wave == 0) {
+        // (a problem without a bias gets zeros: a descriptor that covers no bytes)
+        const uint64_t src = ptr != 0 ? ptr + (uint64_t)n0 * 4 : (uint64_t)batch.prob[0].w;
+        const u32x4_t rs = {uni((uint32_t)src), uni((uint32_t)(src >> 32) & 0xffffu),
+                            uni(ptr != 0 ? (uint32_t)(n - n0) * 4u : 0u), kRsrcFlags};
+        int lane_c = lane;
+        asm volatile("" : "+v"(lane_c));
+        lds_dma_x4_text(rs, (uint32_t)(size_t)(lds_byte_t *)(lds_bias + buf * kBiasBufFloats), (uint32_t)lane_c * 16u);
+      }
+    }
+  };
   // Descriptors of the tile being loaded, as plain register values (base, extent, flags).
   u32x4_t dA, dB0, dB1;
   auto set_copy_offsets = [&](const Tile &t) {
@@ -917,8 +942,10 @@ __device__ __forceinline__ void gemm_persist64_asm_body(const PersistBatch &batc
   PackedTile nxt = fetch_tile(next_turn++);
   Tile ld = unpack_tile(nxt);
   if (!ld.valid) return;
-  if constexpr (GATHER) {
+  int bias_buf = 0;   // buffer of the bias of the tile being multiplied
+  if constexpr (GATHER || HAS_BIAS) {
     copy_row_slots(nxt);
+    copy_bias(nxt, 0);
     pwait_vmcnt<0>();
     phase_barrier();
   }
@@ -931,6 +958,7 @@ __device__ __forceinline__ void gemm_persist64_asm_body(const PersistBatch &batc
     phase_barrier();
     copy_row_slots(nxt);
   }
+  copy_bias(nxt, 1);
   uint32_t koff = 0;
 #pragma unroll
   for (int i = 0; i < 8; ++i) sb[i] = sb_row[i];
@@ -1005,12 +1033,16 @@ __device__ __forceinline__ void gemm_persist64_asm_body(const PersistBatch &batc
     fixed_acc_settle();
     int lane_e = lane;   // (opaque: the epilogue's addresses are worked out here, not held through the k-loop)
     asm volatile("" : "+v"(lane_e));
-    tile_epilogue<MODE, false, kQWaves, TM, TN, false, 0, false, false, kAccBlock0, false, 64>(
-        cp, no_acc, stage_rows, wm * 32, wave_col0, lane_e, nullptr, nullptr, nullptr, live);
+    tile_epilogue<MODE, false, kQWaves, TM, TN, false, HAS_BIAS ? kEpiReserve : 0, false, HAS_BIAS, kAccBlock0, false, 64>(
+        cp, no_acc, stage_rows, wm * 32, wave_col0, lane_e, nullptr, nullptr, lds_bias + bias_buf * kBiasBufFloats, live);
     cp = ld;
     if (!cp.valid) break;
     nxt = fetch_tile(next_turn++);
     copy_row_slots(nxt);
+    // (the buffer written here was last read a whole tile ago; the copy is older than every load of the
+    // coming steps, whose waits therefore cover it)
+    bias_buf = bias_buf == 2 ? 0 : bias_buf + 1;          // the tile multiplied next
+    copy_bias(nxt, bias_buf == 2 ? 0 : bias_buf + 1);     // the one after it
   }
 }
 
@@ -1029,10 +1061,10 @@ __global__ __launch_bounds__(4 * kWave, 1) void gemm_persist_kernel4(PersistBatc
 // The same with the k-loop in assembly (gemm_persist64_asm_body).  The compiler
 // allocates from v0..v127 only; v128..v255 and every accumulation register
 // belong to the assembly text.
-template <int MODE, int BN, bool GATHER, bool REFILL = false>
+template <int MODE, int BN, bool GATHER, bool REFILL = false, bool HAS_BIAS = false>
 __global__ __launch_bounds__(4 * kWave, 1) __attribute__((amdgpu_num_vgpr(128)))
 void gemm_persist_kernel4a(PersistBatch batch) {
-  gemm_persist64_asm_body<MODE, BN, GATHER, REFILL>(batch);
+  gemm_persist64_asm_body<MODE, BN, GATHER, REFILL, HAS_BIAS>(batch);
 }
 
 }  // namespace
@@ -1041,6 +1073,7 @@ void gemm_persist_kernel4a(PersistBatch batch) {
 extern int g_persist_waves;
 int persist_variant(const PersistBatch &b, int mode);
 bool persist_fits_table(const PersistBatch &b, int mode);
+bool persist_fits_table_slim(const PersistBatch &b, int mode);
 int persist_cu_count();
 #define DICE_PERSIST_LAUNCH launch_grouped_gemm_persist_f16
 namespace {
@@ -1124,6 +1157,10 @@ bool persist64_ok(const PersistBatch &b, int mode) {
 }  // namespace
 int persist_cu_count() { return cu_count(); }
 bool persist_fits_table(const PersistBatch &b, int mode) { return persist64_fits_table(b, mode); }
+// ... with 128-row weight tiles (at most twice the tiles of the bound's widths)
+bool persist_fits_table_slim(const PersistBatch &b, int mode) {
+  return 2 * persist64_turn_bound(b, mode, cu_count() / kNumXcd) <= kTableTurns;
+}
 // 0: neither pipeline takes the launch; 4 / 8: the waves of the one that does.
 int persist_variant(const PersistBatch &b, int mode) {
   if (!persist_common_ok(b, mode)) return 0;
@@ -1201,6 +1238,27 @@ int DICE_PERSIST_LAUNCH(const PersistBatch &b, int mode, hipStream_t s) {
     const int64_t m256 = persist_plan(b, kPBN, grid, mode == kFc2).makespan;
     if (m256 * 10 <= m192 * 7) narrow = false;
   }
+  // 128-row weight tiles (fc2, 16-bit weights: the kernel with the generated k-loop).  A step of
+  // such a tile takes about 0.75 of a 192-row tile's (two thirds of the products, 12 % more time per product:
+  // the wave tile is 128 x 64 and reads 6 fragments for 8 products instead of 7 for 12), so they pay where
+  // the finer grain shortens the longest workgroup by more than that: small batches, whose few long tiles
+  // otherwise round up to a whole turn.  Tuning hook fc2 = 54 / 55: always / never.
+  bool slim = mode == kFc2 && waves == 4 && !w8 && persist_slim_choice() >= 0 &&
+              persist_fits_table_slim(b, mode);
+  for (int i = 0; i < b.n_problems; ++i) slim = slim && b.prob[i].n % 128 == 0;
+  // (a single-problem launch with partial-tile slots cuts its last turn along k instead: the better remedy there)
+  if (b.n_problems == 1 && b.split_ws != nullptr) slim = false;
+  // (a biased 256-row tile starts its sums from the bias, a 128-row tile adds it behind them: the last bit could
+  // differ, and with it the result between batch sizes that the model below sends different ways)
+  if (has_bias && !narrow) slim = false;
+  if (slim && persist_slim_choice() == 0) {
+    const int64_t m128 = persist_plan(b, 128, grid, true).makespan;
+    const int64_t other = persist_plan(b, narrow ? 192 : kPBN, grid, true).makespan;
+    // (time per step in units of a 192-row tile's: 128 rows 0.75, 256 rows 1.25)
+    slim = m128 * 75 * 100 <= other * (narrow ? 100 : 125) * 93;
+  }
+  if (slim) narrow = false;
+  const int width = mode == kFc1Swiglu ? kPBN / 2 : slim ? 128 : narrow ? 192 : kPBN;
   if (waves == 4) {
     const bool refill = !persist_fits_table(b, mode);
     if (mode == kFc1Swiglu)
@@ -1209,6 +1267,8 @@ int DICE_PERSIST_LAUNCH(const PersistBatch &b, int mode, hipStream_t s) {
       kern = has_bias ? pick64<kFc1Gelu, true, 192, false>(w8, refill) : pick64<kFc1Gelu, false, 192, false>(w8, refill);
     else if (mode == kFc1Gelu)
       kern = has_bias ? pick64<kFc1Gelu, true, 256, false>(w8, refill) : pick64<kFc1Gelu, false, 256, false>(w8, refill);
+    else if (slim)
+      kern = has_bias ? gemm_persist_kernel4a<kFc2, 128, false, false, true> : gemm_persist_kernel4a<kFc2, 128, false, false>;
     else if (narrow)
       kern = has_bias ? pick64<kFc2, true, 192, false>(w8, refill) : pick64<kFc2, false, 192, false>(w8, refill);
     else
@@ -1234,14 +1294,14 @@ int DICE_PERSIST_LAUNCH(const PersistBatch &b, int mode, hipStream_t s) {
   }
   PersistBatch launch = b;
   launch.band_tiles = persist_band_tiles(mode);
-  const PersistPlan plan = persist_plan(b, mode == kFc1Swiglu ? kPBN / 2 : narrow ? 192 : kPBN, grid, mode == kFc2);
+  const PersistPlan plan = persist_plan(b, width, grid, mode == kFc2);
   if (plan.longest_first)
     std::stable_sort(launch.prob, launch.prob + launch.n_problems,
                      [](const PersistProblem &x, const PersistProblem &y) { return x.k > y.k; });
   launch.xcd_split = plan.xcd_split;
   // (a last turn cut along k: the plain epilogue is linear in k; the 32-k kernel
   // does not read its tiles from the table that describes the pieces)
-  if (mode != kFc2 || waves != 4 || b.n_problems != 1 || grid / kNumXcd < 2 || grid > kPersistSplitSlots ||
+  if (mode != kFc2 || waves != 4 || slim || b.n_problems != 1 || grid / kNumXcd < 2 || grid > kPersistSplitSlots ||
       !split_may_apply(b, grid, narrow ? 192 : kPBN))
     launch.split_ws = nullptr;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(waves * kWave), dyn_lds, s, launch);

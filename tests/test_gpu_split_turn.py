@@ -189,3 +189,47 @@ def test_small_batch_shared_fc2_in_its_own_launch(dev, variant, n_shared, N):
     check_rows(by_rule.view(-1, D)[ok], want.view(-1, D)[ok], BF16_TOL, "separate launches vs oracle")
     check_rows(outs[52].view(-1, D)[ok], want.view(-1, D)[ok], BF16_TOL, "joint launch vs oracle")
     check_rows(by_rule.view(-1, D), outs[52].view(-1, D), BF16_TOL / 2, "separate vs joint launch")
+
+
+def _slim_and_not(blk, x):
+    """The block's output with the fc2 launches on 128-row weight tiles wherever they can
+    take them (tuning hook fc2 = 54), then with such tiles ruled out (55)."""
+    from dice_amd import lib
+    try:
+        lib.load().dice_set_gemm_config(0, 54)
+        slim = blk(x).clone()
+        lib.load().dice_set_gemm_config(0, 55)
+        wide = blk(x).clone()
+    finally:
+        lib.load().dice_set_gemm_config(0, 0)
+    return slim.cpu(), wide.cpu()
+
+
+@pytest.mark.parametrize("variant,D,ratio,E,n_shared,N,dtype", [
+    ("swiglu", 1152, 4, 8, 2, 1536, torch.bfloat16),      # the reference block at a mid batch: what the model picks them for
+    ("swiglu", 1152, 4, 8, 2, 1000, torch.bfloat16),      # ragged groups, short last tiles of every number of live blocks
+    ("gelu_tanh", 1152, 4, 8, 8, 2048, torch.bfloat16),   # config-literal: biased, shared tiles twice as long (bias staged in LDS)
+    ("gelu_tanh", 768, 2, 4, 2, 1300, torch.bfloat16),
+    ("swiglu", 1024, 2, 4, 2, 1280, torch.float16),       # the fp16 build; 256 | n: against the 256-row tiles
+    ("gelu_tanh", 1152, 2, 8, 2, 1111, torch.float16),
+])
+def test_fc2_on_128_row_weight_tiles(dev, variant, D, ratio, E, n_shared, N, dtype):
+    """fc2 of a joint launch in 128-row weight tiles (the kernel with the generated k-loop,
+    wave tile 128 x 64): the same sums in the same order as on the wider tiles, so the
+    outputs must be identical bit for bit, and meet the oracle."""
+    p = O.make_block_params(D, E, 2, ratio, n_shared, seed=51, dtype=dtype, variant=variant)
+    if variant == "gelu_tanh":
+        _bias_params(p, 52, dtype)
+    x = torch.randn(1, N, D, generator=_gen(53)).to(dtype)
+    blk = block_from_params(p, D, variant, dtype, dev)
+    slim, wide = _slim_and_not(blk, x.to(dev))
+    want, _, _, logits = O.sparse_moe_block_forward(p, x)
+    ok = ~O.gate_tie_rows(logits, 2).view(-1)
+    tol = BF16_TOL if dtype == torch.bfloat16 else F16_TOL
+    check_rows(slim.view(-1, D)[ok], want.view(-1, D)[ok], tol, "128-row tiles vs oracle")
+    # (biased launches whose other choice is the 256-row tile, which starts its sums from the bias, never take
+    # them: the parameter with D = 768 checks that the hook leaves those alone)
+    assert torch.equal(slim, wide), "128-row weight tiles changed the result"
+    # (and the default choice is one of the two)
+    dflt = blk(x.to(dev)).cpu()
+    assert torch.equal(dflt, wide) or torch.equal(dflt, slim)
