@@ -26,6 +26,15 @@ tile.  The second statement opens with the workgroup barrier; block D then
 reads the first fragments of step s + 1, writes quarter 0 of stage S (step
 s + 2) to slot S and refills it with quarter 0 of step s + 4.
 
+Kinds 0, 1, 4 are the 16-bit shapes (SwiGLU fc1 on 256 weight rows, fc2 on 192
+and on 128).  Kinds 2 and 3 are the kernel for fp8 activations and weights
+(grouped_gemm_persist_f8.hip): the same stages, slots and quarters, but a step
+is 128 k in two k-blocks of 64, a fragment is 32 bytes per lane (two LDS reads)
+and there is one set of eight fragments in v[0:63] (weight block j at 8 j, row
+block i at 32 + 8 i), each replaced in place by the next k-block's as soon as
+its last product has been issued; the first statement of a step is k-block 0
+and the first weight block of k-block 1, the second the barrier and the rest.
+
 The script simulates the instruction stream of the prologue and a few steps,
 finds for every instruction the memory operations it depends on, and emits
 ``s_waitcnt`` with the exact number of younger operations that may still be
