@@ -115,6 +115,9 @@ def _packed(p, variant, dev):
     (512, 4, 8, [0, 1, 700, 0, 257, 3, 1086, 1]),          # fc1 too short (k = 512): refused, see below
     (1024, 2, 8, [0, 1, 700, 0, 257, 3, 1086, 1]),         # empty, one-row and ragged groups
     (2048, 4, 16, None),                                   # DiT-G width
+    # a group's last tile multiplies only its live 64-row blocks: every residue around the block edges
+    (768, 2, 16, [63, 64, 65, 127, 128, 129, 191, 192, 193, 255, 256, 257, 320, 0, 1, 7]),
+    (1024, 2, 8, [256 + 63, 256 + 64, 256 + 65, 512 + 128, 512 + 129, 256 + 191, 256 + 193, 513]),
 ])
 def test_mlp_a8_matches_oracle(dev, variant, D, ratio, E, counts):
     """``dice_grouped_mlp_a8`` (rows gathered through the permutation by the
@@ -122,7 +125,8 @@ def test_mlp_a8_matches_oracle(dev, variant, D, ratio, E, counts):
     row; ``h`` after stage 1 as well."""
     from dice_amd import ops
     from dice_amd.lib import DiceError
-    N = 1024
+    N = 1024 if counts is None else sum(counts) // 2
+    assert counts is None or sum(counts) == 2 * N
     g = _gen(77 + D)
     p = O.make_block_params(D, E, 2, ratio, n_shared=0, seed=8, dtype=torch.bfloat16, variant=variant)
     if variant == "gelu_tanh":

@@ -317,6 +317,24 @@ def test_mlp_bf16_persistent_kernels(dev, variant, cfg):
     _check_mlp_persistent(dev, 512, 512, 8, 2, variant, cfg, counts=[1024, 0, 0, 0, 0, 0, 0, 0])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mlp_live_row_blocks_of_a_last_tile(dev, dtype):
+    """The kernels with the generated k-loop multiply only the live 64-row blocks of a
+    group's last tile (and the two waves that share a tile's columns take alternate
+    32-row blocks): group heights at every residue around the block edges, through
+    fc1 with gathered rows and fc2 on 192-, 256- and 128-row weight tiles."""
+    edges = [256 + 63, 256 + 64, 256 + 65, 512 + 127, 512 + 128, 512 + 129, 256 + 191, 256 + 193]
+    tol = BF16_TOL if dtype == torch.bfloat16 else F16_TOL
+    n = sum(edges)
+    assert n % 2 == 0
+    for fc2_cfg in (0, 54):     # 54: fc2 on 128-row weight tiles wherever a launch can take them
+        _check_mlp(dev, n // 2, 1152, 8, 4, dtype, "swiglu", counts=edges, cfg=(0, fc2_cfg), tol=tol)
+    _check_mlp(dev, n // 2, 1024, 8, 2, dtype, "swiglu", counts=edges, tol=tol)
+    small = [1, 63, 64, 65, 191, 192, 193, 255, 256, 257, 0, 511, 512, 513, 640, 33]
+    assert sum(small) % 2 == 0
+    _check_mlp(dev, sum(small) // 2, 1152, 16, 2, dtype, "swiglu", counts=small, cfg=(21, 21), tol=tol)
+
+
 @pytest.mark.parametrize("cfg", [0, 21])   # 0: groups of few rows take the 64-row tiles; 21: they stay on the persistent kernels
 @pytest.mark.parametrize("variant", ["swiglu", "gelu_tanh"])
 def test_mlp_few_rows_per_group(dev, variant, cfg):
