@@ -168,3 +168,48 @@ def test_generated_text_names_only_planned_registers():
                "DICE_MFMA8"}
     for m in re.finditer(r'^\s*"(?:" )?([A-Za-z_0-9]+)', text, re.M):
         assert m.group(1) in allowed, m.group(0)
+
+
+def _fake_asm(kernel, lines):
+    return "\n".join([f"{kernel}:", *lines, "\ts_endpgm", ""])
+
+
+def test_register_check_flags_compiler_code_in_the_assemblys_registers(tmp_path):
+    """dice_amd/check_acc_regs.py on synthetic device assembly: compiler-generated instructions
+    (outside the inline-assembly markers) must stay out of the registers the kernels' assembly
+    owns; the same instructions inside the markers are the assembly's own."""
+    from dice_amd.check_acc_regs import check
+    k4_256 = "_ZN4dice12_GLOBAL__N_120gemm_persist_kernel4ILi0ELb0ELi256ELb1ELb0ELb0EEEvNS_12PersistBatchE"
+    k4_192 = "_ZN4dice12_GLOBAL__N_120gemm_persist_kernel4ILi2ELb1ELi192ELb0ELb0ELb0EEEvNS_12PersistBatchE"
+    k4a = "_ZN4dice12_GLOBAL__N_121gemm_persist_kernel4aILi0ELi256ELb1ELb0ELb0EEEvNS_12PersistBatchE"
+    kf8 = "_ZN4dice12_GLOBAL__N_123gemm_persist_kernel_f8aILi0ELb0ELb0EEEvNS_12PersistBatchE"
+    inside = ["\t;;#ASMSTART", "\tv_mfma_f32_32x32x16_bf16 a[240:255], v[0:3], v[16:19], a[240:255]",
+              "\tbuffer_load_dwordx4 v[252:255], v70, s[8:11], s72 offen", "\t;;#ASMEND"]
+    ok = {
+        k4_256: inside + ["\tv_add_u32_e32 v200, 4, v200"],                 # all vector registers are the compiler's here
+        k4_192: inside + ["\tv_accvgpr_write_b32 a63, v9"],                 # twelve-block tiles leave a0..a63 to the compiler
+        k4a: inside + ["\tv_add_u32_e32 v127, 4, v64", "\tds_read_b128 v[100:103], v90"],
+        kf8: inside + ["\tv_lshlrev_b32_e32 v5, 7, v95"],
+    }
+    bad = {
+        k4_256: ["\tv_accvgpr_write_b32 a3, v9"],
+        k4_192: ["\tv_accvgpr_read_b32 v9, a64"],
+        k4a: ["\tv_mov_b32_e32 v128, v5"],
+        kf8: ["\tv_accvgpr_write_b32 a0, v5"],
+    }
+    path = tmp_path / "ok.s"
+    path.write_text("".join(_fake_asm(k, v) for k, v in ok.items()))
+    assert check(str(path)) == 4
+    for kernel, extra in bad.items():
+        path = tmp_path / "bad.s"
+        path.write_text(_fake_asm(kernel, ok[kernel] + extra))
+        with pytest.raises(RuntimeError, match="registers that belong to the kernel's assembly"):
+            check(str(path))
+    # a tuple that only reaches into the owned range counts too
+    path.write_text(_fake_asm(k4a, ["\tds_read_b128 v[126:129], v90"]))
+    with pytest.raises(RuntimeError):
+        check(str(path))
+    # a translation unit without any checked kernel is an error of the build, not a pass
+    path.write_text("_Z5otherv:\n\ts_endpgm\n")
+    with pytest.raises(RuntimeError, match="no checked kernel"):
+        check(str(path))
