@@ -780,27 +780,29 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
 template <int MODE, bool HAS_BIAS, int BN, bool GATHER, bool W8>
 constexpr bool persist64_asm_applies() {
   return !W8 && ((!HAS_BIAS && MODE == kFc1Swiglu && BN == 256 && GATHER) || (!HAS_BIAS && MODE == kFc2 && BN == 192) ||
-                 (MODE == kFc2 && BN == 128));
+                 (MODE == kFc2 && BN == 128) || (MODE == kFc1Gelu && BN == 256));
 }
 
-// HAS_BIAS (128-row weight tiles only: the wider tiles' staging rows leave no room): the
-// tile's bias is staged in LDS a tile ahead, as the fp8 kernel does, and added in the epilogue.
+// HAS_BIAS (fc2 on 128-row weight tiles and GELU fc1, whose staging rows leave room for it):
+// the tile's bias is staged in LDS a tile ahead, as the fp8 kernel does, and added in the epilogue.
 template <int MODE, int BN, bool GATHER, bool REFILL, bool HAS_BIAS = false>
 __device__ __forceinline__ void gemm_persist64_asm_body(const PersistBatch &batch) {
   constexpr bool SWIGLU = MODE == kFc1Swiglu;
-  constexpr int KIND = SWIGLU ? 0 : BN == 192 ? 1 : 4;
-  static_assert(SWIGLU ? BN == 256 : (BN == 192 || BN == 128), "the shapes the generator writes");
+  constexpr int KIND = SWIGLU ? 0 : MODE == kFc1Gelu ? 5 : BN == 192 ? 1 : 4;
+  static_assert(SWIGLU || MODE == kFc1Gelu ? BN == 256 : (BN == 192 || BN == 128), "the shapes the generator writes");
   constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
   constexpr int WTN = BN / 2, TM = 4, TN = WTN / 32;
   constexpr int kCopiesA = kPBM / 8 / kQWaves, kCopiesB = BN / 8 / kQWaves;
   constexpr int kAccBlock0 = 16 - TM * TN;
-  static_assert(!HAS_BIAS || (BN == 128 && !GATHER), "no LDS for a staged bias beside wider tiles' staging rows");
+  static_assert(!HAS_BIAS || (BN == 128 && !GATHER) || MODE == kFc1Gelu, "no LDS for a staged bias beside these staging rows");
   constexpr int kTableBytes = kTableTurns * kTileWords * 4, kRowSlotBytes = kPBM * 4;
   // (three bias buffers: the epilogue of a tile reads its bias while the first wave, a little ahead, may already
   // stage that of the tile after the next)
   constexpr int kBiasBufFloats = 256, kBiasBytes = HAS_BIAS ? 3 * kBiasBufFloats * 4 : 0;
   constexpr int kEpiReserve = kTableBytes + (GATHER ? kRowSlotBytes : 0) + kBiasBytes;
-  using Epi = EpiGeom<MODE, kQWaves, TM, TN, HAS_BIAS ? kEpiReserve : 0>;
+  // (what the epilogue's staging rows must leave free: passed on where it decides the height of a band)
+  constexpr int kReserveArg = HAS_BIAS || MODE == kFc1Gelu ? kEpiReserve : 0;
+  using Epi = EpiGeom<MODE, kQWaves, TM, TN, kReserveArg>;
   typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
 
   __shared__ __attribute__((aligned(1024))) unsigned char lds_slot0[kQSlotBytes];
@@ -1033,7 +1035,7 @@ __device__ __forceinline__ void gemm_persist64_asm_body(const PersistBatch &batc
     fixed_acc_settle();
     int lane_e = lane;   // (opaque: the epilogue's addresses are worked out here, not held through the k-loop)
     asm volatile("" : "+v"(lane_e));
-    tile_epilogue<MODE, false, kQWaves, TM, TN, false, HAS_BIAS ? kEpiReserve : 0, false, HAS_BIAS, kAccBlock0, false, 64>(
+    tile_epilogue<MODE, false, kQWaves, TM, TN, false, kReserveArg, false, HAS_BIAS, kAccBlock0, false, 64>(
         cp, no_acc, stage_rows, wm * 32, wave_col0, lane_e, nullptr, nullptr, lds_bias + bias_buf * kBiasBufFloats, live);
     cp = ld;
     if (!cp.valid) break;
@@ -1143,9 +1145,13 @@ bool persist64_ok(const PersistBatch &b, int mode) {
     if (p.a_scale) return false;  // fp8 activations: the kernel of the fp8 compilation unit
     if (p.k < kQBK * kQMinSteps) return false;
     if (p.w_scale && b.n_problems != 1) return false;  // fp8 weights: single-problem launches
-    if (p.a_rows) {  // gathered activation rows: SwiGLU instantiation only (the GELU one would
-                     // spill, and measures no faster than a gathered copy plus the plain kernel)
-      if (mode != kFc1Swiglu) return false;
+    if (p.a_rows) {  // gathered activation rows: the fc1 kernels with the generated k-loop (SwiGLU, and GELU on
+                     // 256-row tiles of 16-bit weights; left to the compiler the GELU instantiation spilled)
+      // (... and launches that fit the tile table: with the table's rewriting as well the instantiation runs out
+      // of scalar registers, and the build check refuses where the compiler then parks them)
+      if (mode == kFc2 || (mode == kFc1Gelu && (p.w_scale || (p.n % 192 == 0 && p.n % 256 != 0) ||
+                                                 !persist64_fits_table(b, mode))))
+        return false;
       if (p.a_div < 1 || p.a_div > 16 || (int64_t)p.a_src_rows * p.a_div >= (1ll << 28)) return false;
       if ((size_t)p.a_src_rows * p.lda * 2 >= (1ull << 31)) return false;
     }
@@ -1202,11 +1208,15 @@ typedef void (*PersistKernel)(PersistBatch);
 // the rewriting of the tile table.
 template <int MODE, bool HAS_BIAS, int BN, bool GATHER>
 PersistKernel pick64(bool w8, bool refill) {
-  if (w8)
-    return refill ? gemm_persist_kernel4<MODE, HAS_BIAS, BN, GATHER, true, true>
-                  : gemm_persist_kernel4<MODE, HAS_BIAS, BN, GATHER, true, false>;
-  if constexpr (persist64_asm_applies<MODE, HAS_BIAS, BN, GATHER, false>())
-    return refill ? gemm_persist_kernel4a<MODE, BN, GATHER, true> : gemm_persist_kernel4a<MODE, BN, GATHER, false>;
+  if constexpr (!(MODE == kFc1Gelu && GATHER)) {   // (GELU fc1 gathers only with 16-bit weights: persist64_ok)
+    if (w8)
+      return refill ? gemm_persist_kernel4<MODE, HAS_BIAS, BN, GATHER, true, true>
+                    : gemm_persist_kernel4<MODE, HAS_BIAS, BN, GATHER, true, false>;
+  }
+  if constexpr (MODE == kFc1Gelu && GATHER)   // (only launches that fit the tile table: persist64_ok)
+    return gemm_persist_kernel4a<MODE, BN, GATHER, false, HAS_BIAS>;
+  else if constexpr (persist64_asm_applies<MODE, HAS_BIAS, BN, GATHER, false>())
+    return refill ? gemm_persist_kernel4a<MODE, BN, GATHER, true, HAS_BIAS> : gemm_persist_kernel4a<MODE, BN, GATHER, false, HAS_BIAS>;
   else
   return refill ? gemm_persist_kernel4<MODE, HAS_BIAS, BN, GATHER, false, true>
                 : gemm_persist_kernel4<MODE, HAS_BIAS, BN, GATHER, false, false>;
@@ -1265,6 +1275,8 @@ int DICE_PERSIST_LAUNCH(const PersistBatch &b, int mode, hipStream_t s) {
       kern = gathered ? pick64<kFc1Swiglu, false, 256, true>(w8, refill) : pick64<kFc1Swiglu, false, 256, false>(w8, refill);
     else if (mode == kFc1Gelu && narrow)
       kern = has_bias ? pick64<kFc1Gelu, true, 192, false>(w8, refill) : pick64<kFc1Gelu, false, 192, false>(w8, refill);
+    else if (mode == kFc1Gelu && gathered)
+      kern = has_bias ? pick64<kFc1Gelu, true, 256, true>(w8, refill) : pick64<kFc1Gelu, false, 256, true>(w8, refill);
     else if (mode == kFc1Gelu)
       kern = has_bias ? pick64<kFc1Gelu, true, 256, false>(w8, refill) : pick64<kFc1Gelu, false, 256, false>(w8, refill);
     else if (slim)
