@@ -156,6 +156,28 @@ def time_after_idle(blk, x, calls=64, idle_s=2.0):
     return [round(ev[i].elapsed_time(ev[i + 1]), 4) for i in range(calls)]
 
 
+def time_batch_sizes(cfg, variant, dev, sizes=(256, 1024, 1536, 2048, 4096), calls=200):
+    """ms per layer call of the same block at other token counts (sampling batches of 1 to 16 images):
+    `calls` back-to-back calls after 20 warm-ups each."""
+    out = {}
+    for n in sizes:
+        c = dict(cfg)
+        c["tokens"], c["samples"] = n, max(1, n // 256)
+        blk = make_block(c, variant, dev)
+        x = make_input(c, dev)
+        y = torch.empty_like(x)
+        for _ in range(20):
+            blk.run(x, y=y)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(calls):
+            blk.run(x, y=y)
+        torch.cuda.synchronize()
+        out[str(n)] = round((time.perf_counter() - t0) / calls * 1e3, 5)
+        del blk, x, y
+    return out
+
+
 def time_stages(blk, x, steps):
     """Mean duration of every launch of the layer in ms, from the library's own
     stage timers: HIP events recorded between the launches of dice_moe_forward
@@ -859,6 +881,9 @@ def main():
     if not args.no_staleness and main_cfg == "c2":
         # configs[3] with one cache entry per layer over a stack of eight distinct blocks (not part of `value`)
         out["staleness_loop_50_steps_8_layers"] = time_staleness_layers(CONFIGS["c4"], args.variant, dev)
+    if not args.no_configs and main_cfg == "c2":
+        # (not part of `value`) the same block at the token counts of small sampling batches
+        out["ms_per_call_at_other_batch_sizes"] = time_batch_sizes(cfg, args.variant, dev)
     if not args.no_lagged and main_cfg == "c2":
         # the same layer under the reference's step-lagged schedules (not part of `value`)
         out["step_lag_ms_per_layer_call"] = {
