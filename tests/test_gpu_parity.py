@@ -715,16 +715,17 @@ def test_block_xl_width_large_batch_matches_chunks(dev):
     assert rel_l2(y.view(-1, D)[sub][ok], want[ok]) < BF16_TOL
 
 
-@pytest.mark.parametrize("variant,dtype,fp8,N", [
-    ("gelu_tanh", torch.bfloat16, False, 344064),   # biased tiles: the bias buffers are staged across a table rewrite
-    ("swiglu", torch.float16, True, 172032),        # fp8 weights: so are the scale buffers
+@pytest.mark.parametrize("variant,dtype,fp8,N,D,ratio", [
+    ("gelu_tanh", torch.bfloat16, False, 344064, 384, 4),   # biased tiles: the bias buffers are staged across a table rewrite
+    ("swiglu", torch.float16, True, 172032, 384, 4),        # fp8 weights: so are the scale buffers
+    ("swiglu", torch.bfloat16, "act", 180224, 768, 2),      # fp8 activations too: the fp8 kernel's scales and row scales
+    ("gelu_tanh", torch.bfloat16, "act", 180224, 768, 2),   # ... and its bias
 ])
-def test_rewritten_tile_table_other_kernels(dev, variant, dtype, fp8, N):
+def test_rewritten_tile_table_other_kernels(dev, variant, dtype, fp8, N, D, ratio):
     """The other instantiations that rewrite their tile table (more than 64 tiles
     per workgroup): every token bit-identical to the same block run on chunks
     that need no rewrite."""
-    D = 384
-    p = O.make_block_params(D, 8, 2, 4, 2, seed=12, dtype=dtype, variant=variant)
+    p = O.make_block_params(D, 8, 2, ratio, 2, seed=12, dtype=dtype, variant=variant)
     if variant == "gelu_tanh":
         g = _gen(13)
         for e in list(p.experts) + [p.shared]:
@@ -732,7 +733,7 @@ def test_rewritten_tile_table_other_kernels(dev, variant, dtype, fp8, N):
             e.fc2_b = (torch.randn(e.fc2_b.shape, generator=g) * 0.1).to(dtype)
     blk = block_from_params(p, D, variant, dtype, dev)
     if fp8:
-        blk.quantize_fp8()
+        blk.quantize_fp8(activations=fp8 == "act")
     x = torch.randn(1, N, D, generator=torch.Generator(device=dev).manual_seed(14), device=dev).to(dtype)
     with whole_fc2_tiles():
         y = blk(x)
