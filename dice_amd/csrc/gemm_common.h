@@ -185,7 +185,7 @@ size_t persist_split_ws_bytes();         // kPersistSplitSlots tiles of 256 x 25
 bool persist_supported(const PersistBatch &b, int mode);
 int persist_cu_count();  // compute units of the current device
 int persist_band_tiles(int mode);  // tuning hook state: band height of the tile order for this stage (0 = default rule)
-int persist_slim_choice();         // tuning hook state: 128-row weight tiles for fc2 launches that can take them: 1 = always, -1 = never, 0 = by the model
+int persist_slim_choice(int mode);  // tuning hook state: 128-row weight tiles for launches of this stage that can take them: 1 = always, -1 = never, 0 = by the model
 int shared_fc2_launch_choice();   // tuning hook state: 1 = the shared expert's fc2 as a launch of its own, -1 = never, 0 = by size
 bool persist_split_allowed();      // tuning hook state: fc2 launches of the layer call may cut their last turn along k
 bool route_in_prologue_allowed();   // tuning hook state: the modulated layer call may route inside its prologue kernel

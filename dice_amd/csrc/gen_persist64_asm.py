@@ -26,8 +26,8 @@ tile.  The second statement opens with the workgroup barrier; block D then
 reads the first fragments of step s + 1, writes quarter 0 of stage S (step
 s + 2) to slot S and refills it with quarter 0 of step s + 4.
 
-Kinds 0, 1, 4, 5 are the 16-bit shapes (SwiGLU fc1 on 256 weight rows, fc2 on 192
-and on 128, GELU fc1 on 256).  Kinds 2 and 3 are the kernel for fp8 activations and weights
+Kinds 0, 1, 4, 5, 6 are the 16-bit shapes (SwiGLU fc1 on 256 weight rows, fc2 on 192
+and on 128, GELU fc1 on 256, SwiGLU fc1 on 128).  Kinds 2 and 3 are the kernel for fp8 activations and weights
 (grouped_gemm_persist_f8.hip): the same stages, slots and quarters, but a step
 is 128 k in two k-blocks of 64, a fragment is 32 bytes per lane (two LDS reads)
 and there is one set of eight fragments in v[0:63] (weight block j at 8 j, row
@@ -52,6 +52,7 @@ KINDS = {
     1: dict(name="fc2, 192 weight rows", TN=3, CB=6, brow=[0, 32, 64], acc0=4, up_from=99),
     4: dict(name="fc2, 128 weight rows", TN=2, CB=4, brow=[0, 32], acc0=8, up_from=99),
     5: dict(name="GELU fc1, 256 weight rows", TN=4, CB=8, brow=[0, 32, 64, 96], acc0=0, up_from=99),
+    6: dict(name="fc1 SwiGLU, 128 weight rows", TN=2, CB=4, brow=[0, 64], acc0=8, up_from=2),
     # fp8 activations and weights (grouped_gemm_persist_f8.hip): a step is 128 k in two halves of 64 k
     2: dict(name="fp8 SwiGLU fc1, 256 weight rows", TN=4, CB=8, brow=[0, 32, 128, 160], acc0=0, up_from=4, f8=True),
     3: dict(name="fp8 GELU fc1 / fc2, 256 weight rows", TN=4, CB=8, brow=[0, 32, 64, 96], acc0=0, up_from=99, f8=True),

@@ -416,7 +416,10 @@ int persist_band_tiles(int mode) {
   const int cfg = mode == kFc2 ? g_cfg_fc2 : g_cfg_fc1;
   return cfg > 30 && cfg <= 46 ? cfg - 30 : 0;
 }
-int persist_slim_choice() { return g_cfg_fc2 == 54 ? 1 : g_cfg_fc2 == 55 ? -1 : 0; }
+int persist_slim_choice(int mode) {
+  const int cfg = mode == kFc2 ? g_cfg_fc2 : g_cfg_fc1;
+  return cfg == 54 ? 1 : cfg == 55 ? -1 : 0;
+}
 bool persist_split_allowed() { return g_cfg_fc2 != 50; }
 int shared_fc2_launch_choice() { return g_cfg_fc2 == 51 ? 1 : g_cfg_fc2 == 52 ? -1 : 0; }
 bool route_in_prologue_allowed() { return g_cfg_fc1 != 50; }
@@ -434,8 +437,8 @@ bool gemm_config_is_default(int mode) { return (mode == kFc2 ? g_cfg_fc2 : g_cfg
 // along k; 50 (fc1) has dice_moe_forward_modulated launch the router on its own
 // instead of inside the prologue kernel; 51 / 52 (fc2) have the layer call launch
 // the shared expert's fc2 on its own always / never (by default it does for small
-// batches, where both launches then cut their tiles along k); 54 / 55 (fc2) have
-// launches that can take 128-row weight tiles do so always / never (by default
+// batches, where both launches then cut their tiles along k); 54 / 55 (either stage)
+// have launches that can take 128-row weight tiles do so always / never (by default
 // where the host's model says they shorten the launch).  Any value from 20 on also keeps a
 // dice_grouped_mlp stage whose groups average at most 128 rows on the persistent
 // kernels (21 does only that; by default such a stage takes this file's 64-row

@@ -779,7 +779,7 @@ __device__ __forceinline__ void gemm_persist64_body(const PersistBatch &batch) {
 
 template <int MODE, bool HAS_BIAS, int BN, bool GATHER, bool W8>
 constexpr bool persist64_asm_applies() {
-  return !W8 && ((!HAS_BIAS && MODE == kFc1Swiglu && BN == 256 && GATHER) || (!HAS_BIAS && MODE == kFc2 && BN == 192) ||
+  return !W8 && ((!HAS_BIAS && MODE == kFc1Swiglu && (BN == 256 || BN == 128) && GATHER) || (!HAS_BIAS && MODE == kFc2 && BN == 192) ||
                  (MODE == kFc2 && BN == 128) || (MODE == kFc1Gelu && BN == 256));
 }
 
@@ -788,8 +788,9 @@ constexpr bool persist64_asm_applies() {
 template <int MODE, int BN, bool GATHER, bool REFILL, bool HAS_BIAS = false>
 __device__ __forceinline__ void gemm_persist64_asm_body(const PersistBatch &batch) {
   constexpr bool SWIGLU = MODE == kFc1Swiglu;
-  constexpr int KIND = SWIGLU ? 0 : MODE == kFc1Gelu ? 5 : BN == 192 ? 1 : 4;
-  static_assert(SWIGLU || MODE == kFc1Gelu ? BN == 256 : (BN == 192 || BN == 128), "the shapes the generator writes");
+  constexpr int KIND = SWIGLU ? (BN == 256 ? 0 : 6) : MODE == kFc1Gelu ? 5 : BN == 192 ? 1 : 4;
+  static_assert(SWIGLU ? (BN == 256 || BN == 128) : MODE == kFc1Gelu ? BN == 256 : (BN == 192 || BN == 128),
+                "the shapes the generator writes");
   constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
   constexpr int WTN = BN / 2, TM = 4, TN = WTN / 32;
   constexpr int kCopiesA = kPBM / 8 / kQWaves, kCopiesB = BN / 8 / kQWaves;
@@ -1253,7 +1254,7 @@ int DICE_PERSIST_LAUNCH(const PersistBatch &b, int mode, hipStream_t s) {
   // the wave tile is 128 x 64 and reads 6 fragments for 8 products instead of 7 for 12), so they pay where
   // the finer grain shortens the longest workgroup by more than that: small batches, whose few long tiles
   // otherwise round up to a whole turn.  Tuning hook fc2 = 54 / 55: always / never.
-  bool slim = mode == kFc2 && waves == 4 && !w8 && persist_slim_choice() >= 0 &&
+  bool slim = mode == kFc2 && waves == 4 && !w8 && persist_slim_choice(kFc2) >= 0 &&
               persist_fits_table_slim(b, mode);
   for (int i = 0; i < b.n_problems; ++i) slim = slim && b.prob[i].n % 128 == 0;
   // (a single-problem launch with partial-tile slots cuts its last turn along k instead: the better remedy there)
@@ -1261,17 +1262,32 @@ int DICE_PERSIST_LAUNCH(const PersistBatch &b, int mode, hipStream_t s) {
   // (a biased 256-row tile starts its sums from the bias, a 128-row tile adds it behind them: the last bit could
   // differ, and with it the result between batch sizes that the model below sends different ways)
   if (has_bias && !narrow) slim = false;
-  if (slim && persist_slim_choice() == 0) {
+  if (slim && persist_slim_choice(kFc2) == 0) {
     const int64_t m128 = persist_plan(b, 128, grid, true).makespan;
     const int64_t other = persist_plan(b, narrow ? 192 : kPBN, grid, true).makespan;
     // (time per step in units of a 192-row tile's: 128 rows 0.75, 256 rows 1.25)
     slim = m128 * 75 * 100 <= other * (narrow ? 100 : 125) * 93;
   }
   if (slim) narrow = false;
-  const int width = mode == kFc1Swiglu ? kPBN / 2 : slim ? 128 : narrow ? 192 : kPBN;
+  // (time of a step of a 64-output fc1 tile in per cent of a 128-output tile's)
+  constexpr int kSlimFc1StepCost = 60;
+  // The same for SwiGLU fc1 with gathered rows: 128 weight rows (64 gate + 64 up: 64 outputs per tile).  Small
+  // batches, where a tile is mostly the streaming of its weight rows and a launch two turns of which the second
+  // is nearly empty.  Tuning hook fc1 = 54 / 55: always / never.
+  bool slim1 = mode == kFc1Swiglu && waves == 4 && !w8 && gathered && persist_slim_choice(kFc1Swiglu) >= 0 &&
+               persist_fits_table_slim(b, mode);
+  for (int i = 0; i < b.n_problems; ++i) slim1 = slim1 && b.prob[i].n % 64 == 0;
+  if (slim1 && persist_slim_choice(kFc1Swiglu) == 0) {
+    const int64_t m64 = persist_plan(b, 64, grid, false).makespan;
+    const int64_t m128 = persist_plan(b, kPBN / 2, grid, false).makespan;
+    slim1 = m64 * kSlimFc1StepCost <= m128 * 93;
+  }
+  const int width = mode == kFc1Swiglu ? (slim1 ? 64 : kPBN / 2) : slim ? 128 : narrow ? 192 : kPBN;
   if (waves == 4) {
     const bool refill = !persist_fits_table(b, mode);
-    if (mode == kFc1Swiglu)
+    if (mode == kFc1Swiglu && slim1)
+      kern = gemm_persist_kernel4a<kFc1Swiglu, 128, true, false>;
+    else if (mode == kFc1Swiglu)
       kern = gathered ? pick64<kFc1Swiglu, false, 256, true>(w8, refill) : pick64<kFc1Swiglu, false, 256, false>(w8, refill);
     else if (mode == kFc1Gelu && narrow)
       kern = has_bias ? pick64<kFc1Gelu, true, 192, false>(w8, refill) : pick64<kFc1Gelu, false, 192, false>(w8, refill);

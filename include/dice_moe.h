@@ -428,9 +428,11 @@ int dice_profile_read(float *ms_out, int n);
 #define DICE_GEMM_CFG_FC2_WHOLE_TILES 50 /* fc2: no last turn is cut along k (as batch_invariant, for every layer) */
 #define DICE_GEMM_CFG_FC2_SHARED_ALONE 51 /* fc2: the shared expert's fc2 always in a launch of its own */
 #define DICE_GEMM_CFG_FC2_SHARED_JOINT 52 /* fc2: ... never (by default: small batches only) */
-#define DICE_GEMM_CFG_FC2_SLIM_TILES 54   /* fc2: 128-row weight tiles wherever a launch can take them */
-#define DICE_GEMM_CFG_FC2_NO_SLIM_TILES 55 /* fc2: ... never (by default: where the host's model of the workgroups'
-                                              loads says they shorten the launch: mid-size batches) */
+#define DICE_GEMM_CFG_SLIM_TILES 54      /* either stage: 128-row weight tiles wherever a launch can take them (fc2;
+                                            SwiGLU fc1 with gathered rows) */
+#define DICE_GEMM_CFG_NO_SLIM_TILES 55   /* ... never (by default: where the host's model of the workgroups' loads
+                                            says they shorten the launch: fc1 below about 1000 tokens at DiT-XL width,
+                                            fc2 between about 1000 and 2000) */
 int dice_set_gemm_config(int fc1_cfg, int fc2_cfg);
 
 /*

@@ -117,7 +117,7 @@ class Replay:
                 raise AssertionError(f"unexpected instruction {ln}")
 
 
-@pytest.mark.parametrize("kind", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("kind", [0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("live", [1, 2, 3, 4])
 def test_generated_loop_waits_cover_every_dependence(kind, live):
     gen = _load()

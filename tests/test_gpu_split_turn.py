@@ -233,3 +233,35 @@ def test_fc2_on_128_row_weight_tiles(dev, variant, D, ratio, E, n_shared, N, dty
     # (and the default choice is one of the two)
     dflt = blk(x.to(dev)).cpu()
     assert torch.equal(dflt, wide) or torch.equal(dflt, slim)
+
+
+@pytest.mark.parametrize("D,ratio,E,n_shared,N,dtype", [
+    (1152, 4, 8, 2, 256, torch.bfloat16),     # one image: what the model picks them for
+    (1152, 4, 8, 2, 77, torch.bfloat16),      # ragged, most tiles hold a handful of rows
+    (1152, 4, 8, 2, 1000, torch.bfloat16),    # (hook only: the model leaves this size alone)
+    (768, 2, 4, 2, 640, torch.float16),       # the fp16 build
+    (1024, 2, 16, 0, 512, torch.bfloat16),    # no shared expert: one problem per launch
+])
+def test_fc1_on_128_row_weight_tiles(dev, D, ratio, E, n_shared, N, dtype):
+    """SwiGLU fc1 with gathered rows on 128 weight rows per tile (64 gate + 64 up: the kernel
+    with the generated k-loop, wave tile 128 x 64 with one output block per wave): the same
+    sums in the same order as on the 256-row tiles, so the outputs must be identical bit for
+    bit, and meet the oracle."""
+    from dice_amd import lib
+    p = O.make_block_params(D, E, 2, ratio, n_shared, seed=61, dtype=dtype, variant="swiglu")
+    x = torch.randn(1, N, D, generator=_gen(63)).to(dtype)
+    blk = block_from_params(p, D, "swiglu", dtype, dev)
+    try:
+        lib.load().dice_set_gemm_config(54, 0)
+        slim = blk(x.to(dev)).clone().cpu()
+        lib.load().dice_set_gemm_config(55, 0)
+        wide = blk(x.to(dev)).clone().cpu()
+    finally:
+        lib.load().dice_set_gemm_config(0, 0)
+    want, _, _, logits = O.sparse_moe_block_forward(p, x)
+    ok = ~O.gate_tie_rows(logits, 2).view(-1)
+    tol = BF16_TOL if dtype == torch.bfloat16 else F16_TOL
+    check_rows(slim.view(-1, D)[ok], want.view(-1, D)[ok], tol, "128-row fc1 tiles vs oracle")
+    assert torch.equal(slim, wide), "128-row weight tiles changed the result"
+    dflt = blk(x.to(dev)).cpu()
+    assert torch.equal(dflt, wide)
