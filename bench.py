@@ -1,7 +1,7 @@
 """Benchmark of the MoE layer hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1|c2|c3|c4|c5]
-                    [--variant swiglu|gelu_tanh] [--activations bf16|fp8]
+                    [--variant swiglu|gelu_tanh] [--activations bf16|fp8|fp8_blocks]
 
 A step is one call of the whole layer (router -> dispatch -> grouped expert
 MLP + shared expert -> combine) with inputs and weights resident in HBM.  The
@@ -77,7 +77,7 @@ def make_block(cfg, variant, dev, layer_idx=0, total_layers=1, para_mode=None, a
         pr = torch.tensor([(e + 1.0) ** -cfg["zipf"] for e in range(E)])
         blk.gate.bias = (pr / pr.sum()).log().float().to(dev)
     if cfg.get("fp8"):
-        blk.quantize_fp8(activations=(activations == "fp8"))
+        blk.quantize_fp8(activations=activations.startswith("fp8"), h_blocks=(activations == "fp8_blocks"))
     return blk
 
 
@@ -608,8 +608,10 @@ def workload_text(cfg, variant, activations):
     shared = f"{D}->{2 * D}->{D} (reference)" if variant == "swiglu" else f"2 x ({D}->{inter}->{D})"
     if cfg.get("fp8"):
         prec = ("routed experts e4m3 weights (per-output-channel scales), "
-                + ("activations quantised per token to e4m3 in front of each GEMM, fp8 MFMA"
-                   if activations == "fp8" else "bf16 activations (weights widened, bf16 MFMA)")
+                + ("activations quantised per token to e4m3 in front of each GEMM, fp8 MFMA" if activations == "fp8"
+                   else "x quantised per token to e4m3, h per token and 32 columns inside fc1's epilogue (power-of-two "
+                        "scales, scaled fp8 MFMA in fc2)" if activations == "fp8_blocks"
+                   else "bf16 activations (weights widened, bf16 MFMA)")
                 + ", shared expert bf16")
     else:
         prec = f"{cfg['dtype']} in/out, fp32 accumulate"
@@ -625,7 +627,7 @@ def measure(cfg_name, variant, activations, dev, steps, warmup, stages=True):
     sec, fc1_ms = time_layer(blk, x, steps, warmup)
     flops = layer_flops(cfg, variant)
     total_flops = sum(flops.values())
-    a8 = bool(cfg.get("fp8")) and activations == "fp8"
+    a8 = bool(cfg.get("fp8")) and activations.startswith("fp8")
     pipe = "fp8" if a8 else cfg["dtype"]
     res = {"tokens_per_s": cfg["tokens"] / sec, "ms_per_step": sec * 1e3, "workload": workload_text(cfg, variant, activations),
            "layer_tflops": total_flops / sec / 1e12}
@@ -662,7 +664,8 @@ def measure(cfg_name, variant, activations, dev, steps, warmup, stages=True):
                 "fc2": flops["fc2"] / (st["moe.mlp.fc2"] * 1e-3) / 1e12 / PEAK_TFLOPS["fp8"]}
             slots, D, inter = cfg["tokens"] * cfg["topk"], cfg["D"], cfg["ratio"] * cfg["D"]
             res["quantiser_gbs"] = {"x": slots * D * 3 / (st["moe.gather"] * 1e-3) / 1e9,
-                                    "h": slots * inter * 3 / (st["moe.quant_h"] * 1e-3) / 1e9}
+                                    "h": slots * inter * 3 / (st["moe.quant_h"] * 1e-3) / 1e9
+                                    if activations == "fp8" else None}
         hbm = hbm_stage_bytes(cfg, x.element_size())
         res["hbm_stage_gbs"] = {s: hbm[s] / (st[s] * 1e-3) / 1e9 for s in hbm if st[s] > 0}
         res["hbm_stage_frac_of_peak"] = {s: v / PEAK_HBM_GBS for s, v in res["hbm_stage_gbs"].items()}
@@ -765,8 +768,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
     ap.add_argument("--variant", default="swiglu", choices=["swiglu", "gelu_tanh"])
-    ap.add_argument("--activations", default="fp8", choices=["bf16", "fp8"],
-                    help="c5 only: bf16 = fp8 weights widened onto the bf16 MFMA; fp8 = rows quantised per token, fp8 MFMA")
+    ap.add_argument("--activations", default="fp8", choices=["bf16", "fp8", "fp8_blocks"],
+                    help="c5 only: bf16 = fp8 weights widened onto the bf16 MFMA; fp8 = rows quantised per token, fp8 MFMA; "
+                         "fp8_blocks = fp8 with h quantised inside fc1's epilogue (one power-of-two scale per row and 32 columns)")
     ap.add_argument("--fc1-cfg", type=int, default=0)
     ap.add_argument("--fc2-cfg", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -833,7 +837,7 @@ def main():
 
     cfg, blk, x, res = measure(main_cfg, args.variant, args.activations, dev, args.steps, args.warmup,
                                stages=not args.no_stages)
-    a8 = bool(cfg.get("fp8")) and args.activations == "fp8"
+    a8 = bool(cfg.get("fp8")) and args.activations.startswith("fp8")
     metric = {"c1": "MoE-layer tokens/s, DiT-S/2-MoE 1024 tok fp32", "c2": "MoE-layer tokens/s, DiT-XL/2-MoE 8192 tok bf16",
               "c3": "MoE-layer tokens/s, DiT-XL/2-MoE 16384 tok bf16 Zipf router",
               "c5": "MoE-layer tokens/s, DiT-G/2-MoE 8192 tok fp8 experts"}[main_cfg]

@@ -8,7 +8,8 @@ see none of that, a kernel of twelve blocks keeps its sums in a64 .. a255 and
 leaves a0 .. a63 to the compiler.  A kernel whose k-loop is assembly text
 (gemm_persist_kernel4a, gemm_persist_kernel_f8a) also names its register stages, v128 .. v255, in that
 text only: it is compiled with a budget of 128 vector registers and must see
-the compiler neither above v127 nor in any accumulation register.  This script
+the compiler neither above v127 nor in any accumulation register
+(gemm_persist_kernel_f8s: the text names v117 .. v127 as well).  This script
 reads the device assembly the compiler wrote for a translation unit and fails
 the build if an instruction outside the inline assembly touches a register that
 belongs to the assembly.
@@ -18,7 +19,7 @@ from __future__ import annotations
 import re
 import sys
 
-_KERNEL = re.compile(r"^(_ZN4dice\S*gemm_persist_kernel(?:4a?|_f8a)I\S+):")
+_KERNEL = re.compile(r"^(_ZN4dice\S*gemm_persist_kernel(?:4a?|_f8[as])I\S+):")
 _ANY_FN = re.compile(r"^(\S+):\s*(;.*)?$")
 _REG = re.compile(r"\b([av])(\d+)\b|\b([av])\[(\d+):(\d+)\]")
 
@@ -27,6 +28,8 @@ def _owned_from(mangled: str):
     """(first accumulation register, first vector register) the assembly owns."""
     if "gemm_persist_kernel4aI" in mangled or "gemm_persist_kernel_f8aI" in mangled:
         return 0, 128
+    if "gemm_persist_kernel_f8sI" in mangled:     # the scaled kind's text also names v117 .. v127
+        return 0, 117
     # gemm_persist_kernel4<MODE, HAS_BIAS, BN, ...>: ILi<mode>ELb<bias>ELi<BN>E...
     m = re.search(r"gemm_persist_kernel4ILi\d+ELb[01]ELi(\d+)E", mangled)
     if not m:

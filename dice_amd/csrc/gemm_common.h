@@ -167,7 +167,16 @@ struct PersistProblem {
   const float *w_scale;    // [n_experts, w_rows] per-output-channel scales: the weights are fp8 (e4m3) bytes; NULL: bf16
   const float *a_scale;    // [max_rows] per-row scales in grouped order: the activations too are fp8 (e4m3) bytes
                            // (lda then counts bytes) and the products run on the fp8 matrix pipe; NULL: 16-bit rows
+  // Block scales (fp8 kernels only): one power of two per row and 32 columns, as a byte (the exponent biased by 127,
+  // what the scaled MFMA takes), laid out [columns / 128][max_rows][4]: the four scales of a row's 128 columns - one
+  // step of the fp8 kernel - are one dword, the dwords of consecutive rows are adjacent (a tile's scales of a step are
+  // 1 KB of contiguous memory), and within a dword the bytes are ordered 0, 2, 1, 3 (block_scale_pos).
+  const uint8_t *a_block_scale;  // the activations are e4m3 bytes with these scales instead of a_scale (fc2)
+  uint8_t *c_block_scale;        // the output is written as e4m3 bytes (ldc counts bytes) with these scales (fc1)
 };
+// Byte of the scale of 32-column block `cb` within its dword: the fp8 kernel's lane half h reads the scales of both
+// 64-k blocks of a 128-k step as two adjacent bytes.
+__host__ __device__ inline int block_scale_pos(int cb) { return ((cb & 1) << 1) | ((cb >> 1) & 1); }
 constexpr int kMaxPersistProblems = 3;
 struct PersistBatch {
   int n_problems;

@@ -35,6 +35,20 @@ block i at 32 + 8 i), each replaced in place by the next k-block's as soon as
 its last product has been issued; the first statement of a step is k-block 0
 and the first weight block of k-block 1, the second the barrier and the rest.
 
+Kind 7 is kind 3 for activations that carry one power-of-two scale (a byte: the
+exponent, biased by 127) per row and 32 k: the scaled form of the instruction
+multiplies the first 16 bytes that the two lanes of a row hold by the scale of
+the lane in 0-31 and their second 16 bytes by the scale of the lane 32 on.  A
+step's scales - four bytes per row, ordered [lane half][k-block] - travel as a
+17th load of the register stage (v117 / v118: one dword per lane, row
+64 wave + lane) into 1 KB behind each LDS slot's own table, and are read two
+bytes per lane and row block (ds_read_u16: the lane half's bytes of both
+k-blocks, `op_sel` picks the k-block's) into v[119 + 4 slot + i] with the first
+fragments of their step; v127 holds the weights' scale (1.0 in every byte).  The
+statements take their own parameter list (p64s_... functions).  Nothing but the
+build-time check of the device assembly keeps the compiler out of v117 .. v127:
+it allocates from v0 upwards and stays below them in the variants that are built.
+
 The script simulates the instruction stream of the prologue and a few steps,
 finds for every instruction the memory operations it depends on, and emits
 ``s_waitcnt`` with the exact number of younger operations that may still be
@@ -56,7 +70,10 @@ KINDS = {
     # fp8 activations and weights (grouped_gemm_persist_f8.hip): a step is 128 k in two halves of 64 k
     2: dict(name="fp8 SwiGLU fc1, 256 weight rows", TN=4, CB=8, brow=[0, 32, 128, 160], acc0=0, up_from=4, f8=True),
     3: dict(name="fp8 GELU fc1 / fc2, 256 weight rows", TN=4, CB=8, brow=[0, 32, 64, 96], acc0=0, up_from=99, f8=True),
+    7: dict(name="fp8 fc2 on block-scaled activations", TN=4, CB=8, brow=[0, 32, 64, 96], acc0=0, up_from=99, f8=True,
+            scaled=True),
 }
+SC_STAGE, SC_REG, SC_UNIT = 117, 119, 127   # registers of the scaled kind (see the docstring)
 CA = 8            # loads of activation rows per wave per step
 TM = 4
 LGKM_MAX, VM_MAX = 15, 63
@@ -137,7 +154,21 @@ class Stream:
         self.frag_op[reg] = self.lds_issued
         self.lds_issued += 1
 
+    def n_loads(self):
+        return CA + self.k["CB"] + (1 if self.k.get("scaled") else 0)
+
+    def qfirst(self, q):
+        """First load of quarter q of a step (the scales' load rides at the end of the last quarter)."""
+        return quarter_first(self.k["CB"], q) if q < 4 else self.n_loads()
+
     def write(self, stage, l):
+        if l == CA + self.k["CB"]:
+            reg = SC_STAGE + stage
+            if reg in self.stage_op:
+                self.wait("vm", self.stage_op[reg] + 1)
+            self.emit(f"ds_write_b32 %[wrs], v{reg} offset:{1024 * stage}")
+            self.lds_issued += 1
+            return
         reg = 128 + 64 * stage + 4 * l
         if reg in self.stage_op:
             self.wait("vm", self.stage_op[reg] + 1)
@@ -147,6 +178,12 @@ class Stream:
         self.lds_issued += 1
 
     def load(self, stage, l):
+        if l == CA + self.k["CB"]:
+            reg = SC_STAGE + stage
+            self.emit(f"buffer_load_dword v{reg}, %[vs], %[dS], %[kso] offen")
+            self.stage_op[reg] = self.vm_issued
+            self.vm_issued += 1
+            return
         reg = 128 + 64 * stage + 4 * l
         if l < CA:
             self.emit(f"buffer_load_dwordx4 v[{reg}:{reg + 3}], %[va{l}], %[dA], %[koff] offen")
@@ -185,24 +222,39 @@ class Stream:
         self.frag_op[reg] = self.lds_issued
         self.lds_issued += 1
 
-    def mfma8(self, i, j, first):
+    def read_scale(self, slot, i):
+        reg = SC_REG + 4 * slot + i
+        self.emit(f"ds_read_u16 v{reg}, %[rs] offset:{1024 * slot + 256 * i}")
+        self.frag_op[reg] = self.lds_issued
+        self.lds_issued += 1
+
+    def mfma8(self, i, j, first, slot, kb):
         w, a = self.frag_reg8("w", j), self.frag_reg8("a", i)
-        need = max(self.frag_op.get(r, -1) for r in (w, w + 4, a, a + 4)) + 1
+        regs = [w, w + 4, a, a + 4]
+        sc = SC_REG + 4 * slot + i
+        if self.k.get("scaled"):
+            regs.append(sc)
+        need = max(self.frag_op.get(r, -1) for r in regs) + 1
         self.wait("lgkm", need)
         acc = 16 * (self.k["acc0"] + i * self.k["TN"] + j)
         c = "0" if first else f"a[{acc}:{acc + 15}]"
-        self.emit(f"MFMA8 a[{acc}:{acc + 15}], v[{w}:{w + 7}], v[{a}:{a + 7}], {c}")
+        if self.k.get("scaled"):
+            self.emit(f"MFMA8S a[{acc}:{acc + 15}], v[{w}:{w + 7}], v[{a}:{a + 7}], {c}, v{SC_UNIT}, v{sc} "
+                      f"op_sel:[0,{kb},0] op_sel_hi:[0,0,0]")
+        else:
+            self.emit(f"MFMA8 a[{acc}:{acc + 15}], v[{w}:{w + 7}], v[{a}:{a + 7}], {c}")
 
     def column(self, j, up):
         rows = range(self.live) if up else range(self.live - 1, -1, -1)
         return [(i, j) for i in rows]
 
-    def run8(self, prods, first_n, n_block, rslot, rkb, carried, wstage, quarters):
+    def run8(self, prods, first_n, n_block, slot, kb, rslot, rkb, carried, wstage, quarters, scales=()):
         """The products `prods` in order, the first first_n of them starting the sums.  The first n_block of them
         are one k-block; behind the last product of that block that uses a fragment come the two reads that
         replace it by the fragment of k-block rkb of slot rslot (`carried` = fragments already free when the
         statement starts); products past n_block use the new fragments.  The quarters' LDS writes and refills
-        are spread over all gaps."""
+        are spread over all gaps.  (slot, kb): the k-block of the first n_block products; `scales`: row blocks
+        whose scales of slot rslot are read behind the first product."""
         cb = self.k["CB"]
         mf = len(prods)
         gaps = [[] for _ in range(mf)]
@@ -217,20 +269,27 @@ class Stream:
             # (both halves before the first product past the block, which may be the fragment's next user)
             gaps[min(g, n_block - 1)].append(("r", (which, idx, 0)))
             gaps[min(g + 1, n_block - 1)].append(("r", (which, idx, 1)))
-        items = [l for q in quarters for l in range(quarter_first(cb, q), quarter_first(cb, q + 1))]
+        for i in scales:
+            gaps[0].append(("s", i))
+        items = [l for q in quarters for l in range(self.qfirst(q), self.qfirst(q + 1))]
         for n, l in enumerate(items):
             gaps[side_slot(n, len(items), mf, 1)].append(("w", l))
         for n, l in enumerate(items):
             gaps[side_slot(n, len(items), mf, 3)].append(("l", l))
         for g in range(mf):
             i, j = prods[g]
-            self.mfma8(i, j, g < first_n)
-            for kind in ("r", "w", "l"):
+            if g < n_block:
+                self.mfma8(i, j, g < first_n, slot, kb)
+            else:
+                self.mfma8(i, j, g < first_n, rslot, rkb)
+            for kind in ("r", "s", "w", "l"):
                 for k2, x in gaps[g]:
                     if k2 != kind:
                         continue
                     if kind == "r":
                         self.read_half8(rslot, rkb, x[0], x[1], x[2])
+                    elif kind == "s":
+                        self.read_scale(rslot, x)
                     elif kind == "w":
                         self.write(wstage, x)
                     else:
@@ -246,7 +305,7 @@ class Stream:
         next step go from register stage slot^1 to LDS slot slot^1 and are refilled."""
         first = 4 * self.live if var == 1 else 0
         half0 = [p for j in range(4) for p in self.column(j, j % 2 == 0)]
-        self.run8(half0 + self.column(0, False), first, len(half0), slot, 1, [], slot ^ 1, (1, 2, 3))
+        self.run8(half0 + self.column(0, False), first, len(half0), slot, 0, slot, 1, [], slot ^ 1, (1, 2, 3))
 
     def d8(self, slot):
         """Second statement: the barrier, then weight blocks 1..3 of kb = 1, the fragments replaced by those of the
@@ -256,7 +315,8 @@ class Stream:
         self.emit("s_barrier")
         prods = [p for j in (1, 2, 3) for p in self.column(j, j % 2 == 1)]
         # weight block 0 of kb = 1 had its last product in the first statement
-        self.run8(prods, 0, len(prods), slot ^ 1, 0, [("w", 0)], slot, (0,))
+        scales = range(self.live) if self.k.get("scaled") else ()
+        self.run8(prods, 0, len(prods), slot, 1, slot ^ 1, 0, [("w", 0)], slot, (0,), scales)
 
     # ---- the pieces ----
     def frag_order(self):
@@ -271,7 +331,7 @@ class Stream:
         if var == 2:
             prods = []
         reads = self.frag_order()
-        f, e = quarter_first(cb, q), quarter_first(cb, q + 1)
+        f, e = self.qfirst(q), self.qfirst(q + 1)
         items = list(range(f, e))
         mf = max(1, len(prods))
         gaps = [[] for _ in range(mf)]
@@ -317,16 +377,15 @@ class Stream:
         self.block(1, slot ^ 1, 0, slot, 0, 0 if var == 1 else var)
 
     def load_step(self, stage):
-        for l in range(CA + self.k["CB"]):
+        for l in range(self.n_loads()):
             self.load(stage, l)
 
     def write_step(self, stage):
-        for l in range(CA + self.k["CB"]):
+        for l in range(self.n_loads()):
             self.write(stage, l)
 
     def quarter(self, stage, q, what):
-        cb = self.k["CB"]
-        for l in range(quarter_first(cb, q), quarter_first(cb, q + 1)):
+        for l in range(self.qfirst(q), self.qfirst(q + 1)):
             (self.write if what == "w" else self.load)(stage, l)
 
     def read_first(self):
@@ -334,6 +393,9 @@ class Stream:
             for which, idx in self.frags8():
                 for t in (0, 1):
                     self.read_half8(0, 0, which, idx, t)
+            if self.k.get("scaled"):
+                for i in range(self.live):
+                    self.read_scale(0, i)
             return
         for which, idx in self.frag_order():
             self.read_frag(0, 0, 0, which, idx)
@@ -398,25 +460,30 @@ def generate() -> str:
     out = ["// Generated by gen_persist64_asm.py - do not edit.  See that script for the register plan,",
            "// the order of the pieces and how the wait counts are derived.",
            "#pragma once"]
-    names = None
-    table = {}
-    for kind in KINDS:
-        for live in range(1, TM + 1):
-            pcs = simulate(kind, live)
-            table[(kind, live)] = pcs
-            names = sorted(pcs)
-    for name in names:
-        out.append(f"template <int KIND, int LIVE>\n__device__ __forceinline__ void p64_{name}(P64_PARAMS) {{")
-        first = True
-        for (kind, live), pcs in table.items():
-            text = [ln.replace("MFMA8", '" DICE_MFMA8 "').replace("MFMA ", '" DICE_MFMA16 " ') for ln in pcs[name]]
-            cond = f"KIND == {kind} && LIVE == {live}"
-            out.append(f"  {'if' if first else 'else if'} constexpr ({cond})")
-            out.append("    asm volatile(")
-            out.append(c_string(text) if text else '      ""')
-            out.append("      P64_CONSTRAINTS);")
-            first = False
-        out.append("  else static_assert(KIND < 0, \"no such variant\");\n}")
+    # (the scaled kind's statements take more operands: a function family of their own)
+    for fam, macro, scaled in (("p64", "P64", False), ("p64s", "P64S", True)):
+        names = None
+        table = {}
+        for kind in KINDS:
+            if bool(KINDS[kind].get("scaled")) != scaled:
+                continue
+            for live in range(1, TM + 1):
+                pcs = simulate(kind, live)
+                table[(kind, live)] = pcs
+                names = sorted(pcs)
+        for name in names:
+            out.append(f"template <int KIND, int LIVE>\n__device__ __forceinline__ void {fam}_{name}({macro}_PARAMS) {{")
+            first = True
+            for (kind, live), pcs in table.items():
+                text = [ln.replace("MFMA8S", '" DICE_MFMA8_SCALED "').replace("MFMA8 ", '" DICE_MFMA8 " ')
+                        .replace("MFMA ", '" DICE_MFMA16 " ') for ln in pcs[name]]
+                cond = f"KIND == {kind} && LIVE == {live}"
+                out.append(f"  {'if' if first else 'else if'} constexpr ({cond})")
+                out.append("    asm volatile(")
+                out.append(c_string(text) if text else '      ""')
+                out.append(f"      {macro}_CONSTRAINTS);")
+                first = False
+            out.append("  else static_assert(KIND < 0, \"no such variant\");\n}")
     return "\n".join(out) + "\n"
 
 

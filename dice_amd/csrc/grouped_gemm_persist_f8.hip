@@ -56,11 +56,24 @@ namespace {
 // tiles are 256 whole rows (SwiGLU: 128 gate + 128 up; the weight loads carry
 // their row in the scalar offset, which the range check does not see),
 // single-problem launches.
-template <int MODE, bool HAS_BIAS, bool REFILL>
+//
+// BLK = 1 (fc1): the output goes out as e4m3 bytes with one power-of-two scale
+// per row and 32 columns (tile_epilogue_blockq) - the quantiser of h fused into
+// the epilogue.  BLK = 2 (fc2): the activations are such bytes; the products run
+// on the scaled form of the instruction, which multiplies each lane's 32 k of the
+// activation operand by a scale byte (generator kind 7: a step's scales travel
+// through the register stage and 1 KB of LDS per slot like the operands
+// themselves).  The hardware applies the byte of a lane in 0-31 to the first 16
+// bytes of that row's operand in BOTH lane halves and the byte of the lane 32 on
+// to the second 16 bytes, so here a lane half holds the 16-byte chunks
+// 4 kb + h and 4 kb + 2 + h of a row and supplies the scale of the row's 32 k
+// at 64 kb + 32 h.  There is no row scale then.
+template <int MODE, bool HAS_BIAS, bool REFILL, int BLK = 0>
 __device__ __forceinline__ void gemm_persist_f8_asm_body(const PersistBatch &batch) {
   constexpr bool SWIGLU = MODE == kFc1Swiglu;
   static_assert(!(SWIGLU && HAS_BIAS), "the SwiGLU expert has no bias");
-  constexpr int KIND = SWIGLU ? 2 : 3;
+  static_assert(BLK == 0 || (BLK == 1 && MODE != kFc2) || (BLK == 2 && MODE == kFc2), "block scales: h only");
+  constexpr int KIND = BLK == 2 ? 7 : SWIGLU ? 2 : 3;
   constexpr int BN_OUT = SWIGLU ? kPBN / 2 : kPBN;
   constexpr int TM = 4, TN = 4;
   constexpr int kFBK = 128;
@@ -86,6 +99,9 @@ __device__ __forceinline__ void gemm_persist_f8_asm_body(const PersistBatch &bat
   float *const lds_rowscale =
       reinterpret_cast<float *>(lds_stage + kPStageArea - kTableBytes - kColScaleBytes - kRowScaleBytes);
   float *const lds_bias = reinterpret_cast<float *>(lds_stage + kPStageArea - kEpiReserve);
+  // (BLK = 2: the row scales' area holds the two slots' block scales instead, 256 rows x 4 bytes each)
+  static_assert(kRowScaleBytes >= 2 * 1024, "block scales of two slots");
+  if constexpr (BLK == 2) asm volatile("v_mov_b32 v127, 0x7f7f7f7f");   // the weights' scale: 1.0 in every byte
   if (wave == 0) {
     TileWalker<BN_OUT> walk(batch, lane);
     walk.build_table(batch, lane, kFBK, tile_table, true, 0, true);
@@ -136,7 +152,7 @@ __device__ __forceinline__ void gemm_persist_f8_asm_body(const PersistBatch &bat
     const uint64_t ptr = ((uint64_t)(uint32_t)__builtin_amdgcn_readlane(pk.words, 21) << 32) |
                          (uint32_t)__builtin_amdgcn_readlane(pk.words, 20);
     const int rows = __builtin_amdgcn_readlane(pk.words, 23);
-    if (wave == 0 && ptr != 0) {
+    if (BLK != 2 && wave == 0 && ptr != 0) {
       int lane_c = lane;
       asm volatile("" : "+v"(lane_c));
       // rows past the group's end read as 0 (their products are never stored)
@@ -170,8 +186,12 @@ __device__ __forceinline__ void gemm_persist_f8_asm_body(const PersistBatch &bat
   // start of every tile (chunk 4 kb + 2 h + t of a row is chunk 2 h with bits 2
   // and 0 flipped; slot 1 lies a constant behind slot 0).
   uint32_t wr0 = slot_base[0] + qring_off(cp_row0, cp_chunk);
-  uint32_t ra0 = slot_base[0] + qring_off(wm * 32 + (lane & 31), (lane >> 5) * 2);
-  uint32_t rb0 = slot_base[0] + kPBM * 128 + qring_off(b_row0 + (lane & 31), (lane >> 5) * 2);
+  // (BLK = 2: the scaled instruction fixes the assignment - it multiplies the first 16 bytes of every lane by
+  // the scale that lanes 0-31 supply and the second 16 by the one of lanes 32-63, so a scale's 32 k must be
+  // the same 16-byte part of both lane halves: part t of half h is the row's chunk 4 kb + 2 t + h)
+  const int half_chunk = BLK == 2 ? (lane >> 5) : (lane >> 5) * 2;
+  uint32_t ra0 = slot_base[0] + qring_off(wm * 32 + (lane & 31), half_chunk);
+  uint32_t rb0 = slot_base[0] + kPBM * 128 + qring_off(b_row0 + (lane & 31), half_chunk);
   static_assert((kQSlotBytes & 1023) == 0, "the xor below must stay inside the chunk field");
   auto set_lds_addresses = [&]() {
     asm volatile("" : "+v"(wr0), "+v"(ra0), "+v"(rb0));
@@ -182,7 +202,7 @@ __device__ __forceinline__ void gemm_persist_f8_asm_body(const PersistBatch &bat
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        const uint32_t flip = (uint32_t)((kb * 4 + t) << 4);
+        const uint32_t flip = (uint32_t)((kb * 4 + (BLK == 2 ? 2 * t : t)) << 4);
         ad.ra[0][kb * 2 + t] = ra0 ^ flip;
         ad.rb[0][kb * 2 + t] = rb0 ^ flip;
         ad.ra[1][kb * 2 + t] = (ra0 ^ flip) + slot1;
@@ -195,8 +215,26 @@ __device__ __forceinline__ void gemm_persist_f8_asm_body(const PersistBatch &bat
   ad.vb = 0;
   uint32_t sb_row[8] = {}, sb[8] = {};   // scalar offsets of the weight loads: row part, and with the step's k offset
   u32x4_t dA, dB0, dB1;
+  // (BLK = 2) block scales: a step's are one dword per row, the next step's max_rows dwords on; this lane loads
+  // those of tile row 64 wave + lane
+  const uint32_t scale_step = (uint32_t)batch.prob[0].max_rows * 4u;
+  const uint32_t scale_lds = (uint32_t)(size_t)(lds_byte_t *)lds_rowscale;
+  P64ScaleAddr sa;
+  sa.vs = 0;
+  sa.wrs = scale_lds + (uint32_t)(wave * 64 + lane) * 4;
+  sa.rs = scale_lds + (uint32_t)(wm * 32 + (lane & 31)) * 4 + (uint32_t)(lane >> 5) * 2;
+  u32x4_t dS = {};
+  uint32_t kso = 0;
   auto set_copy_offsets = [&](const Tile &t) {
     dA = desc(t.a, t.a_bytes);
+    if constexpr (BLK == 2) {
+      // (a raw buffer's range check counts the scalar offset - the step - in: the extent covers every step, and
+      // a row past the group's end gets an offset that no extent covers, so its scales read as 0 like its bytes)
+      dS = desc(t.a_rows, (uint32_t)t.steps * scale_step);
+      int srow = wave * 64 + lane;
+      asm volatile("" : "+v"(srow));
+      sa.vs = srow < t.rows ? (uint32_t)srow * 4u : kOutOfRange;
+    }
     dB0 = desc(t.b0, t.b_bytes);
     dB1 = desc(t.b1, t.b_bytes);
     int row0 = cp_row0;   // (opaque, as the lane above)
@@ -213,6 +251,11 @@ __device__ __forceinline__ void gemm_persist_f8_asm_body(const PersistBatch &bat
     }
   };
 
+#define DICE_F8_STEP(name, live)                                     \
+  do {                                                               \
+    if constexpr (BLK == 2) p64s_##name<KIND, live>(P64S_ARGS);      \
+    else p64_##name<KIND, live>(P64_ARGS);                           \
+  } while (0)
   // ---- pipeline state ----
   int next_turn = 0;
   PackedTile nxt = fetch_tile(next_turn++);
@@ -241,6 +284,7 @@ __device__ __forceinline__ void gemm_persist_f8_asm_body(const PersistBatch &bat
       ld_kt = 0;
     }
     koff = uni((uint32_t)ld_kt * (uint32_t)kFBK);
+    if constexpr (BLK == 2) kso = uni((uint32_t)ld_kt * scale_step);
 #pragma unroll
     for (int i = 0; i < 8; ++i) sb[i] = uni(sb_row[i] + koff);
   };
@@ -251,15 +295,15 @@ __device__ __forceinline__ void gemm_persist_f8_asm_body(const PersistBatch &bat
     asm volatile("" : "={v[0:31]}"(f0), "={v[32:63]}"(f1));
     // Prologue: steps 0 and 1 through the stages into the slots (of step 1 only the
     // first quarter), steps 2 and 3 (first quarter) into the stages behind them.
-    p64_load_step0<KIND, 4>(P64_ARGS);
+    DICE_F8_STEP(load_step0, 4);
     advance_copy();
-    p64_load_step1<KIND, 4>(P64_ARGS);
+    DICE_F8_STEP(load_step1, 4);
     advance_copy();
-    p64_write_step0<KIND, 4>(P64_ARGS);
-    p64_load_step0<KIND, 4>(P64_ARGS);
+    DICE_F8_STEP(write_step0, 4);
+    DICE_F8_STEP(load_step0, 4);
     advance_copy();
-    p64_write_q0_stage1<KIND, 4>(P64_ARGS);
-    p64_load_q0_stage1<KIND, 4>(P64_ARGS);
+    DICE_F8_STEP(write_q0_stage1, 4);
+    DICE_F8_STEP(load_q0_stage1, 4);
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   phase_barrier();
@@ -274,20 +318,20 @@ __device__ __forceinline__ void gemm_persist_f8_asm_body(const PersistBatch &bat
     f32x32_t f0, f1;   // the fragments: live inside the tile's k-loop only
     asm volatile("" : "={v[0:31]}"(f0), "={v[32:63]}"(f1));
     set_lds_addresses();
-    p64_read_first<KIND, LIVE>(P64_ARGS);
-    p64_abc_s0_v1<KIND, LIVE>(P64_ARGS);   // the first k-block's products start the sums
+    DICE_F8_STEP(read_first, LIVE);
+    DICE_F8_STEP(abc_s0_v1, LIVE);   // the first k-block's products start the sums
     advance_copy();
-    p64_d_s0<KIND, LIVE>(P64_ARGS);
-    p64_abc_s1_v0<KIND, LIVE>(P64_ARGS);
+    DICE_F8_STEP(d_s0, LIVE);
+    DICE_F8_STEP(abc_s1_v0, LIVE);
     advance_copy();
-    p64_d_s1<KIND, LIVE>(P64_ARGS);
+    DICE_F8_STEP(d_s1, LIVE);
     for (int s = 2; s < cp.steps; s += 2) {
-      p64_abc_s0_v0<KIND, LIVE>(P64_ARGS);
+      DICE_F8_STEP(abc_s0_v0, LIVE);
       advance_copy();
-      p64_d_s0<KIND, LIVE>(P64_ARGS);
-      p64_abc_s1_v0<KIND, LIVE>(P64_ARGS);
+      DICE_F8_STEP(d_s0, LIVE);
+      DICE_F8_STEP(abc_s1_v0, LIVE);
       advance_copy();
-      p64_d_s1<KIND, LIVE>(P64_ARGS);
+      DICE_F8_STEP(d_s1, LIVE);
     }
   };
 
@@ -300,9 +344,19 @@ __device__ __forceinline__ void gemm_persist_f8_asm_body(const PersistBatch &bat
     fixed_acc_settle();
     int lane_e = lane;   // (opaque: the epilogue's addresses are worked out here, not held through the k-loop)
     asm volatile("" : "+v"(lane_e));
-    tile_epilogue<MODE, false, kQWaves, TM, TN, true, kEpiReserve, true, HAS_BIAS, 0, false, 64>(
-        cp, no_acc, stage_rows, wm * 32, wave_col0, lane_e, lds_colscale + scale_buf * kScaleBufFloats,
-        lds_rowscale + scale_buf * kPBM, lds_bias + scale_buf * kBiasBufFloats, live);
+    if constexpr (BLK == 1) {
+      // the tile's first row of block scales (its rows and the scales' are in the same, grouped order)
+      const PersistProblem &pr = batch.prob[0];
+      const uint32_t tile_row0 = uni((uint32_t)(cp.c - (const unsigned char *)pr.c) / cp.c_pitch);
+      tile_epilogue_blockq<MODE, kQWaves, TM, TN, HAS_BIAS, 64, kEpiReserve>(
+          cp, lds_stage + wave * BlockqGeom<MODE, kQWaves, TN, kEpiReserve>::WAVE_BYTES, wm * 32, wave_col0, lane_e, lds_colscale + scale_buf * kScaleBufFloats,
+          lds_rowscale + scale_buf * kPBM, lds_bias + scale_buf * kBiasBufFloats, live,
+          pr.c_block_scale + (size_t)tile_row0 * 4, (uint32_t)pr.max_rows);
+    } else {
+      tile_epilogue<MODE, false, kQWaves, TM, TN, true, kEpiReserve, BLK != 2, HAS_BIAS, 0, false, 64>(
+          cp, no_acc, stage_rows, wm * 32, wave_col0, lane_e, lds_colscale + scale_buf * kScaleBufFloats,
+          lds_rowscale + scale_buf * kPBM, lds_bias + scale_buf * kBiasBufFloats, live);
+    }
     cp = ld;
     if (!cp.valid) break;
     nxt = fetch_tile(next_turn++);
@@ -313,14 +367,25 @@ __device__ __forceinline__ void gemm_persist_f8_asm_body(const PersistBatch &bat
     copy_rowscale(nxt, scale_buf == 2 ? 0 : scale_buf + 1);
     copy_bias(nxt, scale_buf == 2 ? 0 : scale_buf + 1);
   }
+#undef DICE_F8_STEP
 }
 
 // fp8 activations and weights.  The compiler allocates from v0..v127 only;
 // v128..v255 and every accumulation register belong to the assembly text.
-template <int MODE, bool HAS_BIAS, bool REFILL>
+template <int MODE, bool HAS_BIAS, bool REFILL, bool BLOCK_OUT = false>
 __global__ __launch_bounds__(4 * kWave, 1) __attribute__((amdgpu_num_vgpr(128)))
 void gemm_persist_kernel_f8a(PersistBatch batch) {
-  gemm_persist_f8_asm_body<MODE, HAS_BIAS, REFILL>(batch);
+  gemm_persist_f8_asm_body<MODE, HAS_BIAS, REFILL, BLOCK_OUT ? 1 : 0>(batch);
+}
+// fc2 on block-scaled activations: v117..v127 too belong to the assembly text
+// (the scales' register stage, the scales of the step's row blocks, the weights'
+// scale).  The variant that rebuilds its tile table (more than 64 turns per
+// workgroup) needs those registers for itself and is not built: the launcher
+// refuses such launches.
+template <bool HAS_BIAS>
+__global__ __launch_bounds__(4 * kWave, 1) __attribute__((amdgpu_num_vgpr(128)))
+void gemm_persist_kernel_f8s(PersistBatch batch) {
+  gemm_persist_f8_asm_body<kFc2, HAS_BIAS, false, 2>(batch);
 }
 }  // namespace
 
@@ -332,7 +397,10 @@ bool persist_fits_table(const PersistBatch &b, int mode);
 bool persist_f8_supported(const PersistBatch &b, int mode) {
   if (b.n_problems != 1 || persist_cu_count() < kNumXcd) return false;
   const PersistProblem &p = b.prob[0];
-  if (!p.a_scale || !p.w_scale || p.a_rows) return false;
+  // activations: one scale per row, or (fc2) block scales; block-scaled output: fc1 only
+  if ((!p.a_scale == !p.a_block_scale) || !p.w_scale || p.a_rows) return false;
+  if (p.a_block_scale && mode != kFc2) return false;
+  if (p.c_block_scale && (mode == kFc2 || p.ldc % 16 != 0 || (uint64_t)p.max_rows * p.ldc >= (1ull << 32))) return false;
   if (p.n_experts < 1 || p.n_experts > kWave) return false;
   if (p.k % 256 != 0 || p.k < 128 * kQMinSteps) return false;
   if (p.lda % 16 != 0 || p.ldc % 8 != 0) return false;                  // 16-byte loads and stores
@@ -348,10 +416,20 @@ int launch_grouped_gemm_persist_f8(const PersistBatch &b, int mode, hipStream_t 
   const int grid = persist_cu_count() / kNumXcd * kNumXcd;
   const bool has_bias = mode != kFc1Swiglu && b.prob[0].bias != nullptr;
   const bool refill = !persist_fits_table(b, mode);
+  if (refill && b.prob[0].a_block_scale)
+    return fail(DICE_ERR_UNSUPPORTED, "fp8 expert GEMM on block-scaled activations: more than 64 tiles per workgroup");
   void (*kern)(PersistBatch) = nullptr;
 #define DICE_F8_PICK(MODE, BIAS) \
   (refill ? gemm_persist_kernel_f8a<MODE, BIAS, true> : gemm_persist_kernel_f8a<MODE, BIAS, false>)
-  if (mode == kFc1Swiglu)
+#define DICE_F8_PICK_OUT(MODE, BIAS) \
+  (refill ? gemm_persist_kernel_f8a<MODE, BIAS, true, true> : gemm_persist_kernel_f8a<MODE, BIAS, false, true>)
+  if (b.prob[0].a_block_scale)
+    kern = has_bias ? gemm_persist_kernel_f8s<true> : gemm_persist_kernel_f8s<false>;
+  else if (b.prob[0].c_block_scale)
+    kern = mode == kFc1Swiglu ? DICE_F8_PICK_OUT(kFc1Swiglu, false)
+           : has_bias         ? DICE_F8_PICK_OUT(kFc1Gelu, true)
+                              : DICE_F8_PICK_OUT(kFc1Gelu, false);
+  else if (mode == kFc1Swiglu)
     kern = DICE_F8_PICK(kFc1Swiglu, false);
   else if (mode == kFc1Gelu && has_bias)
     kern = DICE_F8_PICK(kFc1Gelu, true);
@@ -362,6 +440,7 @@ int launch_grouped_gemm_persist_f8(const PersistBatch &b, int mode, hipStream_t 
   else
     kern = DICE_F8_PICK(kFc2, false);
 #undef DICE_F8_PICK
+#undef DICE_F8_PICK_OUT
   PersistBatch launch = b;
   launch.band_tiles = persist_band_tiles(mode);
   launch.xcd_split = 1;   // (one problem: the two splits are the same)

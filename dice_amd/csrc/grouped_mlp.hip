@@ -155,10 +155,17 @@ namespace {
 // The two fp8 x fp8 problems of an expert MLP whose activations are quantised
 // per row on the way in: fc1 reads q_rows as [rows, hidden] bytes, fc2 as
 // [rows, inter] bytes (the buffer is re-used between the stages).
+// h_blocks: fc1 writes h as e4m3 bytes with one power-of-two scale per row and
+// 32 columns into the buffer `h` itself ([rows, inter] bytes, then [rows,
+// inter / 32] scale bytes: together just over half of the 16-bit h it replaces)
+// and fc2 reads them there; no quantiser runs between the stages.
+uint8_t *h_block_scales(void *h, int64_t max_rows, int inter) {
+  return (uint8_t *)h + (((size_t)max_rows * inter + 255) & ~(size_t)255);
+}
 void a8_problems(const int32_t *offsets, int n_experts, int64_t max_rows, int hidden, int inter, const void *w1,
                  const float *b1, const void *w2, const float *b2, const float *w1_scale, const float *w2_scale,
                  bool swiglu, void *h, void *out, const uint8_t *q_rows, const float *q_scale, PersistBatch *f1,
-                 PersistBatch *f2) {
+                 PersistBatch *f2, bool h_blocks = false) {
   *f1 = PersistBatch{};
   *f2 = PersistBatch{};
   f1->n_problems = f2->n_problems = 1;
@@ -169,6 +176,12 @@ void a8_problems(const int32_t *offsets, int n_experts, int64_t max_rows, int hi
   f1->prob[0].w_scale = w1_scale;
   f2->prob[0].w_scale = w2_scale;
   f1->prob[0].a_scale = f2->prob[0].a_scale = q_scale;
+  if (h_blocks) {
+    f1->prob[0].c_block_scale = h_block_scales(h, max_rows, inter);
+    f2->prob[0].a = h;
+    f2->prob[0].a_scale = nullptr;
+    f2->prob[0].a_block_scale = h_block_scales(h, max_rows, inter);
+  }
 }
 
 // Stage 1: quantise the (gathered) input rows, fc1 + activation -> h (bf16).
@@ -196,8 +209,10 @@ int mlp_a8_run(int stages, const void *x, const int32_t *perm, int slots_per_tok
   if (rc) return rc;
   if (stages & 2) {
     mark(3);
-    rc = quantize_act_impl(h, DICE_BF16, nullptr, 1, offsets + n_experts, max_rows, inter, q_rows, q_scale, s);
-    if (rc) return rc;
+    if (!f2.prob[0].a_block_scale) {   // (else fc1's epilogue has quantised h)
+      rc = quantize_act_impl(h, DICE_BF16, nullptr, 1, offsets + n_experts, max_rows, inter, q_rows, q_scale, s);
+      if (rc) return rc;
+    }
     mark(4);
     rc = launch_grouped_gemm_persist_f8(f2, kFc2, s);
   }
@@ -210,7 +225,7 @@ extern "C" int dice_grouped_mlp_a8(int stages, const void *x, int act_dtype, con
                                    int slots_per_token, const int32_t *offsets, int n_experts,
                                    int64_t max_rows, int hidden, int inter, const void *w1, const float *b1,
                                    const void *w2, const float *b2, const float *w1_scale,
-                                   const float *w2_scale, int act_variant, void *h, void *out,
+                                   const float *w2_scale, int act_variant, int h_blocks, void *h, void *out,
                                    uint8_t *q_rows, float *q_scale, void *stream) {
   using namespace dice;
   DICE_REQUIRE(x && offsets && w1 && w2 && h && out && q_rows && q_scale && w1_scale && w2_scale, DICE_ERR_BAD_ARG,
@@ -228,8 +243,9 @@ extern "C" int dice_grouped_mlp_a8(int stages, const void *x, int act_dtype, con
   if (max_rows == 0) return DICE_OK;
   const bool swiglu = act_variant == DICE_ACT_SWIGLU;
   PersistBatch f1, f2;
+  DICE_REQUIRE(h_blocks == 0 || h_blocks == 1, DICE_ERR_BAD_ARG, "dice_grouped_mlp_a8: h_blocks %d (0 or 1)", h_blocks);
   a8_problems(offsets, n_experts, max_rows, hidden, inter, w1, b1, w2, b2, w1_scale, w2_scale, swiglu, h, out,
-              q_rows, q_scale, &f1, &f2);
+              q_rows, q_scale, &f1, &f2, h_blocks != 0);
   DICE_REQUIRE(persist_f8_supported(f1, swiglu ? kFc1Swiglu : kFc1Gelu) && persist_f8_supported(f2, kFc2),
                DICE_ERR_UNSUPPORTED,
                "dice_grouped_mlp_a8: hidden %d and inter %d must be multiples of 256 (at least 768), n_experts %d at most 64",
@@ -432,10 +448,11 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
                  "%s: shared expert weights / shared_inter %d", who, L->shared_inter);
   }
   if (L->act_quant || LE->act_quant) {
-    DICE_REQUIRE(L->act_quant == 1 && LE->act_quant == 1 && L->act_dtype == DICE_BF16 &&
-                     LE->w_dtype == DICE_FP8_E4M3 && LE->w1_scale && LE->w2_scale,
+    DICE_REQUIRE((L->act_quant == 1 || L->act_quant == 2) && LE->act_quant == L->act_quant &&
+                     L->act_dtype == DICE_BF16 && LE->w_dtype == DICE_FP8_E4M3 && LE->w1_scale && LE->w2_scale,
                  DICE_ERR_UNSUPPORTED,
-                 "%s: act_quant (0 or 1) needs bf16 activations and fp8 expert weights with scales, in both layers", who);
+                 "%s: act_quant (0, 1 or 2) needs bf16 activations and fp8 expert weights with scales, in both layers",
+                 who);
     // (what the fp8 kernels and the row quantiser take, checked before anything is launched)
     DICE_REQUIRE(act_quant_widths_ok(L->hidden, L->inter), DICE_ERR_UNSUPPORTED,
                  "%s: act_quant needs hidden %d and inter %d to be multiples of 256 between 768 and 8192", who,
@@ -556,7 +573,8 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
     const int m1 = swiglu ? kFc1Swiglu : kFc1Gelu;
     PersistBatch f1, f2, s1{}, s2{};
     a8_problems(work.offsets, L->n_experts, max_rows, L->hidden, L->inter, LE->w1, LE->b1, LE->w2, LE->b2,
-                LE->w1_scale, LE->w2_scale, swiglu, w.h, work.rows, w.q_rows, w.q_scale, &f1, &f2);
+                LE->w1_scale, LE->w2_scale, swiglu, w.h, work.rows, w.q_rows, w.q_scale, &f1, &f2,
+                LE->act_quant == 2);
     DICE_REQUIRE(persist_f8_supported(f1, m1) && persist_f8_supported(f2, kFc2), DICE_ERR_UNSUPPORTED,
                  "%s: act_quant needs hidden %d and inter %d to be multiples of 256 (at least 768)", who,
                  L->hidden, L->inter);

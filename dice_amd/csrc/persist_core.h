@@ -479,7 +479,9 @@ struct TileWalker {
     const int row0 = __shfl(g_row0, grp, kWave), cnt = __shfl(g_cnt, grp, kWave);
     const int mt = __shfl(g_mt, grp, kWave), base = __shfl(g_base, grp, kWave);
     // this lane's problem (a handful of selects instead of a divergent struct index)
-    uint64_t pa = 0, pw = 0, pc = 0, pbias = 0, prows = 0, pascale = 0;
+    uint64_t pa = 0, pw = 0, pc = 0, pbias = 0, prows = 0, pascale = 0, pablock = 0;
+    bool c8 = false;
+    int max_rows = 0;
     int lda = 0, ldc = 0, w_rows = 0, up_offset = 0, n = 0, k = 0, a_div = 1, a_src_rows = 0;
     for (int q = 0; q < batch.n_problems; ++q) {
       const PersistProblem &pr = batch.prob[q];
@@ -488,6 +490,9 @@ struct TileWalker {
         lda = pr.lda; ldc = pr.ldc; w_rows = pr.w_rows; up_offset = pr.up_offset; n = pr.n; k = pr.k;
         prows = (uint64_t)pr.a_rows; a_div = pr.a_div; a_src_rows = pr.a_src_rows;
         pascale = (uint64_t)pr.a_scale;
+        pablock = (uint64_t)pr.a_block_scale;
+        c8 = pr.c_block_scale != nullptr;
+        max_rows = pr.max_rows;
       }
     }
     const int r = idc - base;
@@ -502,7 +507,7 @@ struct TileWalker {
     // per-output-channel scale table instead of the gather's reciprocal, which a
     // single-problem launch takes from its arguments)
     const uint32_t a_pitch = (uint32_t)lda * (a8 ? 1 : 2), b_pitch = (uint32_t)k * (w8 ? 1 : 2);
-    uint32_t c_pitch = (uint32_t)ldc * 2, c_extent = (uint32_t)rows * c_pitch;
+    uint32_t c_pitch = (uint32_t)ldc * (c8 ? 1 : 2), c_extent = (uint32_t)rows * c_pitch;
     const uint64_t wexp = pw + (uint64_t)expert * w_rows * b_pitch;
     // Gathered rows are addressed from the start of the source matrix.
     uint64_t ptrs[5] = {prows ? pa : pa + (uint64_t)(row0 + m_tile * kPBM) * a_pitch, wexp + (uint64_t)n0 * b_pitch,
@@ -510,6 +515,7 @@ struct TileWalker {
                         pc + (uint64_t)(row0 + m_tile * kPBM) * c_pitch,
                         pbias ? pbias + ((uint64_t)expert * n) * sizeof(float) : 0};
     int steps = k / bk;
+    uint32_t k_first = 0;
     if (cut && sp.ways != 0) {
       // This position's piece of the tile: its run of steps (the k offset moves
       // the operands' base addresses; range checks look at row offsets only), and
@@ -518,6 +524,7 @@ struct TileWalker {
       const SplitRange run = split_range(steps, sp.piece, sp.ways);
       steps = run.count;
       const uint32_t k0 = (uint32_t)(run.begin * bk);
+      k_first = k0;
       ptrs[0] += (uint64_t)k0 * (a8 ? 1 : 2);
       ptrs[1] += (uint64_t)k0 * (w8 ? 1 : 2);
       ptrs[2] += (uint64_t)k0 * (w8 ? 1 : 2);
@@ -538,7 +545,11 @@ struct TileWalker {
     }
 #pragma unroll
     for (int i = 0; i < 10; ++i) entry[10 + i] = words[i];
-    const uint64_t tile_rows = a8 ? pascale + (uint64_t)(row0 + m_tile * kPBM) * sizeof(float)
+    // (fp8 activations: the tile's first row scale, or the dword of its first row's block scales in the tile's
+    // first step - the next step's lie max_rows dwords on)
+    const uint64_t tile_rows = a8 ? (pablock ? pablock + ((uint64_t)(k_first / 128) * (uint32_t)max_rows +
+                                                          (uint64_t)(row0 + m_tile * kPBM)) * 4
+                                             : pascale + (uint64_t)(row0 + m_tile * kPBM) * sizeof(float))
                                   : (prows ? prows + (uint64_t)(row0 + m_tile * kPBM) * sizeof(int32_t) : 0);
     entry[20] = (uint32_t)tile_rows;
     entry[21] = (uint32_t)(tile_rows >> 32);
@@ -836,6 +847,129 @@ __device__ __forceinline__ void tile_epilogue(const Tile &cp, f32x16_t (&acc)[TM
 #undef DICE_EPI_VALUE
 #undef DICE_EPI_SCALES
 #undef DICE_EPI_STORE_BAND
+}
+
+// The epilogue of an fp8 fc1 tile whose output goes out as e4m3 bytes with one
+// power-of-two scale per row and 32 columns (what the scaled MFMA of the next
+// GEMM takes), instead of 16-bit values that a quantiser launch would read
+// back.  A lane holds 16 of the 32 columns of one row of a block; the other 16
+// sit in the lane 32 on.  Per block, from the activation value rounded to the
+// 16-bit type (so that the bytes are a function of the h the 16-bit epilogue
+// would have written):
+//   amax = max |h|;  t = amax * fp32(1 / 448);  e = exponent field of t, plus one
+//   if t is not a power of two (2^(e - 127) >= amax / 448);  byte = e4m3(rne(h * 2^(127 - e)))
+// A block that holds a NaN or an infinity becomes NaN bytes with scale 1.
+// Scale bytes go to cscale[((column / 128) * scale_rows + row) * 4 + block_scale_pos(column / 32)]
+// (cscale: the dword of the tile's first row in the first step).
+// The sums are in the accumulation registers (block (i, j) = a[16 (i TN + j) ..]).
+template <int MODE, int WAVES, int TN, int RESERVE>
+struct BlockqGeom {
+  static constexpr int OUT_BLOCKS = MODE == kFc1Swiglu ? TN / 2 : TN, OUT_COLS = OUT_BLOCKS * 32, PITCH = OUT_COLS + 16;
+  // rows of a block staged at a time (RESERVE: bytes of the staging area that other tables take)
+  static constexpr int BAND = (WAVES * 32 * PITCH + RESERVE <= kPStageArea) ? 32 : 16;
+  static constexpr int WAVE_BYTES = BAND * PITCH;
+  static_assert(WAVES * WAVE_BYTES + RESERVE <= kPStageArea, "staging area too small");
+};
+template <int MODE, int WAVES, int TM, int TN, bool BIAS_LDS, int ROW_STRIDE, int RESERVE>
+__device__ __forceinline__ void tile_epilogue_blockq(const Tile &cp, unsigned char *stage, int wave_row0, int wave_col0,
+                                                     int lane, const float *scale_lds, const float *rowscale_lds,
+                                                     const float *bias_lds, int live_blocks, unsigned char *cscale,
+                                                     uint32_t scale_rows) {
+  constexpr bool SWIGLU = MODE == kFc1Swiglu;
+  using G = BlockqGeom<MODE, WAVES, TN, RESERVE>;
+  constexpr int OUT_BLOCKS = G::OUT_BLOCKS, OUT_COLS = G::OUT_COLS, PITCH = G::PITCH, BAND = G::BAND;
+  constexpr int LANES_PER_ROW = OUT_COLS / 16, ROWS_PER_PASS = kWave / LANES_PER_ROW, PASSES = BAND / ROWS_PER_PASS;
+  static_assert(PASSES >= 1 && BAND % ROWS_PER_PASS == 0, "whole store passes");
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  const int rd_row = lane / LANES_PER_ROW, rd_chunk = lane % LANES_PER_ROW;
+  const __amdgpu_buffer_rsrc_t crs =
+      __builtin_amdgcn_make_buffer_rsrc((void *)uni(cp.c), 0, uni(cp.c_bytes), kRsrcFlags);
+  const __amdgpu_buffer_rsrc_t srs = __builtin_amdgcn_make_buffer_rsrc(
+      (void *)uni(cscale), 0, uni((uint32_t)((cp.n + 127) >> 7) * scale_rows * 4u), kRsrcFlags);   // (rows are checked below)
+  const int col_base = cp.n0 + wave_col0;
+  static_for<TM>([&](auto i_c) {
+    constexpr int i = decltype(i_c)::value;
+    if (i >= live_blocks) return;
+    const float row_scale = rowscale_lds[wave_row0 + i * ROW_STRIDE + frag_row];
+    uint32_t packed[OUT_BLOCKS][4];
+    static_for<OUT_BLOCKS>([&](auto j_c) {
+      constexpr int j = decltype(j_c)::value;
+      f32x16_t blk = fixed_acc_block<i * TN + j>(), up;
+      if constexpr (SWIGLU) up = fixed_acc_block<i * TN + j + OUT_BLOCKS>();
+      uint32_t amax_bits = 0;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float *sp = scale_lds + wave_col0 + j * 32 + frag_half * 4 + q * 8;
+        f32x4_t sg = *reinterpret_cast<const f32x4_t *>(sp), su, sb;
+        sg *= row_scale;
+        if (SWIGLU) su = *reinterpret_cast<const f32x4_t *>(sp + 128) * row_scale;
+        if (BIAS_LDS) sb = *reinterpret_cast<const f32x4_t *>(bias_lds + wave_col0 + j * 32 + frag_half * 4 + q * 8);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float v = blk[q * 4 + r] * sg[r];
+          if (SWIGLU) {
+            v = silu_fast(v) * (up[q * 4 + r] * su[r]);
+          } else {
+            if (BIAS_LDS) v += sb[r];
+            if (MODE == kFc1Gelu) v = gelu_tanh_fast(v);
+          }
+          v = (float)(h16_t)v;
+          blk[q * 4 + r] = v;
+          const uint32_t mag = __float_as_uint(v) & 0x7fffffffu;
+          amax_bits = mag > amax_bits ? mag : amax_bits;   // (non-negative floats order like their bits; NaN above all)
+        }
+      }
+      // (the row's other 16 columns sit in the lane 32 on: one swap of the lane halves of two copies, then
+      // every lane holds both maxima)
+      {
+        const auto both = __builtin_amdgcn_permlane32_swap(amax_bits, amax_bits, false, false);
+        amax_bits = both[0] > both[1] ? both[0] : both[1];
+      }
+      const bool bad = amax_bits >= 0x7f800000u;
+      const uint32_t tb = __float_as_uint(__uint_as_float(amax_bits) * (1.0f / 448.0f));
+      uint32_t e = (tb >> 23) + ((tb & 0x7fffffu) != 0 ? 1u : 0u);
+      e = bad ? 127u : e;
+      const float inv = __uint_as_float((254u - e) << 23);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float f[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) f[r] = __builtin_amdgcn_fmed3f(blk[q * 4 + r] * inv, -448.f, 448.f);
+        int w = 0;
+        w = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], w, false);
+        w = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], w, true);
+        packed[j][q] = bad ? 0x7f7f7f7fu : (uint32_t)w;
+      }
+      const int n = col_base + j * 32;
+      const int m = wave_row0 + i * ROW_STRIDE + frag_row;
+      const uint32_t voff =
+          (frag_half == 0 && n < cp.n && m < cp.rows) ? (uint32_t)m * 4u + (uint32_t)block_scale_pos(n >> 5) : kOutOfRange;
+      __builtin_amdgcn_raw_buffer_store_b8((unsigned char)e, srs, voff, uni((uint32_t)(n >> 7) * scale_rows * 4u), 0);
+    });
+#pragma unroll
+    for (int band = 0; band < 32 / BAND; ++band) {
+      if (BAND == 32 || (frag_row >> 4) == band) {
+#pragma unroll
+        for (int j = 0; j < OUT_BLOCKS; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            *reinterpret_cast<uint32_t *>(stage + (frag_row & (BAND - 1)) * PITCH + j * 32 + q * 8 + frag_half * 4) =
+                packed[j][q];
+      }
+      wave_lds_sync();
+#pragma unroll
+      for (int ps = 0; ps < PASSES; ++ps) {
+        const int r = ps * ROWS_PER_PASS + rd_row;
+        const u32x4_t v = *reinterpret_cast<const u32x4_any_t *>(stage + r * PITCH + rd_chunk * 16);
+        const int m = wave_row0 + i * ROW_STRIDE + band * BAND + r;
+        const int n = col_base + rd_chunk * 16;
+        const uint32_t voff = n < cp.n ? (uint32_t)m * cp.c_pitch + (uint32_t)n : kOutOfRange;
+        __builtin_amdgcn_raw_buffer_store_b128(v, crs, voff, 0, 0);
+      }
+      wave_lds_sync();   // the next rows overwrite the staging rows
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  });
 }
 
 // ---------------------------------------------------------------------------
@@ -1152,6 +1286,7 @@ void launch_split_sum(const PersistBatch &launch, int grid, int bk, hipStream_t 
 // What the kernels whose k-loop is generated assembly share (gen_persist64_asm.py
 // writes persist64_asm.inc into the build directory).
 #define DICE_MFMA8 "v_mfma_f32_32x32x64_f8f6f4"
+#define DICE_MFMA8_SCALED "v_mfma_scale_f32_32x32x64_f8f6f4"
 // One global memory -> LDS instruction (16 bytes per lane, no register in
 // between) as text.  A load the compiler knows of would have it wait for "its
 // only load" with vmcnt(0) before the next LDS access of its own - which drains
@@ -1193,6 +1328,32 @@ struct P64Addr {
     [va7] "v"(ad.va[7]), [vb] "v"(ad.vb), [dA] "s"(dA), [dB0] "s"(dB0), [dB1] "s"(dB1), [koff] "s"(koff),       \
     [sb0] "s"(sb[0]), [sb1] "s"(sb[1]), [sb2] "s"(sb[2]), [sb3] "s"(sb[3]), [sb4] "s"(sb[4]), [sb5] "s"(sb[5]), \
     [sb6] "s"(sb[6]), [sb7] "s"(sb[7])                                                                          \
+  : "memory"
+// The kernel for block-scaled fp8 activations also passes: the byte offset of this lane's row of block scales in
+// the tile being loaded (vs), the LDS address its scales go to (wrs; slot 1 lies 1 KB on) and the one it reads its
+// rows' scales from (rs), the descriptor of the tile's scales (dS) and the step's offset in a row of them (kso).
+// The text also names v117..v127 (the scales' register stage, the scales of the step's row blocks, the weights'
+// scale), which the compiler must not use: it allocates from v0 upwards and parks scalar registers in the lanes of
+// the first vector registers past those - the build-time check of the device assembly (check_acc_regs.py) fails an
+// instantiation in which either reaches v117.  (A value pinned to these registers and passed through every
+// statement does not keep them free: the compiler moves it out and back around the epilogue.)
+struct P64ScaleAddr {
+  uint32_t vs, wrs, rs;
+};
+#define P64S_PARAMS P64_PARAMS, const P64ScaleAddr &sa, u32x4_t dS, uint32_t kso
+#define P64S_ARGS P64_ARGS, sa, dS, kso
+#define P64S_CONSTRAINTS                                                                                        \
+  : "+{v[0:31]}"(f0), "+{v[32:63]}"(f1)                                                                         \
+  : [wr0] "v"(ad.wr[0]), [wr1] "v"(ad.wr[1]), [ra00] "v"(ad.ra[0][0]), [ra01] "v"(ad.ra[0][1]),                 \
+    [ra02] "v"(ad.ra[0][2]), [ra03] "v"(ad.ra[0][3]), [ra10] "v"(ad.ra[1][0]), [ra11] "v"(ad.ra[1][1]),         \
+    [ra12] "v"(ad.ra[1][2]), [ra13] "v"(ad.ra[1][3]), [rb00] "v"(ad.rb[0][0]), [rb01] "v"(ad.rb[0][1]),         \
+    [rb02] "v"(ad.rb[0][2]), [rb03] "v"(ad.rb[0][3]), [rb10] "v"(ad.rb[1][0]), [rb11] "v"(ad.rb[1][1]),         \
+    [rb12] "v"(ad.rb[1][2]), [rb13] "v"(ad.rb[1][3]), [va0] "v"(ad.va[0]), [va1] "v"(ad.va[1]),                 \
+    [va2] "v"(ad.va[2]), [va3] "v"(ad.va[3]), [va4] "v"(ad.va[4]), [va5] "v"(ad.va[5]), [va6] "v"(ad.va[6]),    \
+    [va7] "v"(ad.va[7]), [vb] "v"(ad.vb), [dA] "s"(dA), [dB0] "s"(dB0), [dB1] "s"(dB1), [koff] "s"(koff),       \
+    [sb0] "s"(sb[0]), [sb1] "s"(sb[1]), [sb2] "s"(sb[2]), [sb3] "s"(sb[3]), [sb4] "s"(sb[4]), [sb5] "s"(sb[5]), \
+    [sb6] "s"(sb[6]), [sb7] "s"(sb[7]), [vs] "v"(sa.vs), [wrs] "v"(sa.wrs), [rs] "v"(sa.rs), [dS] "s"(dS),      \
+    [kso] "s"(kso)                                                                                              \
   : "memory"
 typedef float f32x32_t __attribute__((ext_vector_type(32)));
 #include "persist64_asm.inc"

@@ -139,7 +139,7 @@ def load() -> ctypes.CDLL:
     lib.dice_grouped_mlp_a8.restype = c_int
     lib.dice_grouped_mlp_a8.argtypes = [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int64, c_int,
                                         c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
-                                        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+                                        c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
     lib.dice_moe_workspace_bytes.restype = c_size_t
     lib.dice_moe_workspace_bytes.argtypes = [POINTER(MoeLayerDesc), c_int64]
     lib.dice_moe_forward.restype = c_int

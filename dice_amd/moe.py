@@ -196,7 +196,7 @@ class SparseMoeBlock(nn.Module):
         self.inter = inter
         self._packed: Optional[_Packed] = None
         self._fp8 = False
-        self._act_quant = False      # fp8 experts: activations quantised per row too (fp8 matrix pipe)
+        self._act_quant = 0          # fp8 experts: 1 activations quantised per row too (fp8 matrix pipe), 2 h in blocks
         # True: a token's result never depends on what else is in the call (no fc2 tile is cut along k; see
         # dice_moe_layer_t.batch_invariant).  Set it before the first call, or clear ``_desc`` after changing it.
         self.batch_invariant = False
@@ -264,11 +264,16 @@ class SparseMoeBlock(nn.Module):
         self._desc = None
         return p
 
-    def quantize_fp8(self, activations: bool = False):
+    def quantize_fp8(self, activations: bool = False, h_blocks: bool = False):
         """Switches the routed experts to e4m3 weights (build-defined path).
         ``activations=True`` also quantises the routed experts' input rows (per
         token, dynamically, in front of each GEMM), so that the products run on
-        the fp8 matrix pipe; bf16 blocks whose widths are multiples of 256."""
+        the fp8 matrix pipe; bf16 blocks whose widths are multiples of 256.
+        ``h_blocks=True`` (with ``activations``) has fc1's epilogue quantise h
+        itself, with one power-of-two scale per row and 32 columns, instead of
+        a quantiser launch with one scale per row."""
+        if h_blocks and not activations:
+            raise DiceError("quantize_fp8(h_blocks=True) needs activations=True")
         if activations:
             # what the fp8 matrix-pipe kernels and the row quantiser take; refused here, not at the first forward
             for name, width in (("hidden", self.embed_dim), ("expert", self.inter)):
@@ -279,7 +284,7 @@ class SparseMoeBlock(nn.Module):
                 raise DiceError("quantize_fp8(activations=True): act_quant (the fp8 matrix-pipe path) takes bf16 "
                                 "blocks; use quantize_fp8() (e4m3 weights, 16-bit activations)")
         self.pack_weights(fp8=True)
-        self._act_quant = bool(activations)
+        self._act_quant = (2 if h_blocks else 1) if activations else 0
         self._desc = None
         return self
 
@@ -296,7 +301,7 @@ class SparseMoeBlock(nn.Module):
             if out is None:
                 out = torch.zeros((max(max_rows, 1), self.embed_dim), dtype=x.dtype, device=x.device)
             rows, _ = ops.grouped_mlp_a8(x, perm, k, offsets, max_rows, p.w1, p.w2, p.w1_scale, p.w2_scale,
-                                         self.variant, p.b1, p.b2, out=out)
+                                         self.variant, p.b1, p.b2, out=out, h_blocks=self._act_quant == 2)
             return rows
         return ops.grouped_mlp(x, perm, k, offsets, max_rows, p.w1, p.w2, self.variant, p.b1, p.b2,
                                p.w1_scale, p.w2_scale, scatter_to_slots=False, n_out_rows=max(max_rows, 1), out=out)
@@ -322,7 +327,7 @@ class SparseMoeBlock(nn.Module):
             d.w1_scale, d.w2_scale = ptr(p.w1_scale), ptr(p.w2_scale)
             d.shared_w1, d.shared_w2 = ptr(p.sw1), ptr(p.sw2)
             d.shared_b1, d.shared_b2 = ptr(p.sb1), ptr(p.sb2)
-            d.act_quant = int(self._act_quant and self._fp8)
+            d.act_quant = int(self._act_quant) if self._fp8 else 0
             d.batch_invariant = int(self.batch_invariant)
             self._desc = d
         return self._desc

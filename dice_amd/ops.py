@@ -183,10 +183,15 @@ def quantize_fp8_act(x: torch.Tensor, perm: Optional[torch.Tensor] = None, slots
 def grouped_mlp_a8(x: torch.Tensor, perm: Optional[torch.Tensor], slots_per_token: int,
                    offsets: torch.Tensor, max_rows: int, w1: torch.Tensor, w2: torch.Tensor,
                    w1_scale: torch.Tensor, w2_scale: torch.Tensor, variant: str = "swiglu", b1=None, b2=None,
-                   stages: int = 3, h: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None):
+                   stages: int = 3, h: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                   h_blocks: bool = False):
     """Grouped expert MLP with e4m3 weights AND per-row e4m3 activations on the
     fp8 matrix pipe (``dice_grouped_mlp_a8``).  Returns ``(out [max_rows, D]
-    grouped, h [max_rows, I])`` in bf16."""
+    grouped, h [max_rows, I])`` in bf16.  ``h_blocks``: fc1's epilogue writes h
+    as e4m3 bytes with one power-of-two scale per row and 32 columns (no
+    quantiser launch between the GEMMs); the buffer ``h`` then holds
+    ``[max_rows, I]`` bytes followed (from the next multiple of 256 bytes) by
+    ``[I / 128, max_rows, 4]`` scale bytes, see ``split_h_blocks``."""
     e, d, inter = w2.shape
     if h is None:
         h = torch.empty((max(max_rows, 1), inter), dtype=x.dtype, device=x.device)
@@ -196,6 +201,37 @@ def grouped_mlp_a8(x: torch.Tensor, perm: Optional[torch.Tensor], slots_per_toke
     q_scale = torch.empty((max(max_rows, 1),), dtype=torch.float32, device=x.device)
     check(load().dice_grouped_mlp_a8(
         stages, ptr(x), dtype_code(x.dtype), ptr(perm), slots_per_token, ptr(offsets), e, max_rows, d, inter,
-        ptr(w1), ptr(b1), ptr(w2), ptr(b2), ptr(w1_scale), ptr(w2_scale), VARIANTS[variant], ptr(h), ptr(out),
-        ptr(q_rows), ptr(q_scale), stream_ptr()))
+        ptr(w1), ptr(b1), ptr(w2), ptr(b2), ptr(w1_scale), ptr(w2_scale), VARIANTS[variant], int(h_blocks),
+        ptr(h), ptr(out), ptr(q_rows), ptr(q_scale), stream_ptr()))
     return out, h
+
+
+def block_scale_order(n_blocks: int) -> torch.Tensor:
+    """Where each 32-column block's scale byte sits among its row's: the four scales of 128 columns are one
+    dword, stored in the order 0, 2, 1, 3 (``block_scale_pos`` of the library)."""
+    cb = torch.arange(n_blocks)
+    return (cb & ~3) | ((cb & 1) << 1) | ((cb >> 1) & 1)
+
+
+def split_h_blocks(h: torch.Tensor, max_rows: int, inter: int):
+    """The two parts of an h buffer written with ``h_blocks``: ``(bytes [max_rows, I] uint8 (e4m3),
+    exponents [max_rows, I / 32] uint8 in column order)``; a block's values are byte * 2^(exponent - 127)."""
+    flat = h.view(torch.uint8).reshape(-1)
+    q = flat[:max_rows * inter].view(max_rows, inter)
+    start = (max_rows * inter + 255) // 256 * 256
+    # stored [I / 128][max_rows][4]: the dwords of a 128-column step are adjacent row after row
+    sc = flat[start:start + max_rows * (inter // 32)].view(inter // 128, max_rows, 4).permute(1, 0, 2)
+    sc = sc.reshape(max_rows, inter // 32)
+    return q, sc[:, block_scale_order(inter // 32).to(sc.device)]
+
+
+def join_h_blocks(h: torch.Tensor, q: torch.Tensor, exponents: torch.Tensor):
+    """Writes e4m3 bytes and per-block exponents (column order) into an h buffer in the layout fc2 reads."""
+    max_rows, inter = q.shape
+    flat = h.view(torch.uint8).reshape(-1)
+    flat[:max_rows * inter] = q.reshape(-1)
+    start = (max_rows * inter + 255) // 256 * 256
+    stored = torch.empty_like(exponents)
+    stored[:, block_scale_order(inter // 32).to(exponents.device)] = exponents
+    flat[start:start + stored.numel()] = stored.view(max_rows, inter // 128, 4).permute(1, 0, 2).reshape(-1)
+    return h

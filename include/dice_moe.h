@@ -225,6 +225,18 @@ int dice_quantize_fp8_act(const void *x, int in_dtype, const int32_t *perm,
  * lines as dice_grouped_mlp (models.py:252-273, 368-377); the quantisation is
  * build-defined.
  *   stages   1 = fc1 (writes h), 2 = fc2 (reads h), 3 = both
+ *   h_blocks 0: h is BF16 and a quantiser launch (one scale per row) runs in
+ *            front of fc2.  1: fc1's epilogue quantises h itself, from the
+ *            value rounded to BF16, with one power-of-two scale per row and
+ *            32 columns:  t = amax * fp32(1/448);  e = exponent field of t,
+ *            plus one unless t is a power of two;  byte = e4m3(rne(h *
+ *            2^(127 - e)))  (a block with a NaN or an infinity: NaN bytes,
+ *            e = 127).  fc2 multiplies with v_mfma_scale_f32_32x32x64_f8f6f4,
+ *            which applies 2^(e - 127) to the block.  The buffer h then holds
+ *            [max_rows, inter] bytes and, from the next multiple of 256
+ *            bytes, [inter / 128, max_rows, 4] bytes e (the four of a row's
+ *            128 columns in the order 0, 2, 1, 3); no more than 64 tiles of
+ *            256 x 256 per compute unit in fc2.
  *   q_rows   [max_rows, max(hidden, inter)] bytes of scratch (the fp8 rows)
  *   q_scale  [max_rows] floats of scratch (their scales)
  * Output rows are in grouped order.  Limits: act_dtype BF16, hidden and inter
@@ -235,8 +247,9 @@ int dice_grouped_mlp_a8(int stages, const void *x, int act_dtype,
                         const int32_t *offsets, int n_experts, int64_t max_rows,
                         int hidden, int inter, const void *w1, const float *b1,
                         const void *w2, const float *b2, const float *w1_scale,
-                        const float *w2_scale, int act_variant, void *h,
-                        void *out, uint8_t *q_rows, float *q_scale, void *stream);
+                        const float *w2_scale, int act_variant, int h_blocks,
+                        void *h, void *out, uint8_t *q_rows, float *q_scale,
+                        void *stream);
 
 /*
  * Whole layer.  Replaces SparseMoeBlock.forward, inference branch
@@ -259,7 +272,10 @@ typedef struct dice_moe_layer {
   const float *b1, *b2, *w1_scale, *w2_scale;
   const void *shared_w1, *shared_w2; /* one expert, act_dtype */
   const float *shared_b1, *shared_b2;
-  int32_t act_quant;      /* 0: 16-bit activations (fp8 weights are widened and
+  int32_t act_quant;      /* 2: as 1, with h quantised inside fc1's epilogue
+                           * (h_blocks of dice_grouped_mlp_a8) instead of by a
+                           * launch of its own.
+                           * 0: 16-bit activations (fp8 weights are widened and
                            * multiplied on the 16-bit matrix pipe); 1: the routed
                            * experts' activations are quantised per row to e4m3
                            * on the way into each GEMM (dice_quantize_fp8_act)

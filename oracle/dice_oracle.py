@@ -806,15 +806,48 @@ def quantize_fp8_act(x: torch.Tensor):
     return q, scale
 
 
+def quantize_fp8_act_blocks(h: torch.Tensor):
+    """Quantisation of activation rows to OCP e4m3fn with one power-of-two scale
+    per row and 32 columns, as the fp8 fc1 kernel's epilogue writes h for the
+    scaled MFMA of fc2 (build-defined):  ``amax = max|block|``;
+    ``t = amax * fp32(1/448)`` (one fp32 rounding);  ``e`` = the exponent field
+    of ``t``, plus one unless ``t`` is a power of two (or zero), so that
+    ``2^(e-127) >= t``;  ``byte = e4m3(rne(h * 2^(127-e)))``, clamped to +-448.
+    A block that holds a NaN or an infinity becomes NaN bytes with ``e = 127``.
+    Returns (q float8_e4m3fn [rows, cols], e uint8 [rows, cols / 32])."""
+    hf = h.float()
+    rows, cols = hf.shape
+    blk = hf.view(rows, cols // 32, 32)
+    amax = blk.abs().amax(dim=-1)
+    t = amax * torch.tensor(1.0 / 448.0, dtype=torch.float32)
+    bits = t.view(torch.int32)
+    e = (bits >> 23) + ((bits & 0x7FFFFF) != 0).to(torch.int32)
+    bad = ~torch.isfinite(blk).all(dim=-1)
+    e = torch.where(bad, torch.full_like(e, 127), e)
+    inv = ((254 - e) << 23).view(torch.float32)
+    q = (blk * inv[..., None]).clamp(-E4M3_MAX, E4M3_MAX)
+    q = torch.where(bad[..., None], torch.full_like(q, float("nan")), q)
+    return q.reshape(rows, cols).to(torch.float8_e4m3fn), e.to(torch.uint8)
+
+
+def dequantize_fp8_act_blocks(q: torch.Tensor, e: torch.Tensor) -> torch.Tensor:
+    rows, cols = q.shape
+    scale = torch.ldexp(torch.ones((), dtype=torch.float32), e.to(torch.int32) - 127)
+    return (q.float().view(rows, cols // 32, 32) * scale[..., None]).reshape(rows, cols)
+
+
 class Fp8ActExpert:
     """An expert whose two GEMMs take e4m3 weights (``quantize_fp8_rowwise``
     of the master weights) AND e4m3 activations (``quantize_fp8_act`` of the
     rows in front of each GEMM).  Products and sums in fp32, the row's and the
     output channel's scale applied to the sums, the activation function in fp32,
     one rounding to the activation dtype for ``h`` and for the output - the
-    arithmetic of the fp8 kernels.  Wraps a ``SwiGLUExpert`` or ``GeluExpert``."""
+    arithmetic of the fp8 kernels.  Wraps a ``SwiGLUExpert`` or ``GeluExpert``.
+    ``h_blocks``: ``h`` is quantised with ``quantize_fp8_act_blocks`` (from its
+    value rounded to the activation dtype) instead of per row."""
 
-    def __init__(self, master):
+    def __init__(self, master, h_blocks: bool = False):
+        self.h_blocks = h_blocks
         self.swiglu = isinstance(master, SwiGLUExpert)
         if self.swiglu:
             w1 = torch.cat([master.gate_proj, master.up_proj], 0)
@@ -841,8 +874,11 @@ class Fp8ActExpert:
 
     def __call__(self, x: torch.Tensor) -> torch.Tensor:
         h = self.hidden_act(x)
-        qh, sh = quantize_fp8_act(h)
-        o = (qh.float() @ self.q2.float().t()) * (sh[:, None] * self.s2[None, :])
+        if self.h_blocks:
+            o = (dequantize_fp8_act_blocks(*quantize_fp8_act_blocks(h)) @ self.q2.float().t()) * self.s2[None, :]
+        else:
+            qh, sh = quantize_fp8_act(h)
+            o = (qh.float() @ self.q2.float().t()) * (sh[:, None] * self.s2[None, :])
         if self.b2 is not None:
             o = o + self.b2
         return o.to(x.dtype)

@@ -38,6 +38,8 @@ class Replay:
     def __init__(self, kind_desc):
         self.k = kind_desc
         self.f8 = bool(kind_desc.get("f8"))
+        self.scaled = bool(kind_desc.get("scaled"))
+        self.scale_slot_written = [False, False]
         self.lds_issued = self.lds_done = 0
         self.vm_issued = self.vm_done = 0
         self.frag_ready = {}      # first register of a 16-byte fragment part -> index of the LDS read filling it
@@ -72,9 +74,15 @@ class Replay:
                     self.vm_done = max(self.vm_done, self.vm_issued - int(m.group(2)))
             elif op == "s_barrier":
                 assert self.lds_done == self.lds_issued, "barrier with LDS operations in flight"
-            elif op in ("MFMA", "MFMA8"):
-                assert (op == "MFMA8") == self.f8
+            elif op in ("MFMA", "MFMA8", "MFMA8S"):
+                assert (op != "MFMA") == self.f8 and (op == "MFMA8S") == self.scaled
                 parts = 2 if self.f8 else 1
+                scale_args = None
+                if self.scaled:       # ..., C, weights' scale, activations' scale op_sel:[0,kb,0] op_sel_hi:[0,0,0]
+                    m = re.fullmatch(r"v(\d+) op_sel:\[0,([01]),0\] op_sel_hi:\[0,0,0\]", ",".join(args[5:]))
+                    assert m and args[4] == "v127", ln
+                    scale_args = (int(m.group(1)), int(m.group(2)))
+                    args = args[:4]
                 (fa, a0, a1), (_, w0, w1), (_, r0, r1) = _regs(args[0]), _regs(args[1]), _regs(args[2])
                 assert fa == "a" and a1 - a0 == 15 and a0 % 16 == 0 and a1 < 256
                 assert w1 - w0 == 4 * parts - 1 and r1 - r0 == 4 * parts - 1 and w1 < 64 and r1 < 64
@@ -88,6 +96,12 @@ class Replay:
                 if self.f8:      # address index kk = 2 kb + t
                     assert tw[0][0] == tw[1][0] and tw[0][1] % 2 == 0 and tw[1][1] == tw[0][1] + 1, tw
                     self.blocks.append((tw[0][0], tw[0][1] // 2))
+                    if self.scaled:
+                        # the scale register holds this row block's scales of the fragments' slot, its read
+                        # has completed, and op_sel picks the fragments' k-block
+                        reg, byte = scale_args
+                        assert self.frag_ready[reg] < self.lds_done, f"{ln}: scales still in flight"
+                        assert self.frag_tag[reg] == ("s", tw[0][0], i) and byte == tw[0][1] // 2, ln
                 else:
                     self.blocks.append(tw[0])
                 self.mfma += 1
@@ -99,6 +113,37 @@ class Replay:
                 self.frag_ready[d0] = self.lds_issued
                 self.frag_tag[d0] = (m.group(1), int(m.group(2)), int(m.group(3)), int(m.group(4)))
                 self.lds_issued += 1
+            elif op == "ds_read_u16":
+                m = re.fullmatch(r"v(\d+)", args[0])
+                m2 = re.fullmatch(r"%\[rs\] offset:(\d+)", args[1])
+                assert self.scaled and m and m2, ln
+                reg, off = int(m.group(1)), int(m2.group(1))
+                slot, i = divmod(off, 1024)
+                assert i % 256 == 0 and reg == 119 + 4 * slot + i // 256 and slot < 2 and i // 256 < 4, ln
+                # (the slot's table must hold the step's scales: sent there by an LDS write issued earlier)
+                assert self.scale_slot_written[slot], f"{ln}: the slot's scales were never written"
+                self.frag_ready[reg] = self.lds_issued
+                self.frag_tag[reg] = ("s", slot, i // 256)
+                self.lds_issued += 1
+            elif op == "ds_write_b32":
+                m = re.fullmatch(r"%\[wrs\]", args[0])
+                m2 = re.fullmatch(r"v(\d+) offset:(\d+)", args[1])
+                assert self.scaled and m and m2, ln
+                reg, off = int(m2.group(1)), int(m2.group(2))
+                assert reg in (117, 118) and off == 1024 * (reg - 117), ln
+                assert reg in self.stage_ready and self.stage_ready[reg] < self.vm_done, f"{ln}: load in flight"
+                self.stage_sent[reg] = True
+                self.scale_slot_written[reg - 117] = True
+                self.lds_issued += 1
+            elif op == "buffer_load_dword":
+                m = re.fullmatch(r"v(\d+)", args[0])
+                assert self.scaled and m and int(m.group(1)) in (117, 118), ln
+                assert [a.split(" ")[0] for a in args[1:]] == ["%[vs]", "%[dS]", "%[kso]"], ln
+                reg = int(m.group(1))
+                assert self.stage_sent.get(reg, True), f"{ln}: refilled before it was sent to LDS"
+                self.stage_ready[reg] = self.vm_issued
+                self.stage_sent[reg] = False
+                self.vm_issued += 1
             elif op == "ds_write_b128":
                 _, d0, d1 = _regs(args[1].split(" ")[0])
                 assert d1 - d0 == 3 and 128 <= d0 and d1 < 256
@@ -117,7 +162,7 @@ class Replay:
                 raise AssertionError(f"unexpected instruction {ln}")
 
 
-@pytest.mark.parametrize("kind", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("kind", [0, 1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("live", [1, 2, 3, 4])
 def test_generated_loop_waits_cover_every_dependence(kind, live):
     gen = _load()
@@ -147,13 +192,15 @@ def test_generated_loop_waits_cover_every_dependence(kind, live):
         r.lds_done = r.lds_issued                  # the epilogue drains the LDS queue; vector loads stay in flight
         r.vm_issued += 24                          # ... and issues stores of its own: waits only get stricter
     # the first step of a tile starts the sums, every later one adds to them
+    def starts(ln):      # the product's C operand is the constant 0
+        return ln.split(",")[3].strip() == "0"
     first = [ln for ln in pcs["abc_s0_v1"] if ln.startswith("MFMA")]
-    assert all(ln.endswith(", 0") for ln in first[:live * tn])
-    assert not any(ln.endswith(", 0") for ln in first[live * tn:])
+    assert all(starts(ln) for ln in first[:live * tn])
+    assert not any(starts(ln) for ln in first[live * tn:])
     # every block of sums is started exactly once per tile
     started = sorted(ln.split(",")[0] for ln in first[:live * tn])
     assert len(set(started)) == live * tn
-    assert not any(ln.endswith(", 0") for ln in pcs["abc_s0_v0"] if ln.startswith("MFMA"))
+    assert not any(starts(ln) for ln in pcs["abc_s0_v0"] if ln.startswith("MFMA"))
 
 
 def test_generated_text_names_only_planned_registers():
@@ -163,9 +210,12 @@ def test_generated_text_names_only_planned_registers():
     for m in re.finditer(r"\bv\[(\d+):(\d+)\]", text):
         lo, hi = int(m.group(1)), int(m.group(2))
         assert hi < 64 or lo >= 128, m.group(0)     # fragments or stages, never the compiler's v64..v127
+    # single registers: only the scaled kind's (its kernel leaves v117..v127 to the text)
+    singles = {int(m.group(1)) for m in re.finditer(r"\bv(\d+)\b", text)}
+    assert singles and singles <= set(range(117, 128)), singles
     # every instruction of the text is one of these (the replay above refuses anything else, too)
     allowed = {"s_waitcnt", "s_barrier", "ds_read_b128", "ds_write_b128", "buffer_load_dwordx4", "DICE_MFMA16",
-               "DICE_MFMA8"}
+               "DICE_MFMA8", "DICE_MFMA8_SCALED", "ds_read_u16", "ds_write_b32", "buffer_load_dword"}
     for m in re.finditer(r'^\s*"(?:" )?([A-Za-z_0-9]+)', text, re.M):
         assert m.group(1) in allowed, m.group(0)
 

@@ -171,9 +171,9 @@ def test_mlp_a8_matches_oracle(dev, variant, D, ratio, E, counts):
     assert 1e-2 < rel_l2(out, master) < 0.1
 
 
-def _a8_oracle(p):
+def _a8_oracle(p, h_blocks=False):
     p8 = copy.copy(p)
-    p8.experts = [O.Fp8ActExpert(e) for e in p.experts]
+    p8.experts = [O.Fp8ActExpert(e, h_blocks=h_blocks) for e in p.experts]
     return p8
 
 
@@ -204,7 +204,8 @@ def test_block_c5_a8_full_size(dev, variant, n_shared):
     assert not torch.equal(y16, y)
 
 
-def test_block_a8_staleness_identities(dev):
+@pytest.mark.parametrize("h_blocks", [False, True])
+def test_block_a8_staleness_identities(dev, h_blocks):
     """Put and skip steps with fp8 activations: a put step returns the plain
     step's rows, a skip step fed its own cache reproduces them (the recomputed
     slot's rows are quantised row by row, so dropping the other slot changes
@@ -215,7 +216,7 @@ def test_block_a8_staleness_identities(dev):
     p = O.make_block_params(D, E, 2, 4, 2, seed=11, dtype=torch.bfloat16, gate_bias=zipf_bias(E, 3.0))
     x = torch.randn(N, D, generator=_gen(12)).bfloat16().to(dev)
     blk = block_from_params(p, D, "swiglu", torch.bfloat16, dev)
-    blk.quantize_fp8(activations=True)
+    blk.quantize_fp8(activations=True, h_blocks=h_blocks)
     # Bit-identity needs whole fc2 tiles: by default a short last turn is cut along
     # k, a skip step has half the rows and so another cut, and sums of 16-bit pieces
     # differ from a whole tile's in the last bit (tests/test_gpu_split_turn.py).
@@ -238,7 +239,7 @@ def test_block_a8_staleness_identities(dev):
     assert torch.equal(put, blk.run(x))
     check_rows(blk.run(x, lib.MODE_SKIP, mask, cache, None).cpu(), put.cpu(), 4e-3, "skip step on its own cache")
     check_rows(put.cpu(), plain.cpu(), 4e-3, "cut last turn vs whole tiles")
-    want, _, _, logits = O.sparse_moe_block_forward(_a8_oracle(p), x.cpu().view(1, N, D))
+    want, _, _, logits = O.sparse_moe_block_forward(_a8_oracle(p, h_blocks), x.cpu().view(1, N, D))
     ok = ~O.gate_tie_rows(logits, 2).view(-1)
     check_rows(plain.cpu()[ok], want.view(-1, D)[ok], SAME_QUANT_TOL, "zipf-loaded fp8 x fp8 block")
 
@@ -259,7 +260,8 @@ def test_act_quant_needs_fp8_weights_and_bf16(dev):
     assert blk(torch.zeros(1, 64, 1152, dtype=torch.bfloat16, device=dev)).shape == (1, 64, 1152)
 
 
-def test_block_a8_one_arithmetic_behind_every_entry_point(dev):
+@pytest.mark.parametrize("h_blocks", [False, True])
+def test_block_a8_one_arithmetic_behind_every_entry_point(dev, h_blocks):
     """A block that quantises its activations computes its routed experts on the
     fp8 matrix pipe whichever way it is entered: SparseMoeBlock.moe_infer
     (models.py:361-382) and moe_infer_ep (expertpara/ep_fwd.py:19) with the
@@ -274,8 +276,8 @@ def test_block_a8_one_arithmetic_behind_every_entry_point(dev):
     idx = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(N)]).view(-1)
     w = torch.rand(N * k, 1, generator=g).bfloat16()
     blk = block_from_params(p, D, "swiglu", torch.bfloat16, dev, para_mode=ParaMode(ep=True))
-    blk.quantize_fp8(activations=True)
-    want = O.moe_infer(x, _a8_oracle(p).experts, idx, w, k)
+    blk.quantize_fp8(activations=True, h_blocks=h_blocks)
+    want = O.moe_infer(x, _a8_oracle(p, h_blocks).experts, idx, w, k)
     y = blk.moe_infer(x.to(dev), idx.to(dev), w.to(dev)).cpu()
     check_rows(y, want, SAME_QUANT_TOL, "moe_infer on the fp8 matrix pipe vs same quantisation")
     diep.ep_cache_init(cache_capacity=1, noskip_step=1)
@@ -286,7 +288,8 @@ def test_block_a8_one_arithmetic_behind_every_entry_point(dev):
     assert not torch.equal(y16, y)
 
 
-def test_block_a8_step_lag_and_fused_caller(dev):
+@pytest.mark.parametrize("h_blocks", [False, True])
+def test_block_a8_step_lag_and_fused_caller(dev, h_blocks):
     """The fp8 x fp8 experts behind the other two layer entry points: a
     displaced (step-lagged) call returns, bit for bit, what the synchronous
     fp8 block produced two steps earlier, and the fused-caller call equals
@@ -296,10 +299,10 @@ def test_block_a8_step_lag_and_fused_caller(dev):
     D, E, N = 1024, 8, 1024
     p = O.make_block_params(D, E, 2, 4, None, seed=21, dtype=torch.bfloat16)
     sync = block_from_params(p, D, "swiglu", torch.bfloat16, dev)
-    sync.quantize_fp8(activations=True)
+    sync.quantize_fp8(activations=True, h_blocks=h_blocks)
     pm = ParaMode(ep=True, ep_async=True, ep_async_mode="all")
     lag = block_from_params(p, D, "swiglu", torch.bfloat16, dev, para_mode=pm)
-    lag.quantize_fp8(activations=True)
+    lag.quantize_fp8(activations=True, h_blocks=h_blocks)
     g = _gen(22)
     xs = [torch.randn(1, N, D, generator=g).bfloat16().to(dev) for _ in range(4)]
     plain = [sync(x).clone() for x in xs]
@@ -328,3 +331,154 @@ def test_block_a8_step_lag_and_fused_caller(dev):
          + shift.float().unsqueeze(1)).bfloat16()
     want = xb.float() + gate.float().unsqueeze(1) * sync(h).float()
     assert rel_l2(got.float().cpu(), want.cpu()) < 5e-3          # one bf16 rounding of the sum apart
+
+
+# --------------------------------------------------------------------------- #
+# h quantised inside fc1's epilogue: one power-of-two scale per row and 32 columns
+# --------------------------------------------------------------------------- #
+def _mlp_case(variant, D, ratio, E, counts, dev, seed=8):
+    from dice_amd import ops
+    N = 1024 if counts is None else sum(counts) // 2
+    g = _gen(177 + D)
+    p = O.make_block_params(D, E, 2, ratio, n_shared=0, seed=seed, dtype=torch.bfloat16, variant=variant)
+    if variant == "gelu_tanh":
+        _bias_params(p, 9)
+    x = torch.randn(N, D, generator=g).bfloat16()
+    if counts is None:
+        idx = torch.randint(0, E, (N * 2,), generator=g)
+    else:
+        idx = torch.cat([torch.full((c,), e) for e, c in enumerate(counts)])
+        idx = idx[torch.randperm(idx.numel(), generator=g)]
+    _, offsets, perm, _ = O.dispatch_tables(idx, E)
+    w1, w2, b1, b2 = _packed(p, variant, dev)
+    q1, s1 = ops.quantize_fp8_rowwise(w1)
+    q2, s2 = ops.quantize_fp8_rowwise(w2)
+    args = (x.to(dev), perm.int().to(dev), 2, offsets.int().to(dev), idx.numel(), q1, q2, s1, s2, variant, b1, b2)
+    return p, x, perm, offsets, args
+
+
+H_BLOCK_CASES = [
+    ("swiglu", 768, 4, 8, None),
+    ("gelu_tanh", 768, 4, 8, None),
+    ("swiglu", 1024, 2, 8, [0, 1, 700, 0, 257, 3, 1086, 1]),          # empty, one-row and ragged groups
+    ("gelu_tanh", 1024, 2, 8, [0, 1, 700, 0, 257, 3, 1086, 1]),
+    ("swiglu", 2048, 4, 16, None),                                     # DiT-G width
+    # a group's last tile multiplies only its live 64-row blocks: residues around the block edges
+    ("swiglu", 768, 2, 16, [63, 64, 65, 127, 128, 129, 191, 192, 193, 255, 256, 257, 320, 0, 1, 7]),
+    ("gelu_tanh", 1024, 2, 8, [256 + 63, 256 + 64, 256 + 65, 512 + 128, 512 + 129, 256 + 191, 256 + 193, 513]),
+]
+
+
+@pytest.mark.parametrize("variant,D,ratio,E,counts", H_BLOCK_CASES)
+def test_fc1_epilogue_block_quantiser_bit_exact(dev, variant, D, ratio, E, counts):
+    """fc1 with ``h_blocks`` against the oracle's block quantiser applied to the
+    bf16 ``h`` the same kernel writes without it (same sums, same order, the
+    quantiser starts from the value rounded to bf16): bytes and exponents of
+    every row, bit for bit."""
+    from dice_amd import ops
+    p, x, perm, offsets, args = _mlp_case(variant, D, ratio, E, counts, dev)
+    rows, inter = args[4], ratio * D
+    _, h16 = ops.grouped_mlp_a8(*args, stages=1)
+    h8 = torch.zeros((rows, inter), dtype=torch.bfloat16, device=dev)
+    ops.grouped_mlp_a8(*args, stages=1, h=h8, h_blocks=True)
+    q, e = ops.split_h_blocks(h8, rows, inter)
+    want_q, want_e = O.quantize_fp8_act_blocks(h16.cpu())
+    assert torch.equal(e.cpu(), want_e)
+    assert torch.equal(q.cpu(), want_q.view(torch.uint8))
+    # the scales do their work: blocks of one row differ in exponent
+    assert (want_e.max(dim=1).values > want_e.min(dim=1).values).any()
+
+
+@pytest.mark.parametrize("variant,D,ratio,E,counts", H_BLOCK_CASES)
+def test_fc2_on_block_scaled_rows(dev, variant, D, ratio, E, counts):
+    """fc2 alone on block-scaled e4m3 rows made by the oracle - exponents spread
+    over 40 powers of two within a row, so a scale applied to the wrong block,
+    k-block or lane half shows - against the oracle's product of the dequantised
+    rows; then the whole MLP against ``Fp8ActExpert(h_blocks=True)``."""
+    from dice_amd import ops
+    p, x, perm, offsets, args = _mlp_case(variant, D, ratio, E, counts, dev)
+    rows, inter = args[4], ratio * D
+    g = _gen(5 + D)
+    h = torch.randn(rows, inter, generator=g)
+    h = h * torch.exp2(torch.randint(-20, 20, (rows, inter // 32), generator=g).float()).repeat_interleave(32, dim=1)
+    q, e = O.quantize_fp8_act_blocks(h.bfloat16())
+    hbuf = torch.zeros((rows, inter), dtype=torch.bfloat16, device=dev)
+    ops.join_h_blocks(hbuf, q.view(torch.uint8).to(dev), e.to(dev))
+    out, _ = ops.grouped_mlp_a8(*args, stages=2, h=hbuf, h_blocks=True)
+    hd = O.dequantize_fp8_act_blocks(q, e)
+    want = torch.empty(rows, D)
+    for ex in range(E):
+        lo, hi = int(offsets[ex]), int(offsets[ex + 1])
+        if hi > lo:
+            o8 = O.Fp8ActExpert(p.experts[ex])
+            w = (hd[lo:hi] @ o8.q2.float().t()) * o8.s2[None, :]
+            want[lo:hi] = (w + o8.b2 if o8.b2 is not None else w).bfloat16().float()
+    check_rows(out.cpu(), want, SAME_QUANT_TOL, "fc2 on block-scaled rows")
+    # both stages
+    out, _ = ops.grouped_mlp_a8(*args, h_blocks=True)
+    xg = x[perm // 2]
+    want = torch.empty(rows, D)
+    for ex in range(E):
+        lo, hi = int(offsets[ex]), int(offsets[ex + 1])
+        if hi > lo:
+            want[lo:hi] = O.Fp8ActExpert(p.experts[ex], h_blocks=True)(xg[lo:hi]).float()
+    check_rows(out.cpu(), want, SAME_QUANT_TOL, "expert rows, h in blocks")
+
+
+def test_block_quantiser_special_blocks(dev):
+    """All-zero blocks, a block with an infinity, amax exactly 448 x 2^n and tiny values, through fc1's
+    epilogue: arranged with GELU experts whose fc1 weights are zero, so that h = gelu(bias)."""
+    from dice_amd import ops
+    D, ratio, E = 768, 2, 8
+    p, x, perm, offsets, args = _mlp_case("gelu_tanh", D, ratio, E, None, dev)
+    args = list(args)
+    rows, inter = args[4], ratio * D
+    b1 = torch.zeros(E, inter)
+    b1[:, 32:64] = 448.0                       # gelu(448) = 448: amax / 448 a power of two
+    b1[:, 64:96] = torch.linspace(-3, 3, 32)
+    b1[:, 96:128] = 1e-3
+    b1[:, 128:160] = 56.0
+    b1[3, 160] = float("inf")
+    b1[:, 192:224] = torch.randn(E, 32, generator=_gen(1)) * 100
+    args[5] = torch.zeros_like(args[5])        # fc1 weights: e4m3 zeros
+    args[10] = b1.to(dev)
+    h16 = ops.grouped_mlp_a8(*args, stages=1)[1]
+    h8 = torch.zeros((rows, inter), dtype=torch.bfloat16, device=dev)
+    ops.grouped_mlp_a8(*args, stages=1, h=h8, h_blocks=True)
+    q, e = ops.split_h_blocks(h8, rows, inter)
+    want_q, want_e = O.quantize_fp8_act_blocks(h16.cpu())
+    assert torch.equal(e.cpu(), want_e) and torch.equal(q.cpu(), want_q.view(torch.uint8))
+    lo, hi = int(offsets[3]), int(offsets[4])
+    assert hi > lo and (q.cpu()[lo:hi, 160:192] == 0x7F).all() and (e.cpu()[lo:hi, 5] == 127).all()
+    assert (e.cpu()[:, 0] == 0).all() and (q.cpu()[:, :32] == 0).all()
+    assert (e.cpu()[:, 1] == 127).all() or (e.cpu()[:, 1] == 128).all()
+
+
+@pytest.mark.parametrize("variant,n_shared", [("swiglu", 2), ("gelu_tanh", 8)])
+def test_block_c5_h_blocks_full_size(dev, variant, n_shared):
+    """The DiT-G/2-like block with ``quantize_fp8(activations=True, h_blocks=True)``: every token against the
+    bf16 masters (5e-2), against the oracle with the same quantisation, and no further from the masters than
+    the per-row form."""
+    D, E = 2048, 16
+    p = O.make_block_params(D, E, 2, 4, n_shared, seed=3, dtype=torch.bfloat16, variant=variant)
+    if variant == "gelu_tanh":
+        _bias_params(p, 4)
+    x = torch.randn(32, 256, D, generator=_gen(5)).bfloat16()
+    blk = block_from_params(p, D, variant, torch.bfloat16, dev)
+    blk.quantize_fp8(activations=True, h_blocks=True)
+    y = blk(x.to(dev)).cpu()
+    want, _, _, logits = O.sparse_moe_block_forward(p, x)
+    ok = ~O.gate_tie_rows(logits, 2).view(-1)
+    err = check_rows(y.view(-1, D)[ok], want.view(-1, D)[ok], FP8_TOL, "C5, h in blocks, vs bf16 masters")
+    p8 = copy.copy(p)
+    p8.experts = [O.Fp8ActExpert(e, h_blocks=True) for e in p.experts]
+    same, _, _, _ = O.sparse_moe_block_forward(p8, x)
+    check_rows(y.view(-1, D)[ok], same.view(-1, D)[ok], SAME_QUANT_TOL, "C5, h in blocks, vs same quantisation")
+    blk.quantize_fp8(activations=True)
+    y_rows = blk(x.to(dev)).cpu()
+    err_rows = rel_l2(y_rows.view(-1, D)[ok], want.view(-1, D)[ok])
+    assert not torch.equal(y_rows, y) and err < 1.05 * err_rows
+    # the routed-experts entry of the module computes what the layer call does
+    blk.quantize_fp8(activations=True, h_blocks=True)
+    idx, wt, _ = blk.gate(x.to(dev))
+    assert blk._desc is None or blk._desc.act_quant == 2

@@ -297,6 +297,82 @@ def test_fp8_act_quantiser_properties():
     assert ((deq - x.float()).abs() <= x.float().abs().amax(1, keepdim=True) * 2 ** -4).all()
 
 
+def test_fp8_block_quantiser_against_bruteforce():
+    """``quantize_fp8_act_blocks`` against its definition worked out another way: per block the
+    exponent is the smallest e with amax * fp32(1/448) <= 2^(e-127) (found by a search over all 255
+    exponents in float64, which holds every float32 and every power of two exactly), the bytes are the
+    nearest e4m3 codes of block * 2^(127-e) (search over all codes, ties to even)."""
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(19, 256, generator=g) * torch.exp2(torch.randint(-30, 30, (19, 8), generator=g).float()
+                                                       ).repeat_interleave(32, dim=1)
+    x = x.bfloat16()
+    x[2, 32:64] = 0
+    x[5, 0:32] = 448.0 * 2.0 ** -7                    # amax / 448 a power of two: that very power
+    x[6, 0:32] = 450.0 * 2.0 ** -7                    # just above it: the next power
+    q, e = O.quantize_fp8_act_blocks(x)
+    assert q.dtype == torch.float8_e4m3fn and e.dtype == torch.uint8 and e.shape == (19, 8)
+    xn = x.float().numpy().reshape(19, 8, 32)
+    amax = np.abs(xn).max(-1)
+    t = (amax * np.float32(1.0 / 448.0)).astype(np.float32).astype(np.float64)
+    pw = np.ldexp(1.0, np.arange(255) - 127)          # 2^(e-127), e = 0 .. 254
+    want_e = (t[..., None] <= pw).argmax(-1)
+    assert np.array_equal(e.numpy(), want_e)
+    scaled = xn.astype(np.float64) * np.ldexp(1.0, 127 - want_e)[..., None]
+    want_q = _nearest_e4m3(np.clip(scaled, -448, 448)).reshape(19, 256)
+    got = q.view(torch.uint8).numpy()
+    zero = scaled.reshape(19, 256) == 0
+    assert np.array_equal(got[~zero], want_q[~zero]) and not (got[zero] & 0x7f).any()
+    assert e[2, 1] == 0 and e[5, 0] == 127 - 7 and e[6, 0] == 127 - 6
+
+
+def test_fp8_block_quantiser_properties():
+    g = torch.Generator().manual_seed(23)
+    x = torch.randn(33, 128, generator=g).bfloat16()
+    q, e = O.quantize_fp8_act_blocks(x)
+    deq = O.dequantize_fp8_act_blocks(q, e)
+    blk_amax = x.float().view(33, 4, 32).abs().amax(-1)
+    # the scaled block maximum lies in (224, 448] (the smallest power of two that keeps it representable),
+    # so its code is one of 224 .. 448
+    top = q.float().view(33, 4, 32).abs().amax(-1)
+    assert (top >= 224).all() and (top <= 448).all()
+    scaled = blk_amax * torch.exp2(127 - e.float())
+    assert (scaled > 224).all() and (scaled <= 448).all()
+    assert ((deq - x.float()).view(33, 4, 32).abs() <= blk_amax[..., None] * 2 ** -4).all()
+    # a power-of-two factor per block moves the exponent by that power and changes no byte
+    f = torch.tensor([3, -2, 0, 5]).repeat(33, 1)
+    x2 = (x.float().view(33, 4, 32) * torch.exp2(f.float())[..., None]).reshape(33, 128).bfloat16()
+    q2, e2 = O.quantize_fp8_act_blocks(x2)
+    assert torch.equal(q2.view(torch.uint8), q.view(torch.uint8)) and torch.equal(e2.int(), e.int() + f)
+    # idempotence of the values: what it returns re-quantises to the same numbers (a block whose maximum was
+    # rounded down to the code 224 comes back with the next smaller exponent and doubled codes)
+    q3, e3 = O.quantize_fp8_act_blocks(deq.bfloat16())       # e4m3 values times powers of two are exact in bf16
+    assert torch.equal(O.dequantize_fp8_act_blocks(q3, e3), deq)
+    assert ((e3 == e) | ((e3.int() == e.int() - 1) & (top == 224))).all()
+    # blocks are independent; a block with an infinity or a NaN becomes NaN bytes with a unit scale
+    y = x.clone()
+    y[7, 40] = float("inf")
+    y[8, 100] = float("nan")
+    q4, e4 = O.quantize_fp8_act_blocks(y)
+    same = torch.ones(33, 4, dtype=torch.bool)
+    same[7, 1] = same[8, 3] = False
+    assert torch.equal(q4.view(torch.uint8).view(33, 4, 32)[same], q.view(torch.uint8).view(33, 4, 32)[same])
+    assert torch.equal(e4[same], e[same]) and e4[7, 1] == 127 and e4[8, 3] == 127
+    assert (q4.view(torch.uint8).view(33, 4, 32)[~same] & 0x7f == 0x7f).all()
+    assert torch.isnan(O.dequantize_fp8_act_blocks(q4, e4)[7, 32:64]).all()
+
+
+def test_fp8_act_expert_with_h_blocks_is_the_product_of_dequantised_operands():
+    p = O.make_block_params(256, 2, 1, 2, None, seed=5, dtype=torch.bfloat16)
+    ex = O.Fp8ActExpert(p.experts[0], h_blocks=True)
+    x = torch.randn(9, 256, generator=torch.Generator().manual_seed(6)).bfloat16()
+    h = ex.hidden_act(x)
+    assert torch.equal(h, O.Fp8ActExpert(p.experts[0]).hidden_act(x))      # fc1 is the same either way
+    q, e = O.quantize_fp8_act_blocks(h)
+    want = (O.dequantize_fp8_act_blocks(q, e).double() @ ex.q2.double().t()) * ex.s2.double()[None, :]
+    got = ex(x).double()
+    assert float((got - want).norm() / want.norm()) < 1e-2 and not torch.equal(ex(x), O.Fp8ActExpert(p.experts[0])(x))
+
+
 @pytest.mark.parametrize("variant", ["swiglu", "gelu_tanh"])
 def test_fp8_act_expert_is_the_product_of_dequantised_operands(variant):
     """``Fp8ActExpert`` against float64 numpy on the dequantised operands: the
