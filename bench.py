@@ -915,11 +915,13 @@ def main():
         legs = {}
         short = max(10, args.steps // 2)
         for name, var, act in (("c1", args.variant, "bf16"), ("c3", args.variant, "bf16"),
-                               ("c5", args.variant, "fp8"), ("c5", args.variant, "bf16"),
+                               ("c5", args.variant, "fp8"), ("c5", args.variant, "fp8_blocks"),
+                               ("c5", args.variant, "bf16"),
                                ("c2", "gelu_tanh" if args.variant == "swiglu" else "swiglu", "bf16"),
                                ("c5", "gelu_tanh" if args.variant == "swiglu" else "swiglu", "fp8")):
             c, b, xx, r = measure(name, var, act, dev, short, 5, stages=not args.no_stages)
-            key = name + ("_" + var if var != args.variant else "") + ("_w8a16" if c.get("fp8") and act == "bf16" else "")
+            key = (name + ("_" + var if var != args.variant else "") + ("_w8a16" if c.get("fp8") and act == "bf16" else "")
+                   + ("_h_blocks" if act == "fp8_blocks" else ""))
             keep = {q: r[q] for q in ("tokens_per_s", "ms_per_step", "layer_tflops", "workload", "roofline",
                                       "fp8_launch_frac_of_fp8_peak", "quantiser_gbs", "hbm_stage_frac_of_peak") if q in r}
             if "stage_ms" in r:
