@@ -896,7 +896,11 @@ __device__ __forceinline__ void tile_epilogue_blockq(const Tile &cp, unsigned ch
       constexpr int j = decltype(j_c)::value;
       f32x16_t blk = fixed_acc_block<i * TN + j>(), up;
       if constexpr (SWIGLU) up = fixed_acc_block<i * TN + j + OUT_BLOCKS>();
-      uint32_t amax_bits = 0;
+      // (maxima of the magnitudes as packed 16-bit integers: non-negative values of the 16-bit type order like
+      // their bits, NaN above all)
+      typedef h16_t h16pair_t __attribute__((ext_vector_type(2)));
+      typedef unsigned short u16pair_t __attribute__((ext_vector_type(2)));
+      u16pair_t amax2 = {0, 0};
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const float *sp = scale_lds + wave_col0 + j * 32 + frag_half * 4 + q * 8;
@@ -904,6 +908,7 @@ __device__ __forceinline__ void tile_epilogue_blockq(const Tile &cp, unsigned ch
         sg *= row_scale;
         if (SWIGLU) su = *reinterpret_cast<const f32x4_t *>(sp + 128) * row_scale;
         if (BIAS_LDS) sb = *reinterpret_cast<const f32x4_t *>(bias_lds + wave_col0 + j * 32 + frag_half * 4 + q * 8);
+        float vv[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           float v = blk[q * 4 + r] * sg[r];
@@ -913,12 +918,19 @@ __device__ __forceinline__ void tile_epilogue_blockq(const Tile &cp, unsigned ch
             if (BIAS_LDS) v += sb[r];
             if (MODE == kFc1Gelu) v = gelu_tanh_fast(v);
           }
-          v = (float)(h16_t)v;
-          blk[q * 4 + r] = v;
-          const uint32_t mag = __float_as_uint(v) & 0x7fffffffu;
-          amax_bits = mag > amax_bits ? mag : amax_bits;   // (non-negative floats order like their bits; NaN above all)
+          vv[r] = v;
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r += 2) {
+          static_assert(MODE < 0 || !DICE_PERSIST_F16, "bf16 rows (the fp8 kernels take no other)");
+          const h16pair_t hp = {(h16_t)vv[r], (h16_t)vv[r + 1]};
+          const uint32_t pr = __builtin_bit_cast(uint32_t, hp);
+          blk[q * 4 + r] = __uint_as_float(pr << 16);             // (bf16: the value is its bits, 16 up)
+          blk[q * 4 + r + 1] = __uint_as_float(pr & 0xffff0000u);
+          amax2 = __builtin_elementwise_max(amax2, __builtin_bit_cast(u16pair_t, pr & 0x7fff7fffu));
         }
       }
+      uint32_t amax_bits = (uint32_t)(amax2[0] > amax2[1] ? amax2[0] : amax2[1]) << 16;
       // (the row's other 16 columns sit in the lane 32 on: one swap of the lane halves of two copies, then
       // every lane holds both maxima)
       {
@@ -934,7 +946,8 @@ __device__ __forceinline__ void tile_epilogue_blockq(const Tile &cp, unsigned ch
       for (int q = 0; q < 4; ++q) {
         float f[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) f[r] = __builtin_amdgcn_fmed3f(blk[q * 4 + r] * inv, -448.f, 448.f);
+        // (no clamp: the scale is at least amax / 448 for a 16-bit amax, so the products stay within +-448)
+        for (int r = 0; r < 4; ++r) f[r] = blk[q * 4 + r] * inv;
         int w = 0;
         w = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], w, false);
         w = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], w, true);
