@@ -192,6 +192,7 @@ struct PersistBatch {
 constexpr int kPersistSplitSlots = 320;  // partial-tile slots: one per workgroup of a launch (one per compute unit)
 size_t persist_split_ws_bytes();         // kPersistSplitSlots tiles of 256 x 256 16-bit values
 bool persist_supported(const PersistBatch &b, int mode);
+bool persist_fits_table(const PersistBatch &b, int mode);  // at most kTableTurns tiles per workgroup: no kernel has to rebuild its tile table
 int persist_cu_count();  // compute units of the current device
 int persist_band_tiles(int mode);  // tuning hook state: band height of the tile order for this stage (0 = default rule)
 int persist_slim_choice(int mode);  // tuning hook state: 128-row weight tiles for launches of this stage that can take them: 1 = always, -1 = never, 0 = by the model

@@ -1143,7 +1143,7 @@ bool persist64_fits_table(const PersistBatch &b, int mode) {
 bool persist64_ok(const PersistBatch &b, int mode) {
   for (int i = 0; i < b.n_problems; ++i) {
     const PersistProblem &p = b.prob[i];
-    if (p.a_scale) return false;  // fp8 activations: the kernel of the fp8 compilation unit
+    if (p.a_scale || p.a_block_scale || p.c_block_scale) return false;  // fp8 activations: the kernel of the fp8 compilation unit
     if (p.k < kQBK * kQMinSteps) return false;
     if (p.w_scale && b.n_problems != 1) return false;  // fp8 weights: single-problem launches
     if (p.a_rows) {  // gathered activation rows: the fc1 kernels with the generated k-loop (SwiGLU, and GELU on
@@ -1173,7 +1173,8 @@ int persist_variant(const PersistBatch &b, int mode) {
   if (!persist_common_ok(b, mode)) return 0;
   if (g_persist_waves == 4 && persist64_ok(b, mode)) return 4;
   for (int i = 0; i < b.n_problems; ++i)
-    if (b.prob[i].a_rows || b.prob[i].w_scale || b.prob[i].a_scale) return 0;  // the 32-k kernel wants contiguous rows and bf16 operands
+    if (b.prob[i].a_rows || b.prob[i].w_scale || b.prob[i].a_scale || b.prob[i].a_block_scale || b.prob[i].c_block_scale)
+      return 0;  // the 32-k kernel wants contiguous rows and bf16 operands
   return 8;
 }
 

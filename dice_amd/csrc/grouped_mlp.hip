@@ -457,6 +457,19 @@ int forward_impl(const char *who, const dice_moe_layer_t *L, const dice_moe_laye
     DICE_REQUIRE(act_quant_widths_ok(L->hidden, L->inter), DICE_ERR_UNSUPPORTED,
                  "%s: act_quant needs hidden %d and inter %d to be multiples of 256 between 768 and 8192", who,
                  L->hidden, L->inter);
+    if (L->act_quant == 2) {
+      // (fc2 on block-scaled rows has no variant that rebuilds its tile table: refused here, before the
+      // router is launched, and not by the fc2 launch)
+      PersistBatch probe{};
+      probe.n_problems = 1;
+      probe.prob[0].n_experts = L->n_experts;
+      probe.prob[0].n = L->hidden;
+      probe.prob[0].k = L->inter;
+      probe.prob[0].max_rows = (int)(n_tokens * L->top_k);
+      DICE_REQUIRE(persist_fits_table(probe, kFc2), DICE_ERR_UNSUPPORTED,
+                   "%s: act_quant 2 takes at most 64 fc2 tiles of 256 x 256 per compute unit (%lld tokens make more); "
+                   "use act_quant 1 or split the batch", who, (long long)n_tokens);
+    }
   }
   if (combine_mode == 1)
     DICE_REQUIRE(skip_mask && cache_out, DICE_ERR_BAD_ARG, "%s: a put step needs skip_mask and cache_out", who);

@@ -482,3 +482,18 @@ def test_block_c5_h_blocks_full_size(dev, variant, n_shared):
     blk.quantize_fp8(activations=True, h_blocks=True)
     idx, wt, _ = blk.gate(x.to(dev))
     assert blk._desc is None or blk._desc.act_quant == 2
+
+
+def test_h_blocks_refuses_a_call_with_more_tiles_than_its_table_holds(dev):
+    """fc2 on block-scaled rows has no variant that rebuilds its tile table (64 tiles per workgroup):
+    a call that would need it is refused before anything is launched, and the per-row form takes it."""
+    from dice_amd.lib import DiceError
+    D, E, N = 768, 8, 736 * 1024            # (2 N / 256 + 8) x 3 tiles over 256 workgroups: 67 each
+    p = O.make_block_params(D, E, 2, 1, None, seed=2, dtype=torch.bfloat16)
+    blk = block_from_params(p, D, "swiglu", torch.bfloat16, dev)
+    blk.quantize_fp8(activations=True, h_blocks=True)
+    x = torch.zeros(1, N, D, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(DiceError, match="act_quant 2"):
+        blk(x)
+    y = blk(x[:, :4096])
+    assert y.shape == (1, 4096, D) and torch.isfinite(y).all()
