@@ -83,21 +83,23 @@ def test_16bit_block_cut_last_turn(dev, variant, D, ratio, E, n_shared, N, dtype
 
 
 @pytest.mark.parametrize("variant", ["swiglu", "gelu_tanh"])
-@pytest.mark.parametrize("activations", [False, True])
+@pytest.mark.parametrize("activations", [False, True, "h_blocks"])
 def test_fp8_block_cut_last_turn(dev, variant, activations):
     """fp8 weights (bf16 matrix pipe) and fp8 weights x fp8 activations (fp8
-    matrix pipe), shared expert in launches of its own (which cut theirs too)."""
+    matrix pipe; also with h quantised in blocks by fc1's epilogue: a piece of a
+    cut tile then starts part-way into a row of block scales), shared expert in
+    launches of its own (which cut theirs too)."""
     D, E, N = 1024, 8, 1280
     p = O.make_block_params(D, E, 2, 3, 2, seed=31, dtype=torch.bfloat16, variant=variant)
     if variant == "gelu_tanh":
         _bias_params(p, 32)
     x = torch.randn(1, N, D, generator=_gen(33)).bfloat16()
     blk = block_from_params(p, D, variant, torch.bfloat16, dev)
-    blk.quantize_fp8(activations=activations)
+    blk.quantize_fp8(activations=bool(activations), h_blocks=activations == "h_blocks")
     whole, cut = _whole_and_cut(blk, x.to(dev))
     if activations:   # against the oracle with the same quantisation
         ref = copy.copy(p)
-        ref.experts = [O.Fp8ActExpert(e) for e in p.experts]
+        ref.experts = [O.Fp8ActExpert(e, h_blocks=activations == "h_blocks") for e in p.experts]
         tol = SAME_QUANT_TOL
     else:             # against the bf16 master weights
         ref, tol = p, FP8_TOL
