@@ -720,6 +720,9 @@ def test_block_xl_width_large_batch_matches_chunks(dev):
     ("swiglu", torch.float16, True, 172032, 384, 4),        # fp8 weights: so are the scale buffers
     ("swiglu", torch.bfloat16, "act", 180224, 768, 2),      # fp8 activations too: the fp8 kernel's scales and row scales
     ("gelu_tanh", torch.bfloat16, "act", 180224, 768, 2),   # ... and its bias
+    # ... with fc1's epilogue quantising h in blocks (fc1 rewrites its table, fc2 - a quarter of the tiles - does not)
+    ("swiglu", torch.bfloat16, "act_blocks", 180224, 768, 2),
+    ("gelu_tanh", torch.bfloat16, "act_blocks", 180224, 768, 2),
 ])
 def test_rewritten_tile_table_other_kernels(dev, variant, dtype, fp8, N, D, ratio):
     """The other instantiations that rewrite their tile table (more than 64 tiles
@@ -733,7 +736,7 @@ def test_rewritten_tile_table_other_kernels(dev, variant, dtype, fp8, N, D, rati
             e.fc2_b = (torch.randn(e.fc2_b.shape, generator=g) * 0.1).to(dtype)
     blk = block_from_params(p, D, variant, dtype, dev)
     if fp8:
-        blk.quantize_fp8(activations=fp8 == "act")
+        blk.quantize_fp8(activations=fp8 in ("act", "act_blocks"), h_blocks=fp8 == "act_blocks")
     x = torch.randn(1, N, D, generator=torch.Generator(device=dev).manual_seed(14), device=dev).to(dtype)
     with whole_fc2_tiles():
         y = blk(x)
