@@ -61,6 +61,14 @@ Pinning status (what independently fixes each function's result):
                           amax -> +-448, zero rows, power-of-two scale
                           invariance and idempotence; the expert by the float64
                           product of the dequantised operands.
+* ``quantize_fp8_act_blocks`` - build-defined likewise: exponents against a
+                          search over all 255 powers of two in float64 for the
+                          smallest one that covers amax * fp32(1/448), bytes
+                          against the nearest-code search above; scaled block
+                          maxima in (224, 448], per-block power-of-two
+                          invariance, idempotence of the values, blocks
+                          independent of each other, NaN bytes for a block
+                          that holds a NaN or an infinity.
 """
 from __future__ import annotations
 
